@@ -1,0 +1,177 @@
+/*
+ * smr.h - C ABI of libsmr_gfx950.so: the symmetric-memory hot path
+ * (one-shot all-reduce, blockwise barrier / signal-pad flags, all-gather matmul,
+ * split-K GEMV + reduce) as hand-written HIP kernels for MI355X (gfx950).
+ *
+ * Conventions for every entry point
+ *   - returns int: 0 on success, otherwise a hipError_t value or a negative
+ *     SMR_E_* code; smr_last_error_string() describes the last failure of the
+ *     calling thread.  Nothing throws.
+ *   - all pointers are borrowed; "dev" pointers are device addresses.
+ *   - `stream` is a hipStream_t passed as void* (NULL = the null stream); the
+ *     work is enqueued asynchronously on it.
+ *   - `status` (nullable) is a device array of SMR_STATUS_WORDS uint32.  Every
+ *     in-kernel spin is bounded by the spin timeout; a spin that expires writes
+ *     a SMR_ST_* code into status[0] (first error wins), the identity of the
+ *     waiter into status[1..3], and the kernel carries on to its end so that the
+ *     grid always drains.  status[0] == 0 after a synchronize means the result
+ *     is valid.
+ *   - "emulated ranks": the multi-GPU symmetric-memory layout is emulated on one
+ *     GPU.  `buffer_ptrs_dev` / `signal_pad_ptrs_dev` are device arrays of
+ *     world_size uint64 addresses (one buffer / one zero-initialised uint32 pad
+ *     per rank), exactly what the reference hands to its kernels
+ *     (symm_mem_recipes/triton_one_shot_all_reduce.py:115-116,
+ *     symm_mem_recipes/triton_barrier.py:167).
+ */
+#ifndef SMR_H_
+#define SMR_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define SMR_VERSION 100
+
+#define SMR_DTYPE_BF16 0
+#define SMR_DTYPE_FP32 1
+
+#define SMR_MAX_WORLD_SIZE 8
+#define SMR_STATUS_WORDS 4
+
+/* negative return codes (argument validation on the host) */
+#define SMR_E_INVALID   (-1)  /* bad argument (null pointer, size, alignment, dtype) */
+#define SMR_E_UNSUPPORTED (-2) /* shape the kernels do not cover */
+
+/* status[0] codes written by kernels */
+#define SMR_ST_OK            0u
+#define SMR_ST_SEND_TIMEOUT  1u  /* CAS 0->1 on a peer's slot never succeeded (stale non-zero pad) */
+#define SMR_ST_WAIT_TIMEOUT  2u  /* a flag that was waited on never arrived */
+#define SMR_ST_MISMATCH      3u  /* signal-round checksum differed from the expected value */
+
+/* barrier_mode of smr_one_shot_all_reduce */
+#define SMR_BARRIER_NONE   0  /* no handshake: peers' data are already stream-ordered */
+#define SMR_BARRIER_PROXY  1  /* the rank's blocks run the real handshake; one proxy
+                                 workgroup per block plays the other ranks' halves */
+
+int smr_version(void);
+const char* smr_last_error_string(void);
+
+/* Bound for every in-kernel spin, in microseconds of the GPU's constant-rate
+ * clock.  0 = unbounded, which is what the reference does
+ * (triton_barrier.py:119-129, triton_all_gather_matmul.py:80-83).  Default 2 s. */
+int smr_set_spin_timeout_us(int64_t us);
+int64_t smr_get_spin_timeout_us(void);
+
+/* One-shot all-reduce.  Replaces one_shot_all_reduce_kernel + its launch
+ * (symm_mem_recipes/triton_one_shot_all_reduce.py:59-93, :114-124).
+ *   out[j] = cast(((0 + buf_0[j]) + buf_1[j]) + ... + buf_{ws-1}[j]), fp32 accumulator.
+ *   numel      elements per buffer; 16-byte multiple (bf16: %8, fp32: %4), as :103-105
+ *   rank       0..ws-1: that rank's share.  -1: all emulated ranks in one launch
+ *              (out is then [ws, numel], and the ranks run the real barrier
+ *              against each other when barrier_mode != NONE)
+ *   write_all  0: result goes to `out`.  1: result is written back into all ws
+ *              peer buffers in place (`out` may be NULL); rank must be >= 0
+ *   signal_pad_ptrs_dev may be NULL when barrier_mode == SMR_BARRIER_NONE;
+ *              each pad must hold smr_reduce_num_blocks(...) * ws uint32 slots. */
+int smr_one_shot_all_reduce(const uint64_t* buffer_ptrs_dev, const uint64_t* signal_pad_ptrs_dev,
+                            void* out, int64_t numel, int dtype, int rank, int world_size,
+                            int write_all, int barrier_mode, uint32_t* status, void* stream);
+
+/* Number of workgroups (= barrier blocks per rank) the reduce launches for a
+ * message; host-only.  Counterpart of the grid formula at
+ * triton_one_shot_all_reduce.py:97-109, resized for 256 CUs. */
+int smr_reduce_num_blocks(int64_t numel, int dtype);
+
+/* Blockwise barrier, `rounds` back-to-back rounds on `num_blocks` blocks.
+ * Replaces barrier_test_kernel / barrier_test (symm_mem_recipes/triton_barrier.py:156-170)
+ * around the device function blockwise_barrier (:50-153).
+ *   rank -1: all ws emulated ranks in one launch (ws*num_blocks workgroups)
+ *   rank >= 0: only that rank's num_blocks workgroups; its peers must be running
+ *              concurrently on other streams or the spins time out. */
+int smr_barrier(const uint64_t* signal_pad_ptrs_dev, int rank, int world_size, int num_blocks,
+                int rounds, uint32_t* status, void* stream);
+
+/* Host-callable halves of the flag protocol, one workgroup each.
+ * smr_send_signal: release-CAS 0->1 (triton_barrier.py:119-122).
+ * smr_wait_signal: spin until *addr == 1, acquire; never resets the flag
+ *                  (symm_mem_recipes/triton_all_gather_matmul.py:72-95).
+ * smr_wait_signal_reset: CAS 1->0 (triton_barrier.py:124-129).
+ * smr_stream_write_value32: stream-ordered release store of `value`, the
+ *                  stand-in for symm_mem.stream_write_value32
+ *                  (triton_all_gather_matmul.py:50-55). */
+int smr_send_signal(uint32_t* addr_dev, uint32_t* status, void* stream);
+int smr_wait_signal(const uint32_t* addr_dev, uint32_t* status, void* stream);
+int smr_wait_signal_reset(uint32_t* addr_dev, uint32_t* status, void* stream);
+int smr_stream_write_value32(uint32_t* addr_dev, uint32_t value, void* stream);
+
+/* Producer/consumer signal-pad round benchmark: ws*num_blocks workgroups; in each
+ * round workgroup (rank r, block b) publishes its chunk (src words + round) into
+ * rank r's symmetric buffer, runs the blockwise handshake for block b, then sums
+ * the ws chunks of block b and compares with expected_base[b] + ws*words*round.
+ * No counterpart kernel in the reference; it drives blockwise_barrier
+ * (triton_barrier.py:50-153) with a payload.
+ *   src_dev          uint32 [ws, num_blocks, chunk_bytes/4] payload source
+ *   buffer_ptrs_dev  ws symmetric buffers, each >= 2*num_blocks*chunk_bytes
+ *                    (two halves alternate by round parity)
+ *   expected_base_dev uint32 [num_blocks]: wrapping sum of the ws source chunks of a block
+ *   checksums_dev    uint32 [ws, num_blocks]: the last round's sums
+ *   mismatches_dev   uint32 [1]: number of (rank, block, round) sums that differed
+ *   chunk_bytes      0 = flags only (no payload), else a multiple of 16 */
+int smr_signal_round(const uint32_t* src_dev, const uint64_t* buffer_ptrs_dev,
+                     const uint64_t* signal_pad_ptrs_dev, const uint32_t* expected_base_dev,
+                     uint32_t* checksums_dev, uint32_t* mismatches_dev, int world_size,
+                     int num_blocks, int64_t chunk_bytes, int rounds, uint32_t* status,
+                     void* stream);
+
+/* All-gather producer.  Replaces all_gather_with_progress
+ * (symm_mem_recipes/triton_all_gather_matmul.py:20-56): copies every peer's
+ * shard into a_out in the order rank+1, ..., rank+ws-1, rank and, after each
+ * chunk, release-stores 1 into progress[src*splits_per_rank + split].
+ *   buffer_ptrs_dev  ws shard addresses (each shard_bytes long)
+ *   counters_dev     uint32 [ws*splits_per_rank] scratch, zero on entry
+ *   num_workgroups   copy workgroups (0 = default); kept small on purpose so the
+ *                    producer shares the GPU with the consumer GEMM */
+int smr_all_gather_with_progress(const uint64_t* buffer_ptrs_dev, void* a_out_dev,
+                                 uint32_t* progress_dev, uint32_t* counters_dev, int rank,
+                                 int world_size, int64_t shard_bytes, int splits_per_rank,
+                                 int num_workgroups, void* stream);
+
+/* Flag-gated bf16 GEMM.  Replaces matmul_kernel_tma_persistent and its launch
+ * (symm_mem_recipes/triton_all_gather_matmul.py:98-193, :287-315).
+ *   C[M,N] = A[M,K] * B[N,K]^T, fp32 accumulate, bf16 output, all row-major.
+ *   Rows of the local comm blocks (those owned by `rank`) are read from a_shard,
+ *   all others from a_out after waiting for progress[comm_block] == 1; tiles are
+ *   visited starting at the local shard and proceeding in ring order.
+ *   progress_dev NULL = ungated (the reference's mm_only comparator, :246-247).
+ *   comm_block_m  rows per progress flag = M / ws / splits_per_rank. */
+int smr_ag_matmul(const void* a_shard_dev, const void* a_out_dev, const void* b_nk_dev,
+                  void* c_dev, const uint32_t* progress_dev, int M, int N, int K, int rank,
+                  int world_size, int comm_block_m, uint32_t* status, void* stream);
+
+/* Host-only: the tile order smr_ag_matmul uses on a 256-CU part.  Writes up to
+ * max_tiles records of 8 int32 (workgroup, step, row0, col0, tile rows, tile
+ * columns, comm_block, local; grouped by workgroup, in visiting order) and
+ * returns the number of tiles, or a negative SMR_E_* code.
+ * Counterpart of the index arithmetic at triton_all_gather_matmul.py:125-174. */
+int smr_ag_matmul_schedule(int M, int N, int K, int rank, int world_size, int comm_block_m,
+                           int32_t* out_records, int max_tiles);
+
+/* Split-K GEMV + rank-ordered combine through signal-pad flags.  No reference
+ * code exists for it in symm_mem_recipes; it reuses the send/wait protocol of
+ * triton_barrier.py:119-129 and triton_all_gather_matmul.py:72-95.
+ *   x [batch,K] bf16, w [K,N] bf16 row-major, K split into ws shards;
+ *   partials fp32 [ws, batch, N] scratch; flags uint32 [ws * flag_blocks] zero on
+ *   entry and zero again on exit; out [batch,N] bf16 =
+ *   bf16(((0 + p_0) + p_1) + ... + p_{ws-1}).  batch <= 8.
+ *   smr_gemv_flag_blocks(N) gives flag_blocks. */
+int smr_gemv_allreduce(const void* x_dev, const void* w_dev, float* partials_dev,
+                       uint32_t* flags_dev, void* out_dev, int batch, int K, int N,
+                       int world_size, uint32_t* status, void* stream);
+int smr_gemv_flag_blocks(int N);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SMR_H_ */

@@ -1,0 +1,327 @@
+// Flag-gated bf16 GEMM for the all-gather matmul:  C[M,N] = A[M,K] * B[N,K]^T.
+//
+// Shape of the kernel (MI355X / gfx950, 256 CUs in 8 XCDs, 160 KiB LDS per CU):
+//   * persistent grid, one 256-thread workgroup per CU; a workgroup computes
+//     BM x BN output tiles (256x256 by default), 4 waves in a 2x2 arrangement, so
+//     a wave owns a (BM/2)x(BN/2) block held in fp32 accumulators and built from
+//     v_mfma_f32_32x32x16_bf16;
+//   * both operands are K-contiguous, so a tile's K-slab (rows x 64 bf16 = 128 B
+//     per row) is brought straight from global memory into LDS with 128-bit
+//     direct-to-LDS loads (no staging registers), two stages deep: the loads of
+//     slab k+1 are in flight while slab k is multiplied;
+//   * an LDS row is 8 chunks of 16 B; chunk c of row r is stored at position
+//     c ^ s(r), s(r) = (r ^ (r >> 3)) & 7, which makes the 128-bit fragment reads
+//     of 32 consecutive rows hit distinct banks;
+//   * the MFMA is issued with the B fragment as its first operand, so a lane
+//     ends up with 4 consecutive output columns of one row and stores 8 bytes
+//     at a time;
+//   * tiles are walked in the ready order of the all-gather: all tiles of the
+//     local comm block first, then the comm blocks in ring order; a tile of a
+//     non-local comm block first waits for that block's progress flag.  Within
+//     one pass over the grid, XCD x (workgroups with id % 8 == x) takes a
+//     contiguous run of the tile order - 8 row tiles x 4 column tiles when the
+//     pass is full - so the workgroups that share an L2 also share A rows and
+//     B columns.
+#include "smr_device.hpp"
+
+namespace smr {
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef __attribute__((address_space(3))) void LdsVoid;
+typedef __attribute__((address_space(1))) void GlobalVoid;
+
+constexpr int kGemmThreads = 256;
+constexpr int kBK = 64;          // K extent of one LDS stage (128 bytes per row)
+constexpr int kRowBytes = kBK * 2;
+
+struct GemmSchedule {
+  int M, N, K;
+  int rank, world_size, comm_block_m;
+  int BM, BN;
+  int grid;                      // persistent workgroups, a multiple of 8
+};
+
+struct TileRef {
+  int row0, col0;                // output tile origin
+  int comm_block;                // progress flag index
+  int local;                     // rows come from the local shard, no wait
+  int a_row;                     // first row inside the source (shard-relative when local)
+};
+
+// Tile visited by workgroup `wg` in its `step`-th trip; false when it has no more work.
+__host__ __device__ inline bool tile_for(const GemmSchedule& s, int wg, int step, TileRef& t) {
+  const int tn = (s.N + s.BN - 1) / s.BN;
+  const int cb_tiles_m = s.comm_block_m / s.BM;
+  const int n_comm = s.M / s.comm_block_m;
+  const int per_rank = n_comm / s.world_size;
+  const int tiles_per_cb = cb_tiles_m * tn;
+  const int total = n_comm * tiles_per_cb;
+  const int start = step * s.grid;
+  if (start >= total) return false;
+  const int cnt = (total - start) < s.grid ? (total - start) : s.grid;
+  const int per_xcd = (cnt + 7) >> 3;
+  const int slot = wg >> 3;
+  if (slot >= per_xcd) return false;
+  const int in_pass = (wg & 7) * per_xcd + slot;
+  if (in_pass >= cnt) return false;
+  const int lin = start + in_pass;
+  const int ring_pos = lin / tiles_per_cb;
+  const int rem = lin - ring_pos * tiles_per_cb;
+  const int tile_n = rem / cb_tiles_m;
+  const int tile_m = rem - tile_n * cb_tiles_m;
+  const int first_local = s.rank * per_rank;
+  const int cb = (first_local + ring_pos) % n_comm;
+  t.comm_block = cb;
+  t.row0 = cb * s.comm_block_m + tile_m * s.BM;
+  t.col0 = tile_n * s.BN;
+  t.local = (cb / per_rank) == s.rank;
+  t.a_row = t.local ? t.row0 - first_local * s.comm_block_m : t.row0;
+  return true;
+}
+
+// Position swizzle of an LDS row.
+__device__ __forceinline__ int row_swizzle(int r) { return (r ^ (r >> 3)) & 7; }
+
+// Bring ROWS x 64 bf16 (rows `stride_bytes` apart, clamped to `last_row`) into
+// a swizzled LDS tile.  One wave instruction fills 8 rows = 1 KiB of LDS in lane
+// order, so lane l carries row (l >> 3) of the group and the chunk whose
+// swizzled position is (l & 7).
+template <int ROWS>
+__device__ __forceinline__ void load_tile(const uint8_t* __restrict__ base, int64_t stride_bytes,
+                                          int last_row, uint8_t* lds_tile, int wave, int lane) {
+  constexpr int kPerWave = ROWS / 32;
+#pragma unroll
+  for (int j = 0; j < kPerWave; ++j) {
+    const int q = wave * kPerWave + j;           // 8-row group
+    int r = q * 8 + (lane >> 3);
+    const int c = (lane & 7) ^ row_swizzle(r);
+    r = r < last_row ? r : last_row;
+    const uint8_t* g = base + (int64_t)r * stride_bytes + c * 16;
+    __builtin_amdgcn_global_load_lds((const GlobalVoid*)g, (LdsVoid*)(lds_tile + q * 1024), 16, 0, 0);
+  }
+}
+
+__device__ __forceinline__ bf16x8 read_frag(const uint8_t* lds_tile, int row, int chunk) {
+  const int pos = chunk ^ row_swizzle(row);
+  return *reinterpret_cast<const bf16x8*>(lds_tile + row * kRowBytes + pos * 16);
+}
+
+template <int BM, int BN>
+__global__ __launch_bounds__(kGemmThreads, 1) void ag_matmul_kernel(
+    const uint8_t* __restrict__ a_shard, const uint8_t* __restrict__ a_out,
+    const uint8_t* __restrict__ b_nk, uint8_t* __restrict__ c, const uint32_t* __restrict__ progress,
+    GemmSchedule s, uint64_t limit_ticks, uint32_t* status) {
+  constexpr int WM = BM / 2, WN = BN / 2;        // wave tile
+  constexpr int FM = WM / 32, FN = WN / 32;      // 32x32 fragments per wave tile
+  constexpr int kABytes = BM * kRowBytes, kBBytes = BN * kRowBytes;
+  constexpr int kStage = kABytes + kBBytes;
+  __shared__ __attribute__((aligned(1024))) uint8_t lds[2 * kStage];
+
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+  const int64_t row_stride = (int64_t)s.K * 2;
+  const int nk = s.K / kBK;
+
+  for (int step = 0;; ++step) {
+    TileRef t;
+    if (!tile_for(s, blockIdx.x, step, t)) break;
+    const uint8_t* a_base;
+    if (t.local) {
+      a_base = a_shard + (int64_t)t.a_row * row_stride;
+    } else {
+      if (progress != nullptr) wait_signal(progress + t.comm_block, limit_ticks, status, t.comm_block);
+      a_base = a_out + (int64_t)t.a_row * row_stride;
+    }
+    const uint8_t* b_base = b_nk + (int64_t)t.col0 * row_stride;
+    const int b_last = s.N - 1 - t.col0;         // clamp rows past the last column of B
+
+    f32x16 acc[FN][FM];
+#pragma unroll
+    for (int ni = 0; ni < FN; ++ni)
+#pragma unroll
+      for (int mi = 0; mi < FM; ++mi)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) acc[ni][mi][e] = 0.0f;
+
+    load_tile<BM>(a_base, row_stride, BM - 1, lds, wave, lane);
+    load_tile<BN>(b_base, row_stride, b_last, lds + kABytes, wave, lane);
+    __syncthreads();
+
+    for (int kt = 0; kt < nk; ++kt) {
+      uint8_t* cur = lds + (kt & 1) * kStage;
+      if (kt + 1 < nk) {
+        uint8_t* nxt = lds + ((kt + 1) & 1) * kStage;
+        const int64_t koff = (int64_t)(kt + 1) * kRowBytes;
+        load_tile<BM>(a_base + koff, row_stride, BM - 1, nxt, wave, lane);
+        load_tile<BN>(b_base + koff, row_stride, b_last, nxt + kABytes, wave, lane);
+      }
+      const uint8_t* la = cur;
+      const uint8_t* lb = cur + kABytes;
+#pragma unroll
+      for (int kk = 0; kk < kBK / 16; ++kk) {
+        const int chunk = kk * 2 + (lane >> 5);
+        bf16x8 af[FM], bf[FN];
+#pragma unroll
+        for (int mi = 0; mi < FM; ++mi) af[mi] = read_frag(la, wm * WM + mi * 32 + (lane & 31), chunk);
+#pragma unroll
+        for (int ni = 0; ni < FN; ++ni) bf[ni] = read_frag(lb, wn * WN + ni * 32 + (lane & 31), chunk);
+#pragma unroll
+        for (int ni = 0; ni < FN; ++ni)
+#pragma unroll
+          for (int mi = 0; mi < FM; ++mi)
+            acc[ni][mi] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bf[ni], af[mi], acc[ni][mi], 0, 0, 0);
+      }
+      __syncthreads();
+    }
+
+    // D[n][m]: lane holds row m = lane & 31 and, per group of 4 registers, the 4
+    // consecutive columns g*8 + (lane >> 5)*4 .. +3 of the 32x32 fragment.
+#pragma unroll
+    for (int mi = 0; mi < FM; ++mi) {
+      const int m = t.row0 + wm * WM + mi * 32 + (lane & 31);
+      uint8_t* c_row = c + ((int64_t)m * s.N) * 2;
+#pragma unroll
+      for (int ni = 0; ni < FN; ++ni) {
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          const int n = t.col0 + wn * WN + ni * 32 + g * 8 + (lane >> 5) * 4;
+          if (n < s.N) {
+            uint2 v;
+            v.x = pack_bf16x2(acc[ni][mi][g * 4 + 0], acc[ni][mi][g * 4 + 1]);
+            v.y = pack_bf16x2(acc[ni][mi][g * 4 + 2], acc[ni][mi][g * 4 + 3]);
+            *reinterpret_cast<uint2*>(c_row + (int64_t)n * 2) = v;
+          }
+        }
+      }
+    }
+  }
+}
+
+static int pick_tile(int M, int N, int comm_block_m, int& BM, int& BN) {
+  if (comm_block_m % 256 == 0) {
+    BM = 256;
+    BN = N >= 256 ? 256 : 128;
+  } else if (comm_block_m % 128 == 0) {
+    BM = 128;
+    BN = 128;
+  } else {
+    return -1;
+  }
+  return 0;
+}
+
+static int validate(int M, int N, int K, int rank, int world_size, int comm_block_m, const char** why) {
+  *why = nullptr;
+  if (world_size < 1 || world_size > SMR_MAX_WORLD_SIZE || rank < 0 || rank >= world_size)
+    *why = "smr_ag_matmul: rank/world_size";
+  else if (M <= 0 || N <= 0 || K <= 0)
+    *why = "smr_ag_matmul: empty shape";
+  else if (comm_block_m <= 0 || M % comm_block_m != 0 || (M / comm_block_m) % world_size != 0)
+    *why = "smr_ag_matmul: M must be world_size * splits * comm_block_m";
+  if (*why) return SMR_E_INVALID;
+  if (K % kBK != 0)
+    *why = "smr_ag_matmul: K must be a multiple of 64";
+  else if (N % 8 != 0)
+    *why = "smr_ag_matmul: N must be a multiple of 8";
+  else if (comm_block_m % 128 != 0)
+    *why = "smr_ag_matmul: rows per progress flag must be a multiple of 128";
+  if (*why) return SMR_E_UNSUPPORTED;
+  return 0;
+}
+
+static int cu_count() {
+  static int cached = 0;
+  if (cached == 0) {
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) == hipSuccess &&
+        hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0)
+      cached = n;
+    else
+      return 256;
+  }
+  return cached;
+}
+
+static GemmSchedule make_schedule(int M, int N, int K, int rank, int world_size, int comm_block_m,
+                                  int cus) {
+  GemmSchedule s;
+  s.M = M; s.N = N; s.K = K;
+  s.rank = rank; s.world_size = world_size; s.comm_block_m = comm_block_m;
+  pick_tile(M, N, comm_block_m, s.BM, s.BN);
+  const int tn = (N + s.BN - 1) / s.BN;
+  const int total = (M / s.BM) * tn;
+  int grid = (cus / 8) * 8;
+  if (grid < 8) grid = 8;
+  const int need = (total + 7) / 8 * 8;
+  s.grid = need < grid ? need : grid;
+  return s;
+}
+
+}  // namespace smr
+
+extern "C" {
+
+int smr_ag_matmul(const void* a_shard_dev, const void* a_out_dev, const void* b_nk_dev, void* c_dev,
+                  const uint32_t* progress_dev, int M, int N, int K, int rank, int world_size,
+                  int comm_block_m, uint32_t* status, void* stream) {
+  using namespace smr;
+  const char* why;
+  if (int rc = validate(M, N, K, rank, world_size, comm_block_m, &why)) return fail(rc, why);
+  if (a_shard_dev == nullptr || a_out_dev == nullptr || b_nk_dev == nullptr || c_dev == nullptr)
+    return fail(SMR_E_INVALID, "smr_ag_matmul: null pointer");
+  if ((reinterpret_cast<uintptr_t>(a_shard_dev) | reinterpret_cast<uintptr_t>(a_out_dev) |
+       reinterpret_cast<uintptr_t>(b_nk_dev) | reinterpret_cast<uintptr_t>(c_dev)) & 15u)
+    return fail(SMR_E_INVALID, "smr_ag_matmul: operands must be 16-byte aligned");
+  const GemmSchedule s = make_schedule(M, N, K, rank, world_size, comm_block_m, cu_count());
+  hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+  const uint8_t* a0 = reinterpret_cast<const uint8_t*>(a_shard_dev);
+  const uint8_t* a1 = reinterpret_cast<const uint8_t*>(a_out_dev);
+  const uint8_t* b = reinterpret_cast<const uint8_t*>(b_nk_dev);
+  uint8_t* c = reinterpret_cast<uint8_t*>(c_dev);
+  const uint64_t lim = spin_limit_ticks();
+  if (s.BM == 256 && s.BN == 256)
+    hipLaunchKernelGGL((ag_matmul_kernel<256, 256>), dim3(s.grid), dim3(kGemmThreads), 0, st, a0, a1, b,
+                       c, progress_dev, s, lim, status);
+  else if (s.BM == 256)
+    hipLaunchKernelGGL((ag_matmul_kernel<256, 128>), dim3(s.grid), dim3(kGemmThreads), 0, st, a0, a1, b,
+                       c, progress_dev, s, lim, status);
+  else
+    hipLaunchKernelGGL((ag_matmul_kernel<128, 128>), dim3(s.grid), dim3(kGemmThreads), 0, st, a0, a1, b,
+                       c, progress_dev, s, lim, status);
+  return check_hip(hipGetLastError(), "smr_ag_matmul launch");
+}
+
+int smr_ag_matmul_schedule(int M, int N, int K, int rank, int world_size, int comm_block_m,
+                           int32_t* out_records, int max_tiles) {
+  using namespace smr;
+  const char* why;
+  if (int rc = validate(M, N, K, rank, world_size, comm_block_m, &why)) return fail(rc, why);
+  // host-only: the schedule of a 256-CU part, the one the kernels are tuned for
+  const GemmSchedule s = make_schedule(M, N, K, rank, world_size, comm_block_m, 256);
+  int count = 0;
+  for (int wg = 0; wg < s.grid; ++wg) {
+    for (int step = 0;; ++step) {
+      TileRef t;
+      const int tn = (s.N + s.BN - 1) / s.BN;
+      if (step * s.grid >= (s.M / s.BM) * tn) break;
+      if (!tile_for(s, wg, step, t)) continue;
+      if (out_records != nullptr && count < max_tiles) {
+        int32_t* rec = out_records + (size_t)count * 8;
+        rec[0] = wg;
+        rec[1] = step;
+        rec[2] = t.row0;
+        rec[3] = t.col0;
+        rec[4] = s.BM;
+        rec[5] = s.BN;
+        rec[6] = t.comm_block;
+        rec[7] = t.local;
+      }
+      ++count;
+    }
+  }
+  return count;
+}
+
+}  // extern "C"

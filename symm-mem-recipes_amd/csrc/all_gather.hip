@@ -1,0 +1,95 @@
+// All-gather producer with progress flags.
+//
+// The reference drives copy engines from a side stream: one peer-to-peer copy
+// per chunk, then a stream-ordered 32-bit write that raises the chunk's flag.
+// On one GPU the same role is played by a deliberately small copy kernel: a few
+// workgroups walk the chunks in the reference's order (sources rank+1, ...,
+// rank+ws-1, rank), stream every chunk with 128-bit non-temporal loads and
+// stores, and the last workgroup to finish a chunk release-stores its flag.
+// "Last" is decided by a per-chunk arrival counter, so the flag is raised once
+// all of the chunk's bytes have been written and released.
+//
+// The grid is small on purpose: the consumer GEMM owns the compute units; the
+// producer only needs enough workgroups in flight to move 32 MiB chunks faster
+// than the GEMM consumes them.
+#include "smr_device.hpp"
+
+namespace smr {
+
+constexpr int kGatherThreads = 256;
+constexpr int kGatherDefaultWorkgroups = 32;
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(1))) u32x4 GlobalVec;
+
+__global__ __launch_bounds__(kGatherThreads) void all_gather_kernel(
+    const uint64_t* __restrict__ buffer_ptrs, uint8_t* __restrict__ a_out,
+    uint32_t* __restrict__ progress, uint32_t* __restrict__ counters, int rank, int world_size,
+    int64_t chunk_vecs, int splits_per_rank) {
+  const int nwg = gridDim.x;
+  for (int step = 0; step < world_size; ++step) {
+    const int src_rank = (rank + step + 1) % world_size;
+    for (int split = 0; split < splits_per_rank; ++split) {
+      const int idx = src_rank * splits_per_rank + split;
+      const GlobalVec* src =
+          (const GlobalVec*)(uintptr_t)buffer_ptrs[src_rank] + (int64_t)split * chunk_vecs;
+      GlobalVec* dst = (GlobalVec*)(uintptr_t)a_out + (int64_t)idx * chunk_vecs;
+      // 4 independent 16-byte slots per thread per trip
+      const int64_t stride = (int64_t)nwg * kGatherThreads;
+      int64_t i = (int64_t)blockIdx.x * kGatherThreads + threadIdx.x;
+      for (; i + 3 * stride < chunk_vecs; i += 4 * stride) {
+        u32x4 v0 = __builtin_nontemporal_load(src + i);
+        u32x4 v1 = __builtin_nontemporal_load(src + i + stride);
+        u32x4 v2 = __builtin_nontemporal_load(src + i + 2 * stride);
+        u32x4 v3 = __builtin_nontemporal_load(src + i + 3 * stride);
+        __builtin_nontemporal_store(v0, dst + i);
+        __builtin_nontemporal_store(v1, dst + i + stride);
+        __builtin_nontemporal_store(v2, dst + i + 2 * stride);
+        __builtin_nontemporal_store(v3, dst + i + 3 * stride);
+      }
+      for (; i < chunk_vecs; i += stride) {
+        u32x4 v = __builtin_nontemporal_load(src + i);
+        __builtin_nontemporal_store(v, dst + i);
+      }
+      // publish: every wave releases its stores, the workgroup meets, one thread
+      // counts the arrival; the last arrival raises the flag.
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+      __syncthreads();
+      if (threadIdx.x == 0) {
+        const uint32_t prev =
+            __hip_atomic_fetch_add(&counters[idx], 1u, __ATOMIC_ACQ_REL, kScope);
+        if (prev + 1u == (uint32_t)nwg) {
+          __hip_atomic_store(&counters[idx], 0u, __ATOMIC_RELAXED, kScope);
+          __hip_atomic_store(&progress[idx], 1u, __ATOMIC_RELEASE, kScope);
+        }
+      }
+    }
+  }
+}
+
+}  // namespace smr
+
+extern "C" int smr_all_gather_with_progress(const uint64_t* buffer_ptrs_dev, void* a_out_dev,
+                                            uint32_t* progress_dev, uint32_t* counters_dev,
+                                            int rank, int world_size, int64_t shard_bytes,
+                                            int splits_per_rank, int num_workgroups, void* stream) {
+  using namespace smr;
+  if (buffer_ptrs_dev == nullptr || a_out_dev == nullptr || progress_dev == nullptr ||
+      counters_dev == nullptr)
+    return fail(SMR_E_INVALID, "smr_all_gather_with_progress: null pointer");
+  if (world_size < 1 || world_size > SMR_MAX_WORLD_SIZE || rank < 0 || rank >= world_size)
+    return fail(SMR_E_INVALID, "smr_all_gather_with_progress: rank/world_size");
+  if (splits_per_rank < 1 || shard_bytes < 0 || shard_bytes % splits_per_rank != 0)
+    return fail(SMR_E_INVALID, "smr_all_gather_with_progress: shard must divide into the splits");
+  const int64_t chunk_bytes = shard_bytes / splits_per_rank;
+  if (chunk_bytes % 16 != 0 || (reinterpret_cast<uintptr_t>(a_out_dev) & 15u))
+    return fail(SMR_E_INVALID, "smr_all_gather_with_progress: chunks must be 16-byte multiples");
+  if (num_workgroups < 0 || num_workgroups > 1024)
+    return fail(SMR_E_INVALID, "smr_all_gather_with_progress: num_workgroups must be 0..1024");
+  const int nwg = num_workgroups == 0 ? kGatherDefaultWorkgroups : num_workgroups;
+  hipLaunchKernelGGL(all_gather_kernel, dim3(nwg), dim3(kGatherThreads), 0,
+                     reinterpret_cast<hipStream_t>(stream), buffer_ptrs_dev,
+                     reinterpret_cast<uint8_t*>(a_out_dev), progress_dev, counters_dev, rank,
+                     world_size, chunk_bytes / 16, splits_per_rank);
+  return check_hip(hipGetLastError(), "smr_all_gather_with_progress launch");
+}

@@ -1,0 +1,228 @@
+// One-shot all-reduce over the emulated peer buffers of one MI355X.
+//
+// Every thread owns 16-byte slots (8 bf16 or 4 fp32).  For a slot it issues one
+// 128-bit load per peer, all in flight together, then adds the peers into an
+// fp32 accumulator that starts at +0, strictly in rank order 0..ws-1 - the
+// vector dimension runs across elements, never across ranks, so the result is
+// bit-identical to a sequential fp32 sum - and stores one 128-bit result.
+// The kernel is bound by HBM bandwidth: (ws + 1) * 16 bytes per slot.
+//
+// Role of the workgroups (`layout`):
+//   kPlain     grid = nblocks: one rank's share, no handshake
+//   kProxy     grid = nproxy + nblocks: the first nproxy workgroups play the other
+//              ranks' halves of the handshake (8 lanes per block, no arithmetic)
+//              and are dispatched first, so they are resident and spinning by
+//              the time the rank's own workgroups arrive behind the barrier
+//   kAllRanks  grid = ws*nblocks: workgroup id -> (block = id / ws, rank = id % ws);
+//              every emulated rank reduces into its own row of `out`
+// In kAllRanks adjacent ids hold the partners of one handshake, so in-order
+// dispatch makes every partner resident by the time a later workgroup starts:
+// the spins end.
+#include "smr_device.hpp"
+
+namespace smr {
+
+enum ReduceLayout : int { kPlain = 0, kProxy = 1, kAllRanks = 2 };
+
+constexpr int kReduceThreads = 256;
+constexpr int kReduceMaxBlocks = 2048;   // 8 workgroups of 256 threads per CU on 256 CUs
+constexpr int kBlocksPerProxy = kReduceThreads / 8;
+
+struct alignas(16) Vec16 {
+  uint32_t w[4];
+};
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+// Addresses handed over as integers would otherwise be treated as generic
+// (flat) pointers; naming the global address space gives global_load/store.
+typedef __attribute__((address_space(1))) u32x4 GlobalVec;
+
+__device__ __forceinline__ Vec16 load_stream(const GlobalVec* p) {
+  u32x4 t = __builtin_nontemporal_load(p);
+  Vec16 v;
+  v.w[0] = t.x; v.w[1] = t.y; v.w[2] = t.z; v.w[3] = t.w;
+  return v;
+}
+
+__device__ __forceinline__ void store_stream(GlobalVec* p, const Vec16& v) {
+  u32x4 t = {v.w[0], v.w[1], v.w[2], v.w[3]};
+  __builtin_nontemporal_store(t, p);
+}
+
+template <bool BF16, int WS>
+__device__ __forceinline__ Vec16 sum_in_rank_order(const Vec16 (&v)[WS]) {
+  Vec16 o;
+  if constexpr (BF16) {
+    float acc[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc[e] = 0.0f;
+#pragma unroll
+    for (int r = 0; r < WS; ++r) {
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        acc[2 * k] += bf16_lo(v[r].w[k]);
+        acc[2 * k + 1] += bf16_hi(v[r].w[k]);
+      }
+    }
+#pragma unroll
+    for (int k = 0; k < 4; ++k) o.w[k] = pack_bf16x2(acc[2 * k], acc[2 * k + 1]);
+  } else {
+    float acc[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) acc[e] = 0.0f;
+#pragma unroll
+    for (int r = 0; r < WS; ++r) {
+#pragma unroll
+      for (int k = 0; k < 4; ++k) acc[k] += __uint_as_float(v[r].w[k]);
+    }
+#pragma unroll
+    for (int k = 0; k < 4; ++k) o.w[k] = __float_as_uint(acc[k]);
+  }
+  return o;
+}
+
+template <bool BF16, int WS, bool WRITE_ALL>
+__global__ __launch_bounds__(kReduceThreads) void one_shot_all_reduce_kernel(
+    const uint64_t* __restrict__ buffer_ptrs, const uint64_t* __restrict__ signal_pad_ptrs,
+    Vec16* __restrict__ out, int64_t nvec, int rank, int layout, int nblocks, int do_barrier,
+    uint64_t limit_ticks, uint32_t* status) {
+  int block = blockIdx.x;
+  if (layout == kProxy) {
+    const int nproxy = (nblocks + kBlocksPerProxy - 1) / kBlocksPerProxy;
+    if ((int)blockIdx.x < nproxy) {
+      // Peer proxies: 8 lanes per block, lane j stands in for rank j's block b.
+      const int b = blockIdx.x * kBlocksPerProxy + (threadIdx.x >> 3);
+      const int j = threadIdx.x & 7;
+      if (b < nblocks && j < WS && j != rank) {
+        uint32_t* to_rank = reinterpret_cast<uint32_t*>(signal_pad_ptrs[rank]) + (size_t)b * WS + j;
+        uint32_t* from_rank = reinterpret_cast<uint32_t*>(signal_pad_ptrs[j]) + (size_t)b * WS + rank;
+        if (!send_signal(to_rank, limit_ticks)) {
+          report(status, SMR_ST_SEND_TIMEOUT, j, b, rank);
+        } else if (!wait_signal_reset(from_rank, limit_ticks)) {
+          report(status, SMR_ST_WAIT_TIMEOUT, j, b, rank);
+        }
+      }
+      return;
+    }
+    block = blockIdx.x - nproxy;
+  } else if (layout == kAllRanks) {
+    block = blockIdx.x / WS;
+    rank = blockIdx.x % WS;
+    out += (size_t)rank * nvec;
+  }
+
+  if (do_barrier) blockwise_barrier(signal_pad_ptrs, block, rank, WS, limit_ticks, status);
+
+  GlobalVec* src[WS];
+#pragma unroll
+  for (int r = 0; r < WS; ++r) src[r] = (GlobalVec*)(uintptr_t)buffer_ptrs[r];
+  GlobalVec* dst = (GlobalVec*)(uintptr_t)out;
+
+  const int64_t stride = (int64_t)nblocks * kReduceThreads;
+  for (int64_t i = (int64_t)block * kReduceThreads + threadIdx.x; i < nvec; i += stride) {
+    Vec16 v[WS];
+#pragma unroll
+    for (int r = 0; r < WS; ++r) v[r] = load_stream(src[r] + i);
+    Vec16 o = sum_in_rank_order<BF16, WS>(v);
+    if constexpr (WRITE_ALL) {
+#pragma unroll
+      for (int r = 0; r < WS; ++r) store_stream(src[r] + i, o);
+    } else {
+      store_stream(dst + i, o);
+    }
+  }
+}
+
+template <bool BF16, int WS>
+static int launch_ws(bool write_all, dim3 grid, hipStream_t s, const uint64_t* bp, const uint64_t* sp,
+                     Vec16* out, int64_t nvec, int rank, int layout, int nblocks, int do_barrier,
+                     uint32_t* status) {
+  const uint64_t lim = spin_limit_ticks();
+  if (write_all)
+    hipLaunchKernelGGL((one_shot_all_reduce_kernel<BF16, WS, true>), grid, dim3(kReduceThreads), 0, s,
+                       bp, sp, out, nvec, rank, layout, nblocks, do_barrier, lim, status);
+  else
+    hipLaunchKernelGGL((one_shot_all_reduce_kernel<BF16, WS, false>), grid, dim3(kReduceThreads), 0, s,
+                       bp, sp, out, nvec, rank, layout, nblocks, do_barrier, lim, status);
+  return check_hip(hipGetLastError(), "smr_one_shot_all_reduce launch");
+}
+
+template <bool BF16>
+static int launch_dtype(int ws, bool write_all, dim3 grid, hipStream_t s, const uint64_t* bp,
+                        const uint64_t* sp, Vec16* out, int64_t nvec, int rank, int layout,
+                        int nblocks, int do_barrier, uint32_t* status) {
+#define SMR_WS_CASE(W)                                                                          \
+  case W:                                                                                       \
+    return launch_ws<BF16, W>(write_all, grid, s, bp, sp, out, nvec, rank, layout, nblocks,     \
+                              do_barrier, status);
+  switch (ws) {
+    SMR_WS_CASE(1) SMR_WS_CASE(2) SMR_WS_CASE(3) SMR_WS_CASE(4)
+    SMR_WS_CASE(5) SMR_WS_CASE(6) SMR_WS_CASE(7) SMR_WS_CASE(8)
+  }
+#undef SMR_WS_CASE
+  return fail(SMR_E_INVALID, "smr_one_shot_all_reduce: world_size must be 1..8");
+}
+
+}  // namespace smr
+
+extern "C" {
+
+int smr_reduce_num_blocks(int64_t numel, int dtype) {
+  const int per_vec = dtype == SMR_DTYPE_BF16 ? 8 : 4;
+  if (numel <= 0) return 0;
+  const int64_t nvec = numel / per_vec;
+  int64_t nb = (nvec + smr::kReduceThreads - 1) / smr::kReduceThreads;
+  if (nb > smr::kReduceMaxBlocks) nb = smr::kReduceMaxBlocks;
+  if (nb < 1) nb = 1;
+  return (int)nb;
+}
+
+int smr_one_shot_all_reduce(const uint64_t* buffer_ptrs_dev, const uint64_t* signal_pad_ptrs_dev,
+                            void* out, int64_t numel, int dtype, int rank, int world_size,
+                            int write_all, int barrier_mode, uint32_t* status, void* stream) {
+  using namespace smr;
+  if (dtype != SMR_DTYPE_BF16 && dtype != SMR_DTYPE_FP32)
+    return fail(SMR_E_INVALID, "smr_one_shot_all_reduce: dtype must be bf16 (0) or fp32 (1)");
+  if (world_size < 1 || world_size > SMR_MAX_WORLD_SIZE)
+    return fail(SMR_E_INVALID, "smr_one_shot_all_reduce: world_size must be 1..8");
+  if (rank < -1 || rank >= world_size)
+    return fail(SMR_E_INVALID, "smr_one_shot_all_reduce: rank out of range");
+  const int per_vec = dtype == SMR_DTYPE_BF16 ? 8 : 4;
+  if (numel < 0 || numel % per_vec != 0)
+    return fail(SMR_E_INVALID, "smr_one_shot_all_reduce: The number of elements must be 128-bit aligned.");
+  if (buffer_ptrs_dev == nullptr)
+    return fail(SMR_E_INVALID, "smr_one_shot_all_reduce: buffer_ptrs_dev is NULL");
+  if (barrier_mode != SMR_BARRIER_NONE && barrier_mode != SMR_BARRIER_PROXY)
+    return fail(SMR_E_INVALID, "smr_one_shot_all_reduce: unknown barrier_mode");
+  if (barrier_mode != SMR_BARRIER_NONE && signal_pad_ptrs_dev == nullptr)
+    return fail(SMR_E_INVALID, "smr_one_shot_all_reduce: signal pads required for the barrier");
+  if (write_all && rank < 0)
+    return fail(SMR_E_INVALID, "smr_one_shot_all_reduce: write_all needs a single rank");
+  if (!write_all && out == nullptr)
+    return fail(SMR_E_INVALID, "smr_one_shot_all_reduce: out is NULL");
+  if (out != nullptr && (reinterpret_cast<uintptr_t>(out) & 15u))
+    return fail(SMR_E_INVALID, "smr_one_shot_all_reduce: out must be 16-byte aligned");
+  if (numel == 0) return 0;
+
+  const int64_t nvec = numel / per_vec;
+  const int nblocks = smr_reduce_num_blocks(numel, dtype);
+  const int do_barrier = barrier_mode != SMR_BARRIER_NONE;
+  int layout = kPlain;
+  unsigned grid = (unsigned)nblocks;
+  if (rank < 0) {
+    layout = kAllRanks;
+    grid = (unsigned)nblocks * (unsigned)world_size;
+  } else if (do_barrier) {
+    layout = kProxy;
+    grid = (unsigned)nblocks + (unsigned)((nblocks + kBlocksPerProxy - 1) / kBlocksPerProxy);
+  }
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  Vec16* o = reinterpret_cast<Vec16*>(out);
+  if (dtype == SMR_DTYPE_BF16)
+    return launch_dtype<true>(world_size, write_all != 0, dim3(grid), s, buffer_ptrs_dev,
+                              signal_pad_ptrs_dev, o, nvec, rank, layout, nblocks, do_barrier, status);
+  return launch_dtype<false>(world_size, write_all != 0, dim3(grid), s, buffer_ptrs_dev,
+                             signal_pad_ptrs_dev, o, nvec, rank, layout, nblocks, do_barrier, status);
+}
+
+}  // extern "C"

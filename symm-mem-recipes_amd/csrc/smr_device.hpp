@@ -1,0 +1,145 @@
+// Device-side building blocks shared by every kernel of libsmr_gfx950:
+// bf16 packing, the bounded-spin flag protocol (send / wait / blockwise barrier)
+// and the host-side error plumbing.  gfx950 only.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/smr.h"
+
+namespace smr {
+
+// ---------------------------------------------------------------- host side
+void set_last_error(const char* msg);
+int fail(int code, const char* msg);            // records msg, returns code
+int check_hip(hipError_t e, const char* what);  // 0 or the hip error (recorded)
+uint64_t spin_limit_ticks();                    // current timeout in wall_clock64 ticks (0 = none)
+
+// ---------------------------------------------------------------- bf16
+__device__ __forceinline__ float bf16_lo(uint32_t w) { return __uint_as_float(w << 16); }
+__device__ __forceinline__ float bf16_hi(uint32_t w) { return __uint_as_float(w & 0xFFFF0000u); }
+
+// fp32 -> bf16, round-to-nearest-even, NaN quieted; bit pattern in the low half.
+__device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {
+  uint32_t u = __float_as_uint(f);
+  uint32_t r = (u + 0x7FFFu + ((u >> 16) & 1u)) >> 16;
+  uint32_t q = (u >> 16) | 0x40u;
+  return ((u & 0x7FFFFFFFu) > 0x7F800000u) ? q : r;
+}
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
+  return f32_to_bf16_bits(lo) | (f32_to_bf16_bits(hi) << 16);
+}
+
+// ---------------------------------------------------------------- status
+__device__ __forceinline__ void report(uint32_t* status, uint32_t code, uint32_t a, uint32_t b,
+                                       uint32_t c) {
+  if (status == nullptr) return;
+  uint32_t expected = 0u;
+  if (__hip_atomic_compare_exchange_strong(&status[0], &expected, code, __ATOMIC_RELAXED,
+                                           __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) {
+    status[1] = a;
+    status[2] = b;
+    status[3] = c;
+  }
+}
+
+// ---------------------------------------------------------------- flag protocol
+// All flags live in ordinary device memory of one GPU, so agent scope is the
+// widest scope that is ever needed here; a multi-GPU build over xGMI would use
+// __HIP_MEMORY_SCOPE_SYSTEM on fine-grained peer mappings with the same code.
+constexpr int kScope = __HIP_MEMORY_SCOPE_AGENT;
+
+// Spin helper: true while the caller may keep spinning.
+struct SpinClock {
+  uint64_t start, limit;
+  __device__ __forceinline__ explicit SpinClock(uint64_t limit_ticks)
+      : start(limit_ticks ? wall_clock64() : 0), limit(limit_ticks) {}
+  __device__ __forceinline__ bool expired() const {
+    return limit != 0 && (wall_clock64() - start) > limit;
+  }
+};
+
+// Release-CAS 0 -> 1 until it succeeds: publishes everything the calling
+// thread (and, through a preceding workgroup barrier, its workgroup) wrote.
+__device__ __forceinline__ bool send_signal(uint32_t* addr, uint64_t limit_ticks) {
+  SpinClock clk(limit_ticks);
+  for (;;) {
+    uint32_t expected = 0u;
+    if (__hip_atomic_compare_exchange_strong(addr, &expected, 1u, __ATOMIC_RELEASE,
+                                             __ATOMIC_RELAXED, kScope))
+      return true;
+    __builtin_amdgcn_s_sleep(2);
+    if (clk.expired()) return false;
+  }
+}
+
+// CAS 1 -> 0 until it succeeds (consumes and resets the flag).  Relaxed: the
+// caller acquires afterwards, once, for the whole workgroup.
+__device__ __forceinline__ bool wait_signal_reset(uint32_t* addr, uint64_t limit_ticks) {
+  SpinClock clk(limit_ticks);
+  for (;;) {
+    uint32_t expected = 1u;
+    if (__hip_atomic_compare_exchange_strong(addr, &expected, 0u, __ATOMIC_RELAXED,
+                                             __ATOMIC_RELAXED, kScope))
+      return true;
+    __builtin_amdgcn_s_sleep(2);
+    if (clk.expired()) return false;
+  }
+}
+
+// Spin (one thread) until *addr == 1; the flag is left set.
+__device__ __forceinline__ bool wait_flag_set(const uint32_t* addr, uint64_t limit_ticks) {
+  SpinClock clk(limit_ticks);
+  for (;;) {
+    if (__hip_atomic_load(addr, __ATOMIC_RELAXED, kScope) == 1u) return true;
+    __builtin_amdgcn_s_sleep(4);
+    if (clk.expired()) return false;
+  }
+}
+
+// Whole-workgroup wait on a progress flag: thread 0 spins, everyone meets at the
+// workgroup barrier, then every wave acquires so that its later loads cannot be
+// served from lines cached before the flag was set.
+__device__ __forceinline__ void wait_signal(const uint32_t* addr, uint64_t limit_ticks,
+                                            uint32_t* status, uint32_t who) {
+  if (threadIdx.x == 0) {
+    if (!wait_flag_set(addr, limit_ticks)) report(status, SMR_ST_WAIT_TIMEOUT, who, blockIdx.x, 0u);
+  }
+  __syncthreads();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+}
+
+// Blockwise barrier across the (emulated) ranks for one block index.
+//   lane r < world_size:  send on pad[r][block*ws + rank], then consume
+//   pad[rank][block*ws + r].  Pads are all-zero again afterwards.
+// Writes made by this workgroup before the call are published to the peers
+// (every wave releases before the workgroup barrier that precedes the sends);
+// after the call every thread has acquired the peers' earlier writes.
+// Returns false (to every thread of the workgroup alike) when a spin timed out.
+__device__ __forceinline__ bool blockwise_barrier(const uint64_t* signal_pad_ptrs,
+                                                  uint32_t block_id, int rank, int world_size,
+                                                  uint64_t limit_ticks, uint32_t* status) {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+  __syncthreads();
+  const int lane = threadIdx.x;
+  int bad = 0;
+  if (lane < world_size) {
+    uint32_t* remote = reinterpret_cast<uint32_t*>(signal_pad_ptrs[lane]);
+    uint32_t* local = reinterpret_cast<uint32_t*>(signal_pad_ptrs[rank]);
+    uint32_t* send = remote + (size_t)block_id * world_size + rank;
+    uint32_t* wait = local + (size_t)block_id * world_size + lane;
+    if (!send_signal(send, limit_ticks)) {
+      report(status, SMR_ST_SEND_TIMEOUT, rank, block_id, lane);
+      bad = 1;
+    } else if (!wait_signal_reset(wait, limit_ticks)) {
+      report(status, SMR_ST_WAIT_TIMEOUT, rank, block_id, lane);
+      bad = 1;
+    }
+  }
+  bad = __syncthreads_or(bad);
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+  return bad == 0;
+}
+
+}  // namespace smr

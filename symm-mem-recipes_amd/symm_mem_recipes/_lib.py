@@ -1,0 +1,85 @@
+"""ctypes binding of libsmr_gfx950.so (the C ABI declared in include/smr.h).
+
+The library is loaded, never built, from this directory; a missing library is a
+hard error - there is no fallback path of any kind.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+from typing import Optional
+
+LIB_NAME = "libsmr_gfx950.so"
+LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), LIB_NAME)
+
+DTYPE_BF16 = 0
+DTYPE_FP32 = 1
+BARRIER_NONE = 0
+BARRIER_PROXY = 1
+STATUS_WORDS = 4
+MAX_WORLD_SIZE = 8
+
+ST_OK, ST_SEND_TIMEOUT, ST_WAIT_TIMEOUT, ST_MISMATCH = 0, 1, 2, 3
+STATUS_TEXT = {
+    ST_SEND_TIMEOUT: "send_signal timed out (slot never returned to 0)",
+    ST_WAIT_TIMEOUT: "wait_signal timed out (flag never arrived)",
+    ST_MISMATCH: "signal-round checksum mismatch",
+}
+
+_p, _i, _i64, _u32 = C.c_void_p, C.c_int, C.c_int64, C.c_uint32
+
+# name -> (restype, argtypes); mirrors include/smr.h one to one
+SIGNATURES = {
+    "smr_version": (_i, []),
+    "smr_last_error_string": (C.c_char_p, []),
+    "smr_set_spin_timeout_us": (_i, [_i64]),
+    "smr_get_spin_timeout_us": (_i64, []),
+    "smr_one_shot_all_reduce": (_i, [_p, _p, _p, _i64, _i, _i, _i, _i, _i, _p, _p]),
+    "smr_reduce_num_blocks": (_i, [_i64, _i]),
+    "smr_barrier": (_i, [_p, _i, _i, _i, _i, _p, _p]),
+    "smr_send_signal": (_i, [_p, _p, _p]),
+    "smr_wait_signal": (_i, [_p, _p, _p]),
+    "smr_wait_signal_reset": (_i, [_p, _p, _p]),
+    "smr_stream_write_value32": (_i, [_p, _u32, _p]),
+    "smr_signal_round": (_i, [_p, _p, _p, _p, _p, _p, _i, _i, _i64, _i, _p, _p]),
+    "smr_all_gather_with_progress": (_i, [_p, _p, _p, _p, _i, _i, _i64, _i, _i, _p]),
+    "smr_ag_matmul": (_i, [_p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _p, _p]),
+    "smr_ag_matmul_schedule": (_i, [_i, _i, _i, _i, _i, _i, _p, _i]),
+    "smr_gemv_allreduce": (_i, [_p, _p, _p, _p, _p, _i, _i, _i, _i, _p, _p]),
+    "smr_gemv_flag_blocks": (_i, [_i]),
+}
+
+_lib: Optional[C.CDLL] = None
+
+
+class SmrError(RuntimeError):
+    pass
+
+
+def load() -> C.CDLL:
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise SmrError(
+            f"{LIB_PATH} is missing: build it with `make -C symm-mem-recipes_amd/csrc` "
+            "(hipcc, gfx950). There is no fallback implementation.")
+    lib = C.CDLL(LIB_PATH)
+    for name, (res, args) in SIGNATURES.items():
+        fn = getattr(lib, name)          # AttributeError if the symbol is not exported
+        fn.restype = res
+        fn.argtypes = args
+    _lib = lib
+    return lib
+
+
+def check(code: int, what: str) -> None:
+    """Raise on a non-zero return code.  Argument errors become AssertionError, the
+    reference's convention for contract violations
+    (symm_mem_recipes/triton_one_shot_all_reduce.py:102-105)."""
+    if code == 0:
+        return
+    msg = load().smr_last_error_string().decode("utf-8", "replace")
+    if code in (-1, -2):
+        raise AssertionError(f"{what}: {msg}")
+    raise SmrError(f"{what}: error {code}: {msg}")

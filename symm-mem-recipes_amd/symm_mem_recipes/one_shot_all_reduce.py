@@ -1,0 +1,72 @@
+"""One-shot all-reduce on the emulated symmetric buffers.
+
+Drop-in for ``one_shot_all_reduce(tensor)`` of the reference
+(symm_mem_recipes/triton_one_shot_all_reduce.py:96-125): same validation, same
+ownership (a fresh output tensor is returned), same launch stream.  The kernel
+is the library's HIP one; there is no other path.
+"""
+from __future__ import annotations
+
+import torch
+
+from . import _lib
+from .symm_mem import EmulatedSymmetricMemory
+
+NUMEL_PER_THREAD = {torch.bfloat16: 8, torch.float32: 4}      # one 128-bit slot
+_DTYPE_CODE = {torch.bfloat16: _lib.DTYPE_BF16, torch.float32: _lib.DTYPE_FP32}
+
+
+def num_blocks(numel: int, dtype: torch.dtype = torch.bfloat16) -> int:
+    """Workgroups (= barrier blocks per rank) launched for a message; the
+    counterpart of the grid formula at triton_one_shot_all_reduce.py:106-109."""
+    return _lib.load().smr_reduce_num_blocks(int(numel), _DTYPE_CODE[dtype])
+
+
+def one_shot_all_reduce(tensor: torch.Tensor, *, barrier: bool = True, write_all: bool = False,
+                        all_ranks: bool = False) -> torch.Tensor:
+    """Sum the symmetric buffers of all ranks element-wise (fp32 accumulator,
+    rank order 0..world_size-1) and return the calling rank's result.
+
+    ``barrier``    run the blockwise handshake before reading the peers
+                   (triton_one_shot_all_reduce.py:70); the other ranks' halves
+                   are played by proxy workgroups of the same launch.
+    ``write_all``  write the result back into all peer buffers in place and
+                   return the calling rank's buffer (``tensor`` itself).
+    ``all_ranks``  run every emulated rank in one launch, each behind the real
+                   barrier; returns ``[world_size, *tensor.shape]``.
+    """
+    assert tensor.dtype in _DTYPE_CODE, "Only bfloat16 and float32 are supported for now."
+    assert (
+        tensor.numel() % NUMEL_PER_THREAD[tensor.dtype] == 0
+    ), "The number of elements must be 128-bit aligned."
+    assert tensor.is_contiguous(), "tensor must be contiguous"
+    symm_mem = EmulatedSymmetricMemory.rendezvous(tensor)
+    assert symm_mem is not None, "tensor must be allocated via SymmetricMemory"
+    assert not (write_all and all_ranks)
+
+    lib = _lib.load()
+    stream = torch.cuda.current_stream(tensor.device).cuda_stream
+    if write_all:
+        output, out_ptr = tensor, 0
+    elif all_ranks:
+        output = torch.empty((symm_mem.world_size,) + tuple(tensor.shape), dtype=tensor.dtype,
+                             device=tensor.device)
+        out_ptr = output.data_ptr()
+    else:
+        output = torch.empty_like(tensor)
+        out_ptr = output.data_ptr()
+    rc = lib.smr_one_shot_all_reduce(
+        symm_mem.buffer_ptrs_dev,
+        symm_mem.signal_pad_ptrs_dev,
+        out_ptr,
+        tensor.numel(),
+        _DTYPE_CODE[tensor.dtype],
+        -1 if all_ranks else symm_mem.rank,
+        symm_mem.world_size,
+        1 if write_all else 0,
+        _lib.BARRIER_PROXY if barrier else _lib.BARRIER_NONE,
+        symm_mem.status.data_ptr(),
+        stream,
+    )
+    _lib.check(rc, "one_shot_all_reduce")
+    return output

@@ -1,0 +1,78 @@
+"""CPU-side checks of the C-ABI boundary: the library loads, exports every symbol
+include/smr.h declares, and rejects bad arguments on the host before any launch."""
+import ctypes
+import os
+import re
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared_symbols():
+    text = open(os.path.join(ROOT, "include", "smr.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(smr_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_symbols_all_exported(lib):
+    from symm_mem_recipes import _lib
+    declared = _declared_symbols()
+    assert len(declared) >= 15
+    for name in declared:
+        assert hasattr(lib, name), f"{name} declared in smr.h but not exported"
+    assert sorted(_lib.SIGNATURES) == declared, "ctypes table and header disagree"
+
+
+def test_version_and_timeout_roundtrip(lib):
+    assert lib.smr_version() == 100
+    old = lib.smr_get_spin_timeout_us()
+    assert old == 2_000_000
+    assert lib.smr_set_spin_timeout_us(1234) == 0
+    assert lib.smr_get_spin_timeout_us() == 1234
+    assert lib.smr_set_spin_timeout_us(-5) == -1
+    assert b"negative" in lib.smr_last_error_string()
+    lib.smr_set_spin_timeout_us(old)
+
+
+def test_reduce_grid(lib):
+    assert lib.smr_reduce_num_blocks(8192, 0) == 4          # 1024 slots / 256 threads
+    assert lib.smr_reduce_num_blocks(8, 0) == 1
+    assert lib.smr_reduce_num_blocks(1 << 25, 0) == 2048    # capped
+    assert lib.smr_reduce_num_blocks(0, 0) == 0
+    assert lib.smr_reduce_num_blocks(4096, 1) == 4
+
+
+def test_reduce_argument_errors_before_launch(lib):
+    # every call fails validation on the host: nothing touches a GPU
+    bad = lib.smr_one_shot_all_reduce
+    p = 0x1000
+    assert bad(p, p, p, 12, 0, 0, 8, 0, 0, None, None) == -1       # numel % 8
+    assert b"128-bit aligned" in lib.smr_last_error_string()
+    assert bad(p, p, p, 16, 2, 0, 8, 0, 0, None, None) == -1       # dtype
+    assert bad(p, p, p, 16, 0, 8, 8, 0, 0, None, None) == -1       # rank
+    assert bad(p, p, p, 16, 0, 0, 9, 0, 0, None, None) == -1       # world size
+    assert bad(None, p, p, 16, 0, 0, 8, 0, 0, None, None) == -1    # null table
+    assert bad(p, None, p, 16, 0, 0, 8, 0, 1, None, None) == -1    # barrier without pads
+    assert bad(p, p, None, 16, 0, 0, 8, 0, 0, None, None) == -1    # no output
+    assert bad(p, p, p + 4, 16, 0, 0, 8, 0, 0, None, None) == -1   # misaligned output
+    assert bad(p, p, None, 16, 0, -1, 8, 1, 0, None, None) == -1   # write_all needs a rank
+    assert bad(p, p, p, 0, 0, 0, 8, 0, 0, None, None) == 0         # empty message: no launch
+
+
+def test_barrier_argument_errors(lib):
+    assert lib.smr_barrier(None, 0, 8, 1, 1, None, None) == -1
+    assert lib.smr_barrier(0x1000, 0, 8, 0, 1, None, None) == -1
+    assert lib.smr_barrier(0x1000, 9, 8, 1, 1, None, None) == -1
+    assert lib.smr_barrier(0x1000, -1, 8, 2000, 1, None, None) == -2
+    assert lib.smr_signal_round(None, None, 0x1000, None, 0x1000, 0x1000, 8, 304, 24, 1, None, None) == -1
+    assert lib.smr_send_signal(None, None, None) == -1
+    assert lib.smr_wait_signal(None, None, None) == -1
+
+
+def test_missing_library_is_loud(monkeypatch, tmp_path):
+    from symm_mem_recipes import _lib
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "LIB_PATH", str(tmp_path / "nope.so"))
+    with pytest.raises(_lib.SmrError):
+        _lib.load()
