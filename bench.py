@@ -1,0 +1,301 @@
+#!/usr/bin/env python3
+"""Benchmark of the symmetric-memory hot path on one MI355X.
+
+A "step" is one one-shot all-reduce over 8 emulated peer buffers of bf16 resident
+in HBM (single output: one GPU's real share of the job).  Prints ONE JSON line:
+the reduce throughput in GB/s with its HBM roofline, the CPU baseline (the numpy
+oracle timed on the host), and under "extra" the other kernels of the path
+(flag-gated all-gather matmul against the bf16 MFMA roofline, split-K GEMV,
+barrier / signal-pad rounds, smaller reduce sizes with rotating buffer sets).
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--size-mib S] [--no-extra]
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+for _p in (ROOT, os.path.join(ROOT, "symm-mem-recipes_amd")):
+    if _p not in sys.path:
+        sys.path.insert(0, _p)
+
+HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
+MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
+WS = 8
+
+
+def _median(xs):
+    xs = sorted(xs)
+    return xs[len(xs) // 2]
+
+
+def _time_events(fn, iters, warm, pre=None):
+    """Median device time of fn() in microseconds, one event pair per call on the
+    launch stream; `pre` (for example a cache flush) runs before each timed call."""
+    import torch
+    for _ in range(warm):
+        fn()
+    torch.cuda.synchronize()
+    ts = []
+    for _ in range(iters):
+        if pre is not None:
+            pre()
+        a = torch.cuda.Event(enable_timing=True)
+        b = torch.cuda.Event(enable_timing=True)
+        a.record()
+        fn()
+        b.record()
+        torch.cuda.synchronize()
+        ts.append(a.elapsed_time(b) * 1e3)
+    return _median(ts)
+
+
+def bench_reduce(size_mib, steps, warmup, dev):
+    import torch
+    from symm_mem_recipes import EmulatedSymmetricMemory as SM, one_shot_all_reduce
+    nbytes = size_mib << 20
+    numel = nbytes // 2
+    t = SM.empty_strided_p2p((numel,), (1,), torch.bfloat16, dev, world_size=WS, rank=0)
+    h = SM.rendezvous(t)
+    g = torch.Generator(device=dev)
+    for r in range(WS):
+        g.manual_seed(r)
+        h.get_buffer(r, (numel,), torch.bfloat16).normal_(generator=g)
+    out = None
+    for _ in range(warmup):
+        out = one_shot_all_reduce(t, barrier=False)
+    torch.cuda.synchronize()
+    e0 = torch.cuda.Event(enable_timing=True)
+    e1 = torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record()
+    for _ in range(steps):
+        out = one_shot_all_reduce(t, barrier=False)
+    e1.record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    h.check_status()
+    dev_us = e0.elapsed_time(e1) * 1e3 / steps
+    alg_bytes = (WS + 1) * nbytes
+    # the same call behind the blockwise barrier, and the write-back-to-all variant
+    us_barrier = _time_events(lambda: one_shot_all_reduce(t, barrier=True), 20, 3)
+    us_write_all = _time_events(lambda: one_shot_all_reduce(t, barrier=False, write_all=True), 20, 3)
+    h.check_status()
+    SM.release()
+    del out
+    return dict(wall_s=wall, dev_us=dev_us, alg_bytes=alg_bytes, us_barrier=us_barrier,
+                us_write_all=us_write_all, write_all_bytes=2 * WS * nbytes)
+
+
+def bench_reduce_rotating(size_mib, dev, dtype_name="bf16"):
+    """Smaller messages fit the 256 MB last-level cache; rotate over enough buffer
+    sets (> 1 GiB in total) that every call reads from HBM."""
+    import torch
+    from symm_mem_recipes import EmulatedSymmetricMemory as SM, one_shot_all_reduce
+    dtype = torch.bfloat16 if dtype_name == "bf16" else torch.float32
+    nbytes = size_mib << 20
+    numel = nbytes // (2 if dtype == torch.bfloat16 else 4)
+    nsets = max(2, -(-(1 << 30) // (WS * nbytes)))
+    sets = []
+    for _ in range(nsets):
+        t = SM.empty_strided_p2p((numel,), (1,), dtype, dev, world_size=WS, rank=0)
+        h = SM.rendezvous(t)
+        for r in range(WS):
+            h.get_buffer(r, (numel,), dtype).normal_()
+        sets.append(t)
+    idx = [0]
+
+    def call():
+        one_shot_all_reduce(sets[idx[0] % nsets], barrier=False)
+        idx[0] += 1
+    us = _time_events(call, 40, nsets)
+    SM.release()
+    return dict(size_mib=size_mib, dtype=dtype_name, us=us, gbs=(WS + 1) * nbytes / us / 1e3,
+                frac=(WS + 1) * nbytes / us / 1e3 / HBM_PEAK_GBS, buffer_sets=nsets)
+
+
+def bench_ag_matmul(dev):
+    import torch
+    from symm_mem_recipes import EmulatedSymmetricMemory as SM, all_gather_matmul_tma_persistent
+    M, N, K = 16384, 3584, 8192
+    a_shard = SM.empty_strided_p2p((M // WS, K), (K, 1), torch.bfloat16, dev, world_size=WS, rank=0)
+    h = SM.rendezvous(a_shard)
+    g = torch.Generator(device=dev)
+    for r in range(WS):
+        g.manual_seed(r)
+        h.get_buffer(r, (M // WS, K), torch.bfloat16).normal_(0, 0.02, generator=g)
+    g.manual_seed(100)
+    b = torch.empty(N, K, dtype=torch.bfloat16, device=dev).normal_(0, 0.02, generator=g)
+    a_out = torch.cat([h.get_buffer(r, (M // WS, K), torch.bfloat16) for r in range(WS)]).contiguous()
+    c = torch.empty(M, N, dtype=torch.bfloat16, device=dev)
+    flush = torch.empty(1 << 28, dtype=torch.int32, device=dev)      # 1 GiB > last-level cache
+    flops = 2.0 * M * N * K
+    us_ungated = _time_events(lambda: all_gather_matmul_tma_persistent(a_shard, b, a_out, c, None, mm_only=True),
+                              25, 5, pre=flush.zero_)
+    us_gated = _time_events(lambda: all_gather_matmul_tma_persistent(a_shard, b, a_out, c, None),
+                            25, 5, pre=flush.zero_)
+    h.check_status()
+    us_lib = _time_events(lambda: torch.matmul(a_out, b.T, out=c), 25, 5, pre=flush.zero_)
+    SM.release()
+    return dict(workload="all-gather matmul M=16384 N=3584 K=8192 bf16, 8 shards of [2048, 8192], rank 0",
+                flops=flops, us_gated=us_gated, us_ungated=us_ungated,
+                tflops_gated=flops / us_gated / 1e6, tflops_ungated=flops / us_ungated / 1e6,
+                gating_overhead=us_gated / us_ungated - 1.0,
+                roofline={"bound": "mfma", "achieved": flops / us_gated / 1e6, "peak": MFMA_BF16_PEAK_TFLOPS,
+                          "unit": "TFLOP/s", "frac": flops / us_gated / 1e6 / MFMA_BF16_PEAK_TFLOPS,
+                          "traffic": None},
+                torch_matmul_us=us_lib, torch_matmul_tflops=flops / us_lib / 1e6)
+
+
+def bench_gemv(dev):
+    import torch
+    from symm_mem_recipes import GemvWorkspace, gemv_all_reduce
+    K = N = 8192
+    g = torch.Generator(device=dev)
+    g.manual_seed(1)
+    nw = 10                                   # rotate over 1.25 GiB of weights
+    ws_ = [torch.empty(K, N, dtype=torch.bfloat16, device=dev).normal_(0, 0.02, generator=g) for _ in range(nw)]
+    g.manual_seed(0)
+    x = torch.empty(8, K, dtype=torch.bfloat16, device=dev).normal_(generator=g)
+    res = []
+    for batch in (1, 4, 8):
+        xb = x[:batch].contiguous()
+        wsp = GemvWorkspace(batch, N, WS, dev)
+        out = torch.empty(batch, N, dtype=torch.bfloat16, device=dev)
+        idx = [0]
+
+        def call():
+            gemv_all_reduce(xb, ws_[idx[0] % nw], WS, wsp, out)
+            idx[0] += 1
+        us = _time_events(call, 40, nw)
+        wsp.check_status()
+        nbytes = K * N * 2 + batch * K * 2 + batch * N * 2
+        res.append(dict(batch=batch, us=us, gbs=nbytes / us / 1e3, frac=nbytes / us / 1e3 / HBM_PEAK_GBS))
+    return res
+
+
+def bench_barrier(dev):
+    import numpy as np
+    import torch
+    from symm_mem_recipes import EmulatedSymmetricMemory as SM, _lib, blockwise_barrier
+    lib = _lib.load()
+    blocks, chunk = 304, 65536
+    words = chunk // 4
+    t = SM.empty_strided_p2p((2 * blocks * words,), (1,), torch.int32, dev, world_size=WS)
+    h = SM.rendezvous(t)
+    rounds = 10000
+    us_flags = _time_events(lambda: blockwise_barrier(h, blocks, rounds), 3, 1) / rounds
+    h.check_status()
+    src = (torch.rand(WS, blocks, words * 2, device=dev) * 2 - 1).to(torch.bfloat16).view(torch.int32)
+    src = src.reshape(WS, blocks, words).contiguous()
+    # wrapping uint32 sum of each block's source words, stored as the same bits in int32
+    base = src.to(torch.int64).bitwise_and(0xFFFFFFFF).sum(dim=(0, 2)).bitwise_and(0xFFFFFFFF)
+    base = (base - (base >= 2 ** 31).to(torch.int64) * 2 ** 32).to(torch.int32)
+    sums = torch.zeros(WS, blocks, dtype=torch.int32, device=dev)
+    mism = torch.zeros(1, dtype=torch.int32, device=dev)
+    prounds = 1000
+    stream = torch.cuda.current_stream().cuda_stream
+
+    def payload():
+        rc = lib.smr_signal_round(src.data_ptr(), h.buffer_ptrs_dev, h.signal_pad_ptrs_dev, base.data_ptr(),
+                                  sums.data_ptr(), mism.data_ptr(), WS, blocks, chunk, prounds,
+                                  h.status.data_ptr(), stream)
+        assert rc == 0
+    us_payload = _time_events(payload, 3, 1) / prounds
+    h.check_status()
+    assert int(mism.item()) == 0, "signal-round checksum mismatch"
+    SM.release()
+    written = WS * blocks * chunk
+    return dict(workgroups=WS * blocks, rounds_flags=rounds, us_per_round_flags=us_flags,
+                rounds_payload=prounds, us_per_round_payload=us_payload,
+                payload_written_mib=written / 2 ** 20, payload_read_mib=WS * written / 2 ** 20,
+                payload_gbs=(written + WS * written) / us_payload / 1e3)
+
+
+def cpu_baseline(budget_s=10.0):
+    """The numpy oracle of the reduce on the reference's CPU-runnable case: 8 buffers
+    of 1,048,576 bf16, N(0,1) seeded per rank, fp32 accumulation in rank order."""
+    from oracle import oracle as O
+    n = 1 << 20
+    bufs = [O.seeded_normal_bf16_bits(n, seed=r) for r in range(WS)]
+    O.reduce_ref(bufs, "bf16")
+    reps = 0
+    t0 = time.perf_counter()
+    while True:
+        O.reduce_ref(bufs, "bf16")
+        reps += 1
+        el = time.perf_counter() - t0
+        if el >= budget_s:
+            break
+    nbytes = (WS + 1) * n * 2
+    return {"value": nbytes * reps / el / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
+            "sample": f"{reps} repetitions of the 8 x 1,048,576 bf16 reduce (numpy oracle, one thread) in {el:.1f} s",
+            "host_cpus": os.cpu_count()}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--size-mib", type=int, default=64)
+    ap.add_argument("--no-extra", action="store_true")
+    ap.add_argument("--cpu-seconds", type=float, default=10.0)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on exactly one GPU (the 8 ranks are emulated in one "
+              "MI355X's HBM); --gpus must be 1", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    from symm_mem_recipes import _lib
+    _lib.load()                                   # fails loudly when the HIP library is missing
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+
+    r = bench_reduce(args.size_mib, args.steps, args.warmup, dev)
+    value = r["alg_bytes"] * args.steps / r["wall_s"] / 1e9
+    achieved = r["alg_bytes"] / r["dev_us"] / 1e3
+    line = {
+        "metric": "one-shot all-reduce GB/s, 8 x bf16 peer buffers (algorithmic bytes 9*S per call)",
+        "value": value,
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": r["wall_s"] * 1e3 / args.steps,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": f"one-shot all-reduce, 8 emulated peer buffers of {args.size_mib} MiB bf16 "
+                               "N(0,1) seeded per rank, resident in HBM, single output, fp32 accumulation "
+                               "in rank order", "world_size": WS, "bytes_per_buffer": args.size_mib << 20},
+        "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": achieved / HBM_PEAK_GBS, "traffic": None},
+    }
+    extra = {
+        "reduce_kernel_us": r["dev_us"],
+        "reduce_behind_barrier_us": r["us_barrier"],
+        "reduce_write_all_us": r["us_write_all"],
+        "reduce_write_all_gbs": r["write_all_bytes"] / r["us_write_all"] / 1e3,
+    }
+    if not args.no_extra:
+        extra["reduce_rotating"] = [bench_reduce_rotating(s, dev, d)
+                                    for d in ("bf16", "fp32") for s in (8, 16)]
+        extra["all_gather_matmul"] = bench_ag_matmul(dev)
+        extra["gemv_allreduce"] = bench_gemv(dev)
+        extra["barrier"] = bench_barrier(dev)
+    line["extra"] = extra
+    line["cpu_baseline"] = cpu_baseline(args.cpu_seconds)
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

@@ -84,6 +84,12 @@ int smr_one_shot_all_reduce(const uint64_t* buffer_ptrs_dev, const uint64_t* sig
  * triton_one_shot_all_reduce.py:97-109, resized for 256 CUs. */
 int smr_reduce_num_blocks(int64_t numel, int dtype);
 
+/* Tuning knob: threads per workgroup (multiple of 64, <= 1024) and the cap on
+ * workgroups of the reduce; 0 restores a default.  Process-wide.  The reference
+ * hard-codes its counterparts (MAX_NUM_BLOCKS, NUM_WARPS,
+ * triton_one_shot_all_reduce.py:97-100). */
+int smr_set_reduce_launch(int threads, int max_blocks);
+
 /* Blockwise barrier, `rounds` back-to-back rounds on `num_blocks` blocks.
  * Replaces barrier_test_kernel / barrier_test (symm_mem_recipes/triton_barrier.py:156-170)
  * around the device function blockwise_barrier (:50-153).
@@ -156,7 +162,14 @@ int smr_ag_matmul(const void* a_shard_dev, const void* a_out_dev, const void* b_
  * returns the number of tiles, or a negative SMR_E_* code.
  * Counterpart of the index arithmetic at triton_all_gather_matmul.py:125-174. */
 int smr_ag_matmul_schedule(int M, int N, int K, int rank, int world_size, int comm_block_m,
-                           int32_t* out_records, int max_tiles);
+                           int gated, int32_t* out_records, int max_tiles);
+
+/* Workgroups smr_ag_matmul launches on the current device for this shape; a
+ * gated launch (progress_dev != NULL) keeps at least 8 compute units free for the
+ * producer, whose workgroup count should not exceed the number left free.
+ * Host-only, no reference counterpart (the reference's producer is a copy
+ * engine and needs no compute units, triton_all_gather_matmul.py:46-49). */
+int smr_ag_matmul_grid(int M, int N, int K, int world_size, int comm_block_m, int gated);
 
 /* Split-K GEMV + rank-ordered combine through signal-pad flags.  No reference
  * code exists for it in symm_mem_recipes; it reuses the send/wait protocol of

@@ -22,6 +22,8 @@
 //     contiguous run of the tile order - 8 row tiles x 4 column tiles when the
 //     pass is full - so the workgroups that share an L2 also share A rows and
 //     B columns.
+#include <type_traits>
+
 #include "smr_device.hpp"
 
 namespace smr {
@@ -81,61 +83,110 @@ __host__ __device__ inline bool tile_for(const GemmSchedule& s, int wg, int step
 }
 
 // Position swizzle of an LDS row.
-__device__ __forceinline__ int row_swizzle(int r) { return (r ^ (r >> 3)) & 7; }
+__host__ __device__ inline int row_swizzle(int r) { return (r ^ (r >> 3)) & 7; }
 
-// Bring ROWS x 64 bf16 (rows `stride_bytes` apart, clamped to `last_row`) into
-// a swizzled LDS tile.  One wave instruction fills 8 rows = 1 KiB of LDS in lane
-// order, so lane l carries row (l >> 3) of the group and the chunk whose
-// swizzled position is (l & 7).
-template <int ROWS>
-__device__ __forceinline__ void load_tile(const uint8_t* __restrict__ base, int64_t stride_bytes,
-                                          int last_row, uint8_t* lds_tile, int wave, int lane) {
-  constexpr int kPerWave = ROWS / 32;
+typedef __attribute__((address_space(3))) const bf16x8 LdsFrag;
+
+__device__ __forceinline__ uint32_t lds_offset_of(const void* p) {
+  return (uint32_t)(uintptr_t)(LdsVoid*)p;
+}
+__device__ __forceinline__ bf16x8 lds_read_frag(uint32_t addr) {
+  return *reinterpret_cast<LdsFrag*>((uintptr_t)addr);
+}
+
+// One wave instruction of a direct-to-LDS tile load: 64 lanes x 16 B land at
+// lds_dst + lane*16 (one 8-row group, 1 KiB); `voff` is the lane's byte offset
+// from the uniform global base.
+__device__ __forceinline__ void load_group(const uint8_t* base, uint32_t voff, uint32_t lds_dst) {
+  __builtin_amdgcn_global_load_lds((const GlobalVoid*)(base + voff), (LdsVoid*)(uintptr_t)lds_dst, 16, 0, 0);
+}
+
+// Scheduling hint: spread NDS LDS reads evenly under NMFMA matrix instructions.
+template <int NMFMA, int NDS>
+__device__ __forceinline__ void interleave_mfma_dsread() {
+  constexpr int kPer = NMFMA / NDS;     // MFMAs ahead of each LDS read
 #pragma unroll
-  for (int j = 0; j < kPerWave; ++j) {
-    const int q = wave * kPerWave + j;           // 8-row group
-    int r = q * 8 + (lane >> 3);
-    const int c = (lane & 7) ^ row_swizzle(r);
-    r = r < last_row ? r : last_row;
-    const uint8_t* g = base + (int64_t)r * stride_bytes + c * 16;
-    __builtin_amdgcn_global_load_lds((const GlobalVoid*)g, (LdsVoid*)(lds_tile + q * 1024), 16, 0, 0);
+  for (int i = 0; i < NDS; ++i) {
+    __builtin_amdgcn_sched_group_barrier(0x008, kPer, 0);   // MFMA
+    __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);      // DS read
   }
 }
 
-__device__ __forceinline__ bf16x8 read_frag(const uint8_t* lds_tile, int row, int chunk) {
-  const int pos = chunk ^ row_swizzle(row);
-  return *reinterpret_cast<const bf16x8*>(lds_tile + row * kRowBytes + pos * 16);
-}
+template <int BM, int BN>
+struct GemmTile {
+  static constexpr int WM = BM / 2, WN = BN / 2;        // wave tile (2 x 2 waves)
+  static constexpr int FM = WM / 32, FN = WN / 32;      // 32x32 fragments per wave tile
+  static constexpr int GA = BM / 32, GB = BN / 32;      // 8-row load groups per wave and stage
+  static constexpr int kABytes = BM * kRowBytes, kBBytes = BN * kRowBytes;
+  // LDS map: A stage 0 | A stage 1 | B stage 0 | B stage 1.  The second stage of an
+  // operand is a 16-bit immediate away from the first.
+  static constexpr int kBBase = 2 * kABytes;
+  static constexpr int kLdsBytes = 2 * (kABytes + kBBytes);
+};
 
 template <int BM, int BN>
 __global__ __launch_bounds__(kGemmThreads, 1) void ag_matmul_kernel(
     const uint8_t* __restrict__ a_shard, const uint8_t* __restrict__ a_out,
     const uint8_t* __restrict__ b_nk, uint8_t* __restrict__ c, const uint32_t* __restrict__ progress,
     GemmSchedule s, uint64_t limit_ticks, uint32_t* status) {
-  constexpr int WM = BM / 2, WN = BN / 2;        // wave tile
-  constexpr int FM = WM / 32, FN = WN / 32;      // 32x32 fragments per wave tile
-  constexpr int kABytes = BM * kRowBytes, kBBytes = BN * kRowBytes;
-  constexpr int kStage = kABytes + kBBytes;
-  __shared__ __attribute__((aligned(1024))) uint8_t lds[2 * kStage];
+  using T = GemmTile<BM, BN>;
+  constexpr int WM = T::WM, WN = T::WN, FM = T::FM, FN = T::FN, GA = T::GA, GB = T::GB;
+  __shared__ __attribute__((aligned(1024))) uint8_t lds[T::kLdsBytes];
 
   const int lane = threadIdx.x & 63;
-  const int wave = threadIdx.x >> 6;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int wm = wave >> 1, wn = wave & 1;
-  const int64_t row_stride = (int64_t)s.K * 2;
+  const int half = lane >> 5;
+  const uint32_t row_stride = (uint32_t)s.K * 2u;
   const int nk = s.K / kBK;
+  const uint32_t lds0 = lds_offset_of(lds);
+
+  // ---- per-lane fragment read addresses (stage 0).  Row r = w*W + f*32 + (lane & 31)
+  // has swizzle ((lane & 7) ^ ((lane >> 3) & 3)) ^ ((f & 1) << 2); K step kk wants
+  // chunk 2*kk + half.  Hence position = t ^ (v << 1) with the per-lane constant
+  // t = half ^ (lane & 7) ^ ((lane >> 3) & 3) and v = kk ^ ((f & 1) << 1): four
+  // variants per operand, everything else is an immediate offset.
+  const int t = half ^ (lane & 7) ^ ((lane >> 3) & 3);
+  uint32_t a_fr[4], b_fr[4];
+#pragma unroll
+  for (int v = 0; v < 4; ++v) {
+    a_fr[v] = lds0 + (uint32_t)((wm * WM + (lane & 31)) * kRowBytes + ((t ^ (v << 1)) << 4));
+    b_fr[v] = lds0 + T::kBBase + (uint32_t)((wn * WN + (lane & 31)) * kRowBytes + ((t ^ (v << 1)) << 4));
+  }
+
+  // ---- per-lane global offsets of the tile loads.  Load group q = wave*G + j holds
+  // rows q*8 .. q*8+7; lane l carries row q*8 + (l >> 3) and the chunk whose swizzled
+  // position is (l & 7): chunk = (l & 7) ^ (l >> 3) ^ (q & 7).
+  const int u = (lane & 7) ^ (lane >> 3);
+  uint32_t a_off[GA];
+#pragma unroll
+  for (int j = 0; j < GA; ++j) {
+    const int q = wave * GA + j;
+    a_off[j] = (uint32_t)(q * 8 + (lane >> 3)) * row_stride + (uint32_t)((u ^ (q & 7)) << 4);
+  }
 
   for (int step = 0;; ++step) {
-    TileRef t;
-    if (!tile_for(s, blockIdx.x, step, t)) break;
+    TileRef tile;
+    if (!tile_for(s, blockIdx.x, step, tile)) break;
     const uint8_t* a_base;
-    if (t.local) {
-      a_base = a_shard + (int64_t)t.a_row * row_stride;
+    if (tile.local) {
+      a_base = a_shard + (int64_t)tile.a_row * row_stride;
     } else {
-      if (progress != nullptr) wait_signal(progress + t.comm_block, limit_ticks, status, t.comm_block);
-      a_base = a_out + (int64_t)t.a_row * row_stride;
+      if (progress != nullptr)
+        wait_signal(progress + tile.comm_block, limit_ticks, status, tile.comm_block);
+      a_base = a_out + (int64_t)tile.a_row * row_stride;
     }
-    const uint8_t* b_base = b_nk + (int64_t)t.col0 * row_stride;
-    const int b_last = s.N - 1 - t.col0;         // clamp rows past the last column of B
+    const uint8_t* b_base = b_nk + (int64_t)tile.col0 * row_stride;
+    // rows of B past the last column are clamped: they feed outputs that are never stored
+    const int b_last = s.N - 1 - tile.col0;
+    uint32_t b_off[GB];
+#pragma unroll
+    for (int j = 0; j < GB; ++j) {
+      const int q = wave * GB + j;
+      int r = q * 8 + (lane >> 3);
+      r = r < b_last ? r : b_last;
+      b_off[j] = (uint32_t)r * row_stride + (uint32_t)((u ^ (q & 7)) << 4);
+    }
 
     f32x16 acc[FN][FM];
 #pragma unroll
@@ -145,48 +196,85 @@ __global__ __launch_bounds__(kGemmThreads, 1) void ag_matmul_kernel(
 #pragma unroll
         for (int e = 0; e < 16; ++e) acc[ni][mi][e] = 0.0f;
 
-    load_tile<BM>(a_base, row_stride, BM - 1, lds, wave, lane);
-    load_tile<BN>(b_base, row_stride, b_last, lds + kABytes, wave, lane);
+    auto load_stage = [&](int stage, int kt) {
+      const uint8_t* ak = a_base + (int64_t)kt * kRowBytes;
+      const uint8_t* bk = b_base + (int64_t)kt * kRowBytes;
+      const uint32_t la = lds0 + stage * T::kABytes + wave * (GA * 1024);
+      const uint32_t lb = lds0 + T::kBBase + stage * T::kBBytes + wave * (GB * 1024);
+#pragma unroll
+      for (int j = 0; j < GA; ++j) load_group(ak, a_off[j], la + j * 1024);
+#pragma unroll
+      for (int j = 0; j < GB; ++j) load_group(bk, b_off[j], lb + j * 1024);
+    };
+    auto read_frags = [&](bf16x8 (&af)[FM], bf16x8 (&bf)[FN], int stage, int kk) {
+#pragma unroll
+      for (int mi = 0; mi < FM; ++mi)
+        af[mi] = lds_read_frag(a_fr[kk ^ ((mi & 1) << 1)] + stage * T::kABytes + mi * (32 * kRowBytes));
+#pragma unroll
+      for (int ni = 0; ni < FN; ++ni)
+        bf[ni] = lds_read_frag(b_fr[kk ^ ((ni & 1) << 1)] + stage * T::kBBytes + ni * (32 * kRowBytes));
+    };
+    auto mfma_all = [&](const bf16x8 (&af)[FM], const bf16x8 (&bf)[FN]) {
+#pragma unroll
+      for (int ni = 0; ni < FN; ++ni)
+#pragma unroll
+        for (int mi = 0; mi < FM; ++mi)
+          acc[ni][mi] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bf[ni], af[mi], acc[ni][mi], 0, 0, 0);
+    };
+
+    // Prologue: both LDS stages in flight, then the first fragments.
+    load_stage(0, 0);
+    if (nk > 1) load_stage(1, 1);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
 
-    for (int kt = 0; kt < nk; ++kt) {
-      uint8_t* cur = lds + (kt & 1) * kStage;
-      if (kt + 1 < nk) {
-        uint8_t* nxt = lds + ((kt + 1) & 1) * kStage;
-        const int64_t koff = (int64_t)(kt + 1) * kRowBytes;
-        load_tile<BM>(a_base + koff, row_stride, BM - 1, nxt, wave, lane);
-        load_tile<BN>(b_base + koff, row_stride, b_last, nxt + kABytes, wave, lane);
-      }
-      const uint8_t* la = cur;
-      const uint8_t* lb = cur + kABytes;
-#pragma unroll
-      for (int kk = 0; kk < kBK / 16; ++kk) {
-        const int chunk = kk * 2 + (lane >> 5);
-        bf16x8 af[FM], bf[FN];
-#pragma unroll
-        for (int mi = 0; mi < FM; ++mi) af[mi] = read_frag(la, wm * WM + mi * 32 + (lane & 31), chunk);
-#pragma unroll
-        for (int ni = 0; ni < FN; ++ni) bf[ni] = read_frag(lb, wn * WN + ni * 32 + (lane & 31), chunk);
-#pragma unroll
-        for (int ni = 0; ni < FN; ++ni)
-#pragma unroll
-          for (int mi = 0; mi < FM; ++mi)
-            acc[ni][mi] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bf[ni], af[mi], acc[ni][mi], 0, 0, 0);
-      }
-      __syncthreads();
+    // Fragment double buffer: while the MFMAs of K step kk run, the fragments of
+    // step kk+1 are read.  The workgroup barrier sits before the last K step of a
+    // stage, right after that stage's last fragment reads: from there on the stage
+    // is free, so the loads of stage kt+2 are issued into it and have a whole stage
+    // of MFMAs to land, and the first fragments of stage kt+1 are read under the
+    // MFMAs of the last K step.
+    bf16x8 af0[FM], bf0[FN], af1[FM], bf1[FN];
+    read_frags(af0, bf0, 0, 0);
+
+    auto stage_body = [&](auto stage_tag, int kt) {
+      constexpr int S = decltype(stage_tag)::value;
+      read_frags(af1, bf1, S, 1);
+      mfma_all(af0, bf0);
+      interleave_mfma_dsread<FM * FN, FM + FN>();
+      read_frags(af0, bf0, S, 2);
+      mfma_all(af1, bf1);
+      interleave_mfma_dsread<FM * FN, FM + FN>();
+      read_frags(af1, bf1, S, 3);
+      mfma_all(af0, bf0);
+      interleave_mfma_dsread<FM * FN, FM + FN>();
+      // The compiler does not track direct-to-LDS loads across the loop back
+      // edge: wait for this wave's own loads explicitly before the barrier.
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      __syncthreads();     // stage S fully read by everyone; the other stage has landed
+      if (kt + 2 < nk) load_stage(S, kt + 2);
+      if (kt + 1 < nk) read_frags(af0, bf0, S ^ 1, 0);
+      mfma_all(af1, bf1);
+    };
+    int kt = 0;
+    for (; kt + 1 < nk; kt += 2) {
+      stage_body(std::integral_constant<int, 0>{}, kt);
+      stage_body(std::integral_constant<int, 1>{}, kt + 1);
     }
+    if (kt < nk) stage_body(std::integral_constant<int, 0>{}, kt);
+    __syncthreads();       // the next tile's prologue overwrites both stages
 
     // D[n][m]: lane holds row m = lane & 31 and, per group of 4 registers, the 4
     // consecutive columns g*8 + (lane >> 5)*4 .. +3 of the 32x32 fragment.
 #pragma unroll
     for (int mi = 0; mi < FM; ++mi) {
-      const int m = t.row0 + wm * WM + mi * 32 + (lane & 31);
+      const int m = tile.row0 + wm * WM + mi * 32 + (lane & 31);
       uint8_t* c_row = c + ((int64_t)m * s.N) * 2;
 #pragma unroll
       for (int ni = 0; ni < FN; ++ni) {
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
-          const int n = t.col0 + wn * WN + ni * 32 + g * 8 + (lane >> 5) * 4;
+          const int n = tile.col0 + wn * WN + ni * 32 + g * 8 + half * 4;
           if (n < s.N) {
             uint2 v;
             v.x = pack_bf16x2(acc[ni][mi][g * 4 + 0], acc[ni][mi][g * 4 + 1]);
@@ -244,18 +332,26 @@ static int cu_count() {
   return cached;
 }
 
+// Persistent grid: the fewest workgroups (a multiple of 8, one per XCD slot) that
+// still finish in the minimum number of passes.  A gated launch leaves at least
+// kReservedCus compute units to the producer: a workgroup of this kernel fills a
+// compute unit's register file, so a producer that arrives late would otherwise
+// find no room while the consumers spin on its flags.
+constexpr int kReservedCus = 8;
+
 static GemmSchedule make_schedule(int M, int N, int K, int rank, int world_size, int comm_block_m,
-                                  int cus) {
+                                  int cus, bool gated) {
   GemmSchedule s;
   s.M = M; s.N = N; s.K = K;
   s.rank = rank; s.world_size = world_size; s.comm_block_m = comm_block_m;
   pick_tile(M, N, comm_block_m, s.BM, s.BN);
   const int tn = (N + s.BN - 1) / s.BN;
   const int total = (M / s.BM) * tn;
-  int grid = (cus / 8) * 8;
-  if (grid < 8) grid = 8;
-  const int need = (total + 7) / 8 * 8;
-  s.grid = need < grid ? need : grid;
+  int max_grid = ((gated ? cus - kReservedCus : cus) / 8) * 8;
+  if (max_grid < 8) max_grid = 8;
+  const int passes = (total + max_grid - 1) / max_grid;
+  const int need = ((total + passes - 1) / passes + 7) / 8 * 8;
+  s.grid = need < max_grid ? need : max_grid;
   return s;
 }
 
@@ -274,7 +370,7 @@ int smr_ag_matmul(const void* a_shard_dev, const void* a_out_dev, const void* b_
   if ((reinterpret_cast<uintptr_t>(a_shard_dev) | reinterpret_cast<uintptr_t>(a_out_dev) |
        reinterpret_cast<uintptr_t>(b_nk_dev) | reinterpret_cast<uintptr_t>(c_dev)) & 15u)
     return fail(SMR_E_INVALID, "smr_ag_matmul: operands must be 16-byte aligned");
-  const GemmSchedule s = make_schedule(M, N, K, rank, world_size, comm_block_m, cu_count());
+  const GemmSchedule s = make_schedule(M, N, K, rank, world_size, comm_block_m, cu_count(), progress_dev != nullptr);
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
   const uint8_t* a0 = reinterpret_cast<const uint8_t*>(a_shard_dev);
   const uint8_t* a1 = reinterpret_cast<const uint8_t*>(a_out_dev);
@@ -293,13 +389,20 @@ int smr_ag_matmul(const void* a_shard_dev, const void* a_out_dev, const void* b_
   return check_hip(hipGetLastError(), "smr_ag_matmul launch");
 }
 
+int smr_ag_matmul_grid(int M, int N, int K, int world_size, int comm_block_m, int gated) {
+  using namespace smr;
+  const char* why;
+  if (int rc = validate(M, N, K, 0, world_size, comm_block_m, &why)) return fail(rc, why);
+  return make_schedule(M, N, K, 0, world_size, comm_block_m, cu_count(), gated != 0).grid;
+}
+
 int smr_ag_matmul_schedule(int M, int N, int K, int rank, int world_size, int comm_block_m,
-                           int32_t* out_records, int max_tiles) {
+                           int gated, int32_t* out_records, int max_tiles) {
   using namespace smr;
   const char* why;
   if (int rc = validate(M, N, K, rank, world_size, comm_block_m, &why)) return fail(rc, why);
   // host-only: the schedule of a 256-CU part, the one the kernels are tuned for
-  const GemmSchedule s = make_schedule(M, N, K, rank, world_size, comm_block_m, 256);
+  const GemmSchedule s = make_schedule(M, N, K, rank, world_size, comm_block_m, 256, gated != 0);
   int count = 0;
   for (int wg = 0; wg < s.grid; ++wg) {
     for (int step = 0;; ++step) {

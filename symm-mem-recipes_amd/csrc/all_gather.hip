@@ -16,8 +16,11 @@
 
 namespace smr {
 
-constexpr int kGatherThreads = 256;
-constexpr int kGatherDefaultWorkgroups = 32;
+// 1024-thread workgroups: a producer workgroup then fills one compute unit by
+// itself, so "num_workgroups" is also the number of compute units it can occupy
+// whichever of the two kernels is dispatched first.
+constexpr int kGatherThreads = 1024;
+constexpr int kGatherDefaultWorkgroups = 8;
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef __attribute__((address_space(1))) u32x4 GlobalVec;

@@ -24,9 +24,11 @@ namespace smr {
 
 enum ReduceLayout : int { kPlain = 0, kProxy = 1, kAllRanks = 2 };
 
-constexpr int kReduceThreads = 256;
-constexpr int kReduceMaxBlocks = 2048;   // 8 workgroups of 256 threads per CU on 256 CUs
-constexpr int kBlocksPerProxy = kReduceThreads / 8;
+constexpr int kReduceMaxThreads = 1024;
+// Launch shape (threads per workgroup, cap on workgroups = barrier blocks per
+// rank); smr_set_reduce_launch overrides the defaults.
+static int g_reduce_threads = 256;
+static int g_reduce_max_blocks = 2048;   // 8 workgroups of 256 threads per CU on 256 CUs
 
 struct alignas(16) Vec16 {
   uint32_t w[4];
@@ -82,16 +84,18 @@ __device__ __forceinline__ Vec16 sum_in_rank_order(const Vec16 (&v)[WS]) {
 }
 
 template <bool BF16, int WS, bool WRITE_ALL>
-__global__ __launch_bounds__(kReduceThreads) void one_shot_all_reduce_kernel(
+__global__ __launch_bounds__(kReduceMaxThreads) void one_shot_all_reduce_kernel(
     const uint64_t* __restrict__ buffer_ptrs, const uint64_t* __restrict__ signal_pad_ptrs,
     Vec16* __restrict__ out, int64_t nvec, int rank, int layout, int nblocks, int do_barrier,
     uint64_t limit_ticks, uint32_t* status) {
   int block = blockIdx.x;
+  const int nthreads = blockDim.x;
   if (layout == kProxy) {
-    const int nproxy = (nblocks + kBlocksPerProxy - 1) / kBlocksPerProxy;
+    const int per_proxy = nthreads >> 3;
+    const int nproxy = (nblocks + per_proxy - 1) / per_proxy;
     if ((int)blockIdx.x < nproxy) {
       // Peer proxies: 8 lanes per block, lane j stands in for rank j's block b.
-      const int b = blockIdx.x * kBlocksPerProxy + (threadIdx.x >> 3);
+      const int b = blockIdx.x * per_proxy + (threadIdx.x >> 3);
       const int j = threadIdx.x & 7;
       if (b < nblocks && j < WS && j != rank) {
         uint32_t* to_rank = reinterpret_cast<uint32_t*>(signal_pad_ptrs[rank]) + (size_t)b * WS + j;
@@ -118,8 +122,8 @@ __global__ __launch_bounds__(kReduceThreads) void one_shot_all_reduce_kernel(
   for (int r = 0; r < WS; ++r) src[r] = (GlobalVec*)(uintptr_t)buffer_ptrs[r];
   GlobalVec* dst = (GlobalVec*)(uintptr_t)out;
 
-  const int64_t stride = (int64_t)nblocks * kReduceThreads;
-  for (int64_t i = (int64_t)block * kReduceThreads + threadIdx.x; i < nvec; i += stride) {
+  const int64_t stride = (int64_t)nblocks * nthreads;
+  for (int64_t i = (int64_t)block * nthreads + threadIdx.x; i < nvec; i += stride) {
     Vec16 v[WS];
 #pragma unroll
     for (int r = 0; r < WS; ++r) v[r] = load_stream(src[r] + i);
@@ -139,10 +143,10 @@ static int launch_ws(bool write_all, dim3 grid, hipStream_t s, const uint64_t* b
                      uint32_t* status) {
   const uint64_t lim = spin_limit_ticks();
   if (write_all)
-    hipLaunchKernelGGL((one_shot_all_reduce_kernel<BF16, WS, true>), grid, dim3(kReduceThreads), 0, s,
+    hipLaunchKernelGGL((one_shot_all_reduce_kernel<BF16, WS, true>), grid, dim3(g_reduce_threads), 0, s,
                        bp, sp, out, nvec, rank, layout, nblocks, do_barrier, lim, status);
   else
-    hipLaunchKernelGGL((one_shot_all_reduce_kernel<BF16, WS, false>), grid, dim3(kReduceThreads), 0, s,
+    hipLaunchKernelGGL((one_shot_all_reduce_kernel<BF16, WS, false>), grid, dim3(g_reduce_threads), 0, s,
                        bp, sp, out, nvec, rank, layout, nblocks, do_barrier, lim, status);
   return check_hip(hipGetLastError(), "smr_one_shot_all_reduce launch");
 }
@@ -167,12 +171,24 @@ static int launch_dtype(int ws, bool write_all, dim3 grid, hipStream_t s, const 
 
 extern "C" {
 
+int smr_set_reduce_launch(int threads, int max_blocks) {
+  if (threads == 0) threads = 256;
+  if (max_blocks == 0) max_blocks = 2048;
+  if (threads < 64 || threads > smr::kReduceMaxThreads || (threads & 63) != 0)
+    return smr::fail(SMR_E_INVALID, "smr_set_reduce_launch: threads must be a multiple of 64 in 64..1024");
+  if (max_blocks < 1 || max_blocks > 4096)
+    return smr::fail(SMR_E_INVALID, "smr_set_reduce_launch: max_blocks must be 1..4096");
+  smr::g_reduce_threads = threads;
+  smr::g_reduce_max_blocks = max_blocks;
+  return 0;
+}
+
 int smr_reduce_num_blocks(int64_t numel, int dtype) {
   const int per_vec = dtype == SMR_DTYPE_BF16 ? 8 : 4;
   if (numel <= 0) return 0;
   const int64_t nvec = numel / per_vec;
-  int64_t nb = (nvec + smr::kReduceThreads - 1) / smr::kReduceThreads;
-  if (nb > smr::kReduceMaxBlocks) nb = smr::kReduceMaxBlocks;
+  int64_t nb = (nvec + smr::g_reduce_threads - 1) / smr::g_reduce_threads;
+  if (nb > smr::g_reduce_max_blocks) nb = smr::g_reduce_max_blocks;
   if (nb < 1) nb = 1;
   return (int)nb;
 }
@@ -214,7 +230,8 @@ int smr_one_shot_all_reduce(const uint64_t* buffer_ptrs_dev, const uint64_t* sig
     grid = (unsigned)nblocks * (unsigned)world_size;
   } else if (do_barrier) {
     layout = kProxy;
-    grid = (unsigned)nblocks + (unsigned)((nblocks + kBlocksPerProxy - 1) / kBlocksPerProxy);
+    const int per_proxy = g_reduce_threads / 8;
+    grid = (unsigned)nblocks + (unsigned)((nblocks + per_proxy - 1) / per_proxy);
   }
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
   Vec16* o = reinterpret_cast<Vec16*>(out);

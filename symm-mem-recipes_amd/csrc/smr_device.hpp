@@ -60,40 +60,58 @@ struct SpinClock {
   }
 };
 
+// Back-off between polls of a flag: 64 clocks at first, doubling up to 2048.
+// Every poll of an agent-scope flag is a trip to memory, so a tight spin by
+// thousands of waiting lanes would starve the very atomics they wait for.
+__device__ __forceinline__ void backoff_sleep(uint32_t& level) {
+  switch (level) {
+    case 0: __builtin_amdgcn_s_sleep(1); break;
+    case 1: __builtin_amdgcn_s_sleep(2); break;
+    case 2: __builtin_amdgcn_s_sleep(4); break;
+    case 3: __builtin_amdgcn_s_sleep(8); break;
+    case 4: __builtin_amdgcn_s_sleep(16); break;
+    default: __builtin_amdgcn_s_sleep(32); break;
+  }
+  if (level < 5) ++level;
+}
+
+// CAS `from` -> `to` until it succeeds.  Relaxed: the callers put one release
+// fence before and one acquire fence after the whole handshake instead of paying
+// a cache write-back on every attempt.
+__device__ __forceinline__ bool spin_cas(uint32_t* addr, uint32_t from, uint32_t to,
+                                         uint64_t limit_ticks) {
+  SpinClock clk(limit_ticks);
+  uint32_t level = 0;
+  for (;;) {
+    uint32_t expected = from;
+    if (__hip_atomic_compare_exchange_strong(addr, &expected, to, __ATOMIC_RELAXED,
+                                             __ATOMIC_RELAXED, kScope))
+      return true;
+    backoff_sleep(level);
+    if (clk.expired()) return false;
+  }
+}
+
 // Release-CAS 0 -> 1 until it succeeds: publishes everything the calling
 // thread (and, through a preceding workgroup barrier, its workgroup) wrote.
 __device__ __forceinline__ bool send_signal(uint32_t* addr, uint64_t limit_ticks) {
-  SpinClock clk(limit_ticks);
-  for (;;) {
-    uint32_t expected = 0u;
-    if (__hip_atomic_compare_exchange_strong(addr, &expected, 1u, __ATOMIC_RELEASE,
-                                             __ATOMIC_RELAXED, kScope))
-      return true;
-    __builtin_amdgcn_s_sleep(2);
-    if (clk.expired()) return false;
-  }
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+  return spin_cas(addr, 0u, 1u, limit_ticks);
 }
 
 // CAS 1 -> 0 until it succeeds (consumes and resets the flag).  Relaxed: the
 // caller acquires afterwards, once, for the whole workgroup.
 __device__ __forceinline__ bool wait_signal_reset(uint32_t* addr, uint64_t limit_ticks) {
-  SpinClock clk(limit_ticks);
-  for (;;) {
-    uint32_t expected = 1u;
-    if (__hip_atomic_compare_exchange_strong(addr, &expected, 0u, __ATOMIC_RELAXED,
-                                             __ATOMIC_RELAXED, kScope))
-      return true;
-    __builtin_amdgcn_s_sleep(2);
-    if (clk.expired()) return false;
-  }
+  return spin_cas(addr, 1u, 0u, limit_ticks);
 }
 
 // Spin (one thread) until *addr == 1; the flag is left set.
 __device__ __forceinline__ bool wait_flag_set(const uint32_t* addr, uint64_t limit_ticks) {
   SpinClock clk(limit_ticks);
+  uint32_t level = 0;
   for (;;) {
     if (__hip_atomic_load(addr, __ATOMIC_RELAXED, kScope) == 1u) return true;
-    __builtin_amdgcn_s_sleep(4);
+    backoff_sleep(level);
     if (clk.expired()) return false;
   }
 }
@@ -111,12 +129,16 @@ __device__ __forceinline__ void wait_signal(const uint32_t* addr, uint64_t limit
 }
 
 // Blockwise barrier across the (emulated) ranks for one block index.
-//   lane r < world_size:  send on pad[r][block*ws + rank], then consume
-//   pad[rank][block*ws + r].  Pads are all-zero again afterwards.
+//   lane r < ws:         send: CAS 0 -> 1 on pad[r][block*ws + rank]
+//   lane ws + r < 2*ws:  wait: CAS 1 -> 0 on pad[rank][block*ws + r]
+// The two halves are independent memory operations, so they run on different
+// lanes of the same wave and a round costs one atomic round trip, not two.  Pads
+// are all-zero again afterwards.
 // Writes made by this workgroup before the call are published to the peers
 // (every wave releases before the workgroup barrier that precedes the sends);
 // after the call every thread has acquired the peers' earlier writes.
-// Returns false (to every thread of the workgroup alike) when a spin timed out.
+// Needs at least 2*ws threads.  Returns false (to every thread of the workgroup
+// alike) when a spin timed out.
 __device__ __forceinline__ bool blockwise_barrier(const uint64_t* signal_pad_ptrs,
                                                   uint32_t block_id, int rank, int world_size,
                                                   uint64_t limit_ticks, uint32_t* status) {
@@ -124,16 +146,13 @@ __device__ __forceinline__ bool blockwise_barrier(const uint64_t* signal_pad_ptr
   __syncthreads();
   const int lane = threadIdx.x;
   int bad = 0;
-  if (lane < world_size) {
-    uint32_t* remote = reinterpret_cast<uint32_t*>(signal_pad_ptrs[lane]);
-    uint32_t* local = reinterpret_cast<uint32_t*>(signal_pad_ptrs[rank]);
-    uint32_t* send = remote + (size_t)block_id * world_size + rank;
-    uint32_t* wait = local + (size_t)block_id * world_size + lane;
-    if (!send_signal(send, limit_ticks)) {
-      report(status, SMR_ST_SEND_TIMEOUT, rank, block_id, lane);
-      bad = 1;
-    } else if (!wait_signal_reset(wait, limit_ticks)) {
-      report(status, SMR_ST_WAIT_TIMEOUT, rank, block_id, lane);
+  if (lane < 2 * world_size) {
+    const bool is_send = lane < world_size;
+    const int peer = is_send ? lane : lane - world_size;
+    uint32_t* pad = reinterpret_cast<uint32_t*>(signal_pad_ptrs[is_send ? peer : rank]);
+    uint32_t* slot = pad + (size_t)block_id * world_size + (is_send ? rank : peer);
+    if (!spin_cas(slot, is_send ? 0u : 1u, is_send ? 1u : 0u, limit_ticks)) {
+      report(status, is_send ? SMR_ST_SEND_TIMEOUT : SMR_ST_WAIT_TIMEOUT, rank, block_id, peer);
       bad = 1;
     }
   }

@@ -36,6 +36,7 @@ SIGNATURES = {
     "smr_get_spin_timeout_us": (_i64, []),
     "smr_one_shot_all_reduce": (_i, [_p, _p, _p, _i64, _i, _i, _i, _i, _i, _p, _p]),
     "smr_reduce_num_blocks": (_i, [_i64, _i]),
+    "smr_set_reduce_launch": (_i, [_i, _i]),
     "smr_barrier": (_i, [_p, _i, _i, _i, _i, _p, _p]),
     "smr_send_signal": (_i, [_p, _p, _p]),
     "smr_wait_signal": (_i, [_p, _p, _p]),
@@ -44,7 +45,8 @@ SIGNATURES = {
     "smr_signal_round": (_i, [_p, _p, _p, _p, _p, _p, _i, _i, _i64, _i, _p, _p]),
     "smr_all_gather_with_progress": (_i, [_p, _p, _p, _p, _i, _i, _i64, _i, _i, _p]),
     "smr_ag_matmul": (_i, [_p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _p, _p]),
-    "smr_ag_matmul_schedule": (_i, [_i, _i, _i, _i, _i, _i, _p, _i]),
+    "smr_ag_matmul_schedule": (_i, [_i, _i, _i, _i, _i, _i, _i, _p, _i]),
+    "smr_ag_matmul_grid": (_i, [_i, _i, _i, _i, _i, _i]),
     "smr_gemv_allreduce": (_i, [_p, _p, _p, _p, _p, _i, _i, _i, _i, _p, _p]),
     "smr_gemv_flag_blocks": (_i, [_i]),
 }

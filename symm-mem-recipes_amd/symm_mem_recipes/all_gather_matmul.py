@@ -1,0 +1,146 @@
+"""All-gather matmul: a producer that gathers the peers' A shards and raises one
+progress flag per chunk, overlapped with a bf16 GEMM that walks the shards in
+their ready order and waits on those flags.
+
+Drop-ins for the reference's host entry points
+(symm_mem_recipes/triton_all_gather_matmul.py): ``all_gather_with_progress``
+(:20-56), ``all_gather_matmul_tma_persistent`` (:219-319; the name is kept although
+nothing here is TMA - the kernel is an LDS-staged MFMA GEMM) and the torch
+comparator ``all_gather_matmul`` (:322-326).
+"""
+from __future__ import annotations
+
+import os
+from typing import Optional
+
+import torch
+
+from . import _lib
+from .symm_mem import EmulatedSymmetricMemory, _get_backend_stream
+
+
+def all_gather_with_progress(output: torch.Tensor, inp: torch.Tensor, progress: torch.Tensor,
+                             splits_per_rank: int, num_workgroups: int = 0) -> None:
+    """Copy every rank's shard into ``output`` (sources in the order rank+1, ...,
+    rank+world_size-1, rank) and set ``progress[src*splits_per_rank + split]`` to 1
+    after each chunk, on the current stream."""
+    assert inp.is_contiguous()
+
+    symm_mem = EmulatedSymmetricMemory.rendezvous(inp)
+    assert symm_mem is not None
+
+    rank = symm_mem.rank
+    world_size = symm_mem.world_size
+
+    assert inp.numel() % splits_per_rank == 0
+    assert progress.numel() == world_size * splits_per_rank
+    assert progress.element_size() == 4 and progress.is_contiguous()
+
+    output_shape = list(inp.shape)
+    output_shape[0] *= world_size
+    assert list(output.shape) == output_shape, (list(output.shape), output_shape)
+    assert output.is_contiguous() and output.dtype == inp.dtype
+
+    counters = torch.zeros(world_size * splits_per_rank, dtype=torch.int32, device=inp.device)
+    lib = _lib.load()
+    rc = lib.smr_all_gather_with_progress(
+        symm_mem.buffer_ptrs_dev, output.data_ptr(), progress.data_ptr(), counters.data_ptr(),
+        rank, world_size, inp.numel() * inp.element_size(), int(splits_per_rank),
+        int(num_workgroups), torch.cuda.current_stream(inp.device).cuda_stream)
+    _lib.check(rc, "all_gather_with_progress")
+    symm_mem.barrier()
+
+
+def all_gather_matmul_tma_persistent(a_shard: torch.Tensor, b: torch.Tensor, a_out: torch.Tensor,
+                                     c_out: torch.Tensor, configs: Optional[dict] = None,
+                                     mm_only: bool = False, *, splits_per_rank: int = 1) -> torch.Tensor:
+    """``c_out = cat(all ranks' a_shard) @ b.T`` with ``b`` of shape [N, K]
+    (K-contiguous).  ``mm_only`` skips the gather and the flags and multiplies
+    what ``a_shard`` (rank 0's rows) and ``a_out`` already hold: the ungated
+    comparator.  ``configs`` is accepted for compatibility; the tile shape is the
+    library's choice."""
+    if mm_only:
+        symm_mem = None
+        rank = 0
+        world_size = int(os.environ.get("WORLD_SIZE", "8"))
+    else:
+        symm_mem = EmulatedSymmetricMemory.rendezvous(a_shard)
+        assert symm_mem is not None, "a_shard must be allocated via SymmetricMemory"
+        rank = symm_mem.rank
+        world_size = symm_mem.world_size
+
+    assert a_shard.dtype == torch.bfloat16 and b.dtype == torch.bfloat16, "Only bfloat16 is supported for now."
+    M = a_shard.shape[0] * world_size
+    N = b.shape[0]
+    K = a_shard.shape[1]
+
+    assert b.shape[1] == K
+    assert a_out.shape[0] == M
+    assert a_out.shape[1] == K
+    assert c_out.shape[0] == M
+    assert c_out.shape[1] == N
+    assert a_shard.is_contiguous() and b.is_contiguous() and a_out.is_contiguous() and c_out.is_contiguous()
+
+    COMM_BLOCK_SIZE_M = M // world_size // splits_per_rank
+    if configs is not None and "BLOCK_SIZE_M" in configs:
+        assert COMM_BLOCK_SIZE_M % (configs["BLOCK_SIZE_M"] * configs.get("GROUP_SIZE_M", 1)) == 0
+
+    lib = _lib.load()
+    device = a_shard.device
+    current = torch.cuda.current_stream(device)
+    status_ptr = symm_mem.status.data_ptr() if symm_mem is not None else 0
+    if mm_only:
+        progress_ptr = 0
+    else:
+        progress = torch.zeros(world_size * splits_per_rank, dtype=torch.int32, device=device)
+        progress_ptr = progress.data_ptr()
+        symm_mem.barrier(0)
+        backend = _get_backend_stream()
+        backend.wait_stream(current)
+        progress.record_stream(backend)
+        # the producer takes the compute units the GEMM's grid leaves free
+        grid = lib.smr_ag_matmul_grid(M, N, K, world_size, COMM_BLOCK_SIZE_M, 1)
+        if grid < 0:
+            _lib.check(grid, "all_gather_matmul")
+        cus = torch.cuda.get_device_properties(device).multi_processor_count
+        producer_wgs = max(8, min(32, cus - grid))
+        with torch.cuda.stream(backend):
+            all_gather_with_progress(a_out, a_shard, progress, splits_per_rank, producer_wgs)
+
+    rc = lib.smr_ag_matmul(a_shard.data_ptr(), a_out.data_ptr(), b.data_ptr(), c_out.data_ptr(),
+                           progress_ptr, M, N, K, rank, world_size, COMM_BLOCK_SIZE_M, status_ptr,
+                           current.cuda_stream)
+    _lib.check(rc, "all_gather_matmul")
+    if not mm_only:
+        current.wait_stream(backend)
+    return c_out
+
+
+#: the same entry point under a name that says what it is
+all_gather_matmul_fused = all_gather_matmul_tma_persistent
+
+
+def all_gather_matmul(a_shard: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
+    """The unfused comparator: gather the shards, then one library matmul
+    (triton_all_gather_matmul.py:322-326; ``b`` is [K, N] here, as there)."""
+    symm_mem = EmulatedSymmetricMemory.rendezvous(a_shard)
+    assert symm_mem is not None, "a_shard must be allocated via SymmetricMemory"
+    a = torch.cat([symm_mem.get_buffer(r, a_shard.shape, a_shard.dtype)
+                   for r in range(symm_mem.world_size)], dim=0)
+    return torch.matmul(a, b)
+
+
+def gemm_schedule(M: int, N: int, K: int, rank: int, world_size: int, comm_block_m: int,
+                  gated: bool = True):
+    """The tile order the GEMM uses on a 256-CU part, as a list of dicts in each
+    workgroup's visiting order (host-only; the counterpart of the index
+    arithmetic at triton_all_gather_matmul.py:125-174)."""
+    import ctypes
+    lib = _lib.load()
+    n = lib.smr_ag_matmul_schedule(M, N, K, rank, world_size, comm_block_m, int(gated), None, 0)
+    if n < 0:
+        _lib.check(n, "gemm_schedule")
+    buf = (ctypes.c_int32 * (8 * n))()
+    lib.smr_ag_matmul_schedule(M, N, K, rank, world_size, comm_block_m, int(gated), buf, n)
+    keys = ("wg", "step", "row0", "col0", "rows", "cols", "comm_block", "local")
+    return [dict(zip(keys, buf[8 * i:8 * i + 8])) for i in range(n)]

@@ -1,0 +1,87 @@
+"""Host-only properties of the GEMM's tile order (the library's counterpart of the
+index arithmetic at symm_mem_recipes/triton_all_gather_matmul.py:125-174): every
+output tile exactly once, local comm block first, comm blocks in ring order, local
+tiles never wait, one XCD's tiles of a pass form a compact patch."""
+import collections
+
+import pytest
+
+from symm_mem_recipes import gemm_schedule
+
+
+def _by_wg(s):
+    by = collections.defaultdict(list)
+    for t in s:
+        by[t["wg"]].append(t)
+    return by
+
+
+@pytest.mark.parametrize("rank", [0, 3, 7])
+def test_schedule_config5(rank):
+    M, N, K, ws = 16384, 3584, 8192, 8
+    s = gemm_schedule(M, N, K, rank, ws, M // ws)
+    assert len(s) == 64 * 14
+    assert {(t["rows"], t["cols"]) for t in s} == {(256, 256)}
+    assert len({(t["row0"], t["col0"]) for t in s}) == len(s)              # bijection
+    assert {t["row0"] for t in s} == set(range(0, M, 256))
+    assert {t["col0"] for t in s} == set(range(0, N, 256))
+    for t in s:
+        assert t["comm_block"] == t["row0"] // 2048
+        assert t["local"] == int(t["comm_block"] == rank)                  # only local tiles skip the wait
+    by = _by_wg(s)
+    # 896 tiles finish in 4 passes on 224 workgroups as on 256: the balanced grid
+    # leaves 32 compute units to the producer at no cost
+    assert len(by) == 224 and all(len(v) == 4 for v in by.values())
+    for wg, tiles in by.items():
+        assert [t["step"] for t in tiles] == list(range(len(tiles)))
+        ring = [(t["comm_block"] - rank) % ws for t in tiles]
+        assert ring == sorted(ring)                                        # ready order of the gather
+    # the whole local comm block is scheduled in the first pass
+    first = [t for t in s if t["step"] == 0]
+    assert sum(t["local"] for t in first) == 8 * 14
+    # XCD locality: the 32 tiles an XCD holds in the first pass share few A/B slabs
+    for x in range(8):
+        mine = [t for t in first if t["wg"] % 8 == x]
+        assert len(mine) == 28
+        slabs = len({t["row0"] for t in mine}) + len({t["col0"] for t in mine})
+        assert slabs <= 20                                                 # 56 when unrelated
+
+
+@pytest.mark.parametrize("M,N,K,ws,splits", [(1024, 256, 256, 8, 1), (2048, 384, 512, 8, 1),
+                                             (2048, 264, 128, 4, 2), (512, 128, 64, 2, 2),
+                                             (4096, 1792, 4096, 8, 1)])
+def test_schedule_other_shapes(M, N, K, ws, splits):
+    comm = M // ws // splits
+    for rank in range(ws):
+        s = gemm_schedule(M, N, K, rank, ws, comm)
+        bm, bn = s[0]["rows"], s[0]["cols"]
+        assert comm % bm == 0
+        want = {(r, c) for r in range(0, M, bm) for c in range(0, N, bn)}
+        assert {(t["row0"], t["col0"]) for t in s} == want and len(s) == len(want)
+        for t in s:
+            owner = t["comm_block"] // splits
+            assert t["local"] == int(owner == rank)
+        for tiles in _by_wg(s).values():
+            first_local = rank * splits
+            ring = [(t["comm_block"] - first_local) % (ws * splits) for t in tiles]
+            assert ring == sorted(ring)
+
+
+def test_grid_leaves_room_for_the_producer(lib):
+    # gated launches never take every compute unit (256 assumed without a GPU)
+    for (M, N, K) in [(16384, 3584, 8192), (16384, 6656, 16384), (4096, 1792, 4096), (32768, 8192, 1024)]:
+        gated = lib.smr_ag_matmul_grid(M, N, K, 8, M // 8, 1)
+        ungated = lib.smr_ag_matmul_grid(M, N, K, 8, M // 8, 0)
+        assert 8 <= gated <= 248 and gated % 8 == 0
+        assert gated <= ungated <= 256
+
+
+def test_schedule_rejects_bad_shapes():
+    with pytest.raises(AssertionError):
+        gemm_schedule(1000, 256, 256, 0, 8, 125)        # rows per flag not a multiple of 128
+    with pytest.raises(AssertionError):
+        gemm_schedule(1024, 256, 100, 0, 8, 128)        # K not a multiple of 64
+    with pytest.raises(AssertionError):
+        gemm_schedule(1024, 252, 256, 0, 8, 128)        # N not a multiple of 8
+    with pytest.raises(AssertionError):
+        gemm_schedule(1024, 256, 256, 8, 8, 128)        # rank out of range
