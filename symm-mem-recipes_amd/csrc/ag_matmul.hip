@@ -97,8 +97,18 @@ __device__ __forceinline__ bf16x8 lds_read_frag(uint32_t addr) {
 // One wave instruction of a direct-to-LDS tile load: 64 lanes x 16 B land at
 // lds_dst + lane*16 (one 8-row group, 1 KiB); `voff` is the lane's byte offset
 // from the uniform global base.
+//
+// Issued through inline assembly so that the compiler does not count these loads:
+// it cannot tell which LDS bytes they write, so it would make every later
+// fragment read wait for all of them - and for the L2 warm-up loads issued
+// behind them.  All waits on these loads are explicit s_waitcnt vmcnt in the
+// kernel (loads return in order, so "vmcnt(n)" leaves the n youngest in flight).
 __device__ __forceinline__ void load_group(const uint8_t* base, uint32_t voff, uint32_t lds_dst) {
-  __builtin_amdgcn_global_load_lds((const GlobalVoid*)(base + voff), (LdsVoid*)(uintptr_t)lds_dst, 16, 0, 0);
+  // scalar base + 32-bit per-lane offset: no 64-bit address arithmetic per lane
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+               :
+               : "s"(lds_dst), "v"(voff), "s"(base)
+               : "memory", "m0");
 }
 
 // Scheduling hint: spread NDS LDS reads evenly under NMFMA matrix instructions.
@@ -124,13 +134,17 @@ struct GemmTile {
   static constexpr int kLdsBytes = 2 * (kABytes + kBBytes);
 };
 
+// How many stages ahead of its real load a K-slab is touched to pull it into L2.
+constexpr int kWarmAhead = 3;
+
 template <int BM, int BN>
 __global__ __launch_bounds__(kGemmThreads, 1) void ag_matmul_kernel(
     const uint8_t* __restrict__ a_shard, const uint8_t* __restrict__ a_out,
     const uint8_t* __restrict__ b_nk, uint8_t* __restrict__ c, const uint32_t* __restrict__ progress,
-    GemmSchedule s, uint64_t limit_ticks, uint32_t* status) {
+    GemmSchedule s, uint64_t limit_ticks, uint32_t* status, uint64_t* trace) {
   using T = GemmTile<BM, BN>;
   constexpr int WM = T::WM, WN = T::WN, FM = T::FM, FN = T::FN, GA = T::GA, GB = T::GB;
+  constexpr int kWarmLoads = GA / 8 + GB / 8;      // warm-up loads per wave and stage
   __shared__ __attribute__((aligned(1024))) uint8_t lds[T::kLdsBytes];
 
   const int lane = threadIdx.x & 63;
@@ -141,33 +155,52 @@ __global__ __launch_bounds__(kGemmThreads, 1) void ag_matmul_kernel(
   const int nk = s.K / kBK;
   const uint32_t lds0 = lds_offset_of(lds);
 
-  // ---- per-lane fragment read addresses (stage 0).  Row r = w*W + f*32 + (lane & 31)
-  // has swizzle ((lane & 7) ^ ((lane >> 3) & 3)) ^ ((f & 1) << 2); K step kk wants
-  // chunk 2*kk + half.  Hence position = t ^ (v << 1) with the per-lane constant
-  // t = half ^ (lane & 7) ^ ((lane >> 3) & 3) and v = kk ^ ((f & 1) << 1): four
-  // variants per operand, everything else is an immediate offset.
-  const int t = half ^ (lane & 7) ^ ((lane >> 3) & 3);
-  uint32_t a_fr[4], b_fr[4];
-#pragma unroll
-  for (int v = 0; v < 4; ++v) {
-    a_fr[v] = lds0 + (uint32_t)((wm * WM + (lane & 31)) * kRowBytes + ((t ^ (v << 1)) << 4));
-    b_fr[v] = lds0 + T::kBBase + (uint32_t)((wn * WN + (lane & 31)) * kRowBytes + ((t ^ (v << 1)) << 4));
-  }
-
-  // ---- per-lane global offsets of the tile loads.  Load group q = wave*G + j holds
-  // rows q*8 .. q*8+7; lane l carries row q*8 + (l >> 3) and the chunk whose swizzled
-  // position is (l & 7): chunk = (l & 7) ^ (l >> 3) ^ (q & 7).
-  const int u = (lane & 7) ^ (lane >> 3);
-  uint32_t a_off[GA];
-#pragma unroll
-  for (int j = 0; j < GA; ++j) {
-    const int q = wave * GA + j;
-    a_off[j] = (uint32_t)(q * 8 + (lane >> 3)) * row_stride + (uint32_t)((u ^ (q & 7)) << 4);
-  }
+  uint32_t warm_scrap = 0;
 
   for (int step = 0;; ++step) {
     TileRef tile;
     if (!tile_for(s, blockIdx.x, step, tile)) break;
+
+    // The per-lane addresses below are recomputed for every tile from a laundered
+    // copy of the lane id: kept loop-invariant they would stay live across the
+    // register-hungry epilogue, be spilled there, and be reloaded from scratch
+    // in the middle of the K loop.
+    int ln = lane;
+    asm volatile("" : "+v"(ln));
+    // ---- per-lane fragment read addresses (stage 0).  Row r = w*W + f*32 + (ln & 31)
+    // has swizzle ((lane & 7) ^ ((ln >> 3) & 3)) ^ ((f & 1) << 2); K step kk wants
+    // chunk 2*kk + half.  Hence position = t ^ (v << 1) with the per-lane constant
+    // t = half ^ (lane & 7) ^ ((ln >> 3) & 3) and v = kk ^ ((f & 1) << 1): four
+    // variants per operand, everything else is an immediate offset.
+    const int t = (ln >> 5) ^ (ln & 7) ^ ((ln >> 3) & 3);
+    uint32_t a_fr[4], b_fr[4];
+  #pragma unroll
+    for (int v = 0; v < 4; ++v) {
+      a_fr[v] = lds0 + (uint32_t)((wm * WM + (ln & 31)) * kRowBytes + ((t ^ (v << 1)) << 4));
+      b_fr[v] = lds0 + T::kBBase + (uint32_t)((wn * WN + (ln & 31)) * kRowBytes + ((t ^ (v << 1)) << 4));
+    }
+
+    // ---- per-lane global offsets of the tile loads.  Load group q = wave*G + j holds
+    // rows q*8 .. q*8+7; lane l carries row q*8 + (l >> 3) and the chunk whose swizzled
+    // position is (l & 7): chunk = (l & 7) ^ (l >> 3) ^ (q & 7).
+    const int u = (ln & 7) ^ (ln >> 3);
+    uint32_t a_off[GA];
+  #pragma unroll
+    for (int j = 0; j < GA; ++j) {
+      const int q = wave * GA + j;
+      a_off[j] = (uint32_t)(q * 8 + (ln >> 3)) * row_stride + (uint32_t)((u ^ (q & 7)) << 4);
+    }
+
+    // ---- L2 warm-up: one dword per 128-byte row segment, 64 rows per wave instruction
+    uint32_t a_warm[GA / 8 > 0 ? GA / 8 : 1];
+  #pragma unroll
+    for (int j = 0; j < GA / 8; ++j) a_warm[j] = (uint32_t)(wave * (GA * 8) + j * 64 + ln) * row_stride;
+
+    uint64_t* tr = nullptr;
+    if (trace != nullptr && step < kTraceSteps && blockIdx.x < 256 && threadIdx.x == 0) {
+      tr = trace + kTraceProducerWords + ((size_t)blockIdx.x * kTraceSteps + step) * 4;
+      tr[0] = wall_clock64();
+    }
     const uint8_t* a_base;
     if (tile.local) {
       a_base = a_shard + (int64_t)tile.a_row * row_stride;
@@ -176,6 +209,7 @@ __global__ __launch_bounds__(kGemmThreads, 1) void ag_matmul_kernel(
         wait_signal(progress + tile.comm_block, limit_ticks, status, tile.comm_block);
       a_base = a_out + (int64_t)tile.a_row * row_stride;
     }
+    if (tr != nullptr) tr[1] = wall_clock64();
     const uint8_t* b_base = b_nk + (int64_t)tile.col0 * row_stride;
     // rows of B past the last column are clamped: they feed outputs that are never stored
     const int b_last = s.N - 1 - tile.col0;
@@ -183,9 +217,17 @@ __global__ __launch_bounds__(kGemmThreads, 1) void ag_matmul_kernel(
 #pragma unroll
     for (int j = 0; j < GB; ++j) {
       const int q = wave * GB + j;
-      int r = q * 8 + (lane >> 3);
+      int r = q * 8 + (ln >> 3);
       r = r < b_last ? r : b_last;
       b_off[j] = (uint32_t)r * row_stride + (uint32_t)((u ^ (q & 7)) << 4);
+    }
+
+    uint32_t b_warm[GB / 8 > 0 ? GB / 8 : 1];
+#pragma unroll
+    for (int j = 0; j < GB / 8; ++j) {
+      int r = wave * (GB * 8) + j * 64 + ln;
+      r = r < b_last ? r : b_last;
+      b_warm[j] = (uint32_t)r * row_stride;
     }
 
     f32x16 acc[FN][FM];
@@ -205,6 +247,23 @@ __global__ __launch_bounds__(kGemmThreads, 1) void ag_matmul_kernel(
       for (int j = 0; j < GA; ++j) load_group(ak, a_off[j], la + j * 1024);
 #pragma unroll
       for (int j = 0; j < GB; ++j) load_group(bk, b_off[j], lb + j * 1024);
+    };
+    // Touch the K-slab of stage kt (one dword per row) so that its real load,
+    // kWarmAhead stages later, finds the lines in L2.  The loaded dwords go to a
+    // scrap register that is never read for its value.  Inline assembly on
+    // purpose: the compiler must not count these loads, or it would make the wave
+    // wait for them - they are meant to miss - before the next fragment reads.
+    // `warm_scrap` is threaded through every statement and consumed after the
+    // tile loop, so its register stays reserved while loads into it are in flight.
+    auto warm_stage = [&](int kt) {
+      const uint8_t* ak = a_base + (int64_t)kt * kRowBytes;
+      const uint8_t* bk = b_base + (int64_t)kt * kRowBytes;
+#pragma unroll
+      for (int j = 0; j < GA / 8; ++j)
+        asm volatile("global_load_dword %0, %1, %2" : "+v"(warm_scrap) : "v"(a_warm[j]), "s"(ak) : "memory");
+#pragma unroll
+      for (int j = 0; j < GB / 8; ++j)
+        asm volatile("global_load_dword %0, %1, %2" : "+v"(warm_scrap) : "v"(b_warm[j]), "s"(bk) : "memory");
     };
     auto read_frags = [&](bf16x8 (&af)[FM], bf16x8 (&bf)[FN], int stage, int kk) {
 #pragma unroll
@@ -227,6 +286,9 @@ __global__ __launch_bounds__(kGemmThreads, 1) void ag_matmul_kernel(
     if (nk > 1) load_stage(1, 1);
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
+#pragma unroll
+    for (int w = 0; w < kWarmAhead; ++w)
+      if (2 + w < nk) warm_stage(2 + w);
 
     // Fragment double buffer: while the MFMAs of K step kk run, the fragments of
     // step kk+1 are read.  The workgroup barrier sits before the last K step of a
@@ -250,9 +312,17 @@ __global__ __launch_bounds__(kGemmThreads, 1) void ag_matmul_kernel(
       interleave_mfma_dsread<FM * FN, FM + FN>();
       // The compiler does not track direct-to-LDS loads across the loop back
       // edge: wait for this wave's own loads explicitly before the barrier.
-      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      // The warm-up loads issued after them (if any were) may stay in flight:
+      // loads return in order.
+      if (kWarmLoads > 0 && (kt == 0 || kt + 1 + kWarmAhead < nk)) {
+        if constexpr (kWarmLoads == 1) asm volatile("s_waitcnt vmcnt(1)" ::: "memory");
+        else asm volatile("s_waitcnt vmcnt(2)" ::: "memory");
+      } else {
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      }
       __syncthreads();     // stage S fully read by everyone; the other stage has landed
       if (kt + 2 < nk) load_stage(S, kt + 2);
+      if (kt + 2 + kWarmAhead < nk) warm_stage(kt + 2 + kWarmAhead);
       if (kt + 1 < nk) read_frags(af0, bf0, S ^ 1, 0);
       mfma_all(af1, bf1);
     };
@@ -263,6 +333,7 @@ __global__ __launch_bounds__(kGemmThreads, 1) void ag_matmul_kernel(
     }
     if (kt < nk) stage_body(std::integral_constant<int, 0>{}, kt);
     __syncthreads();       // the next tile's prologue overwrites both stages
+    if (tr != nullptr) tr[2] = wall_clock64();
 
     // D[n][m]: lane holds row m = lane & 31 and, per group of 4 registers, the 4
     // consecutive columns g*8 + (lane >> 5)*4 .. +3 of the 32x32 fragment.
@@ -282,9 +353,17 @@ __global__ __launch_bounds__(kGemmThreads, 1) void ag_matmul_kernel(
             *reinterpret_cast<uint2*>(c_row + (int64_t)n * 2) = v;
           }
         }
+        // one fragment at a time: keeps the accumulator read-out from flooding
+        // the vector registers
+        __builtin_amdgcn_sched_barrier(0);
       }
     }
+    if (tr != nullptr) tr[3] = wall_clock64();
   }
+  // Drain the warm-up loads and give the scrap register a use the compiler
+  // cannot remove (K is never negative).
+  asm volatile("s_waitcnt vmcnt(0)" : "+v"(warm_scrap) : : "memory");
+  if (s.K < 0) status[3] = warm_scrap;
 }
 
 static int pick_tile(int M, int N, int comm_block_m, int& BM, int& BN) {
@@ -377,15 +456,16 @@ int smr_ag_matmul(const void* a_shard_dev, const void* a_out_dev, const void* b_
   const uint8_t* b = reinterpret_cast<const uint8_t*>(b_nk_dev);
   uint8_t* c = reinterpret_cast<uint8_t*>(c_dev);
   const uint64_t lim = spin_limit_ticks();
+  uint64_t* tb = trace_buffer(kTraceProducerWords + kTraceGemmWords);
   if (s.BM == 256 && s.BN == 256)
     hipLaunchKernelGGL((ag_matmul_kernel<256, 256>), dim3(s.grid), dim3(kGemmThreads), 0, st, a0, a1, b,
-                       c, progress_dev, s, lim, status);
+                       c, progress_dev, s, lim, status, tb);
   else if (s.BM == 256)
     hipLaunchKernelGGL((ag_matmul_kernel<256, 128>), dim3(s.grid), dim3(kGemmThreads), 0, st, a0, a1, b,
-                       c, progress_dev, s, lim, status);
+                       c, progress_dev, s, lim, status, tb);
   else
     hipLaunchKernelGGL((ag_matmul_kernel<128, 128>), dim3(s.grid), dim3(kGemmThreads), 0, st, a0, a1, b,
-                       c, progress_dev, s, lim, status);
+                       c, progress_dev, s, lim, status, tb);
   return check_hip(hipGetLastError(), "smr_ag_matmul launch");
 }
 

@@ -28,8 +28,9 @@ typedef __attribute__((address_space(1))) u32x4 GlobalVec;
 __global__ __launch_bounds__(kGatherThreads) void all_gather_kernel(
     const uint64_t* __restrict__ buffer_ptrs, uint8_t* __restrict__ a_out,
     uint32_t* __restrict__ progress, uint32_t* __restrict__ counters, int rank, int world_size,
-    int64_t chunk_vecs, int splits_per_rank) {
+    int64_t chunk_vecs, int splits_per_rank, uint64_t* trace) {
   const int nwg = gridDim.x;
+  if (trace != nullptr && blockIdx.x == 0 && threadIdx.x == 0) trace[kTraceProducerWords - 1] = wall_clock64();
   for (int step = 0; step < world_size; ++step) {
     const int src_rank = (rank + step + 1) % world_size;
     for (int split = 0; split < splits_per_rank; ++split) {
@@ -37,18 +38,16 @@ __global__ __launch_bounds__(kGatherThreads) void all_gather_kernel(
       const GlobalVec* src =
           (const GlobalVec*)(uintptr_t)buffer_ptrs[src_rank] + (int64_t)split * chunk_vecs;
       GlobalVec* dst = (GlobalVec*)(uintptr_t)a_out + (int64_t)idx * chunk_vecs;
-      // 4 independent 16-byte slots per thread per trip
+      // 8 independent 16-byte slots per thread per trip: 128 KiB in flight per
+      // workgroup, which is what one compute unit needs to stream at its share
       const int64_t stride = (int64_t)nwg * kGatherThreads;
       int64_t i = (int64_t)blockIdx.x * kGatherThreads + threadIdx.x;
-      for (; i + 3 * stride < chunk_vecs; i += 4 * stride) {
-        u32x4 v0 = __builtin_nontemporal_load(src + i);
-        u32x4 v1 = __builtin_nontemporal_load(src + i + stride);
-        u32x4 v2 = __builtin_nontemporal_load(src + i + 2 * stride);
-        u32x4 v3 = __builtin_nontemporal_load(src + i + 3 * stride);
-        __builtin_nontemporal_store(v0, dst + i);
-        __builtin_nontemporal_store(v1, dst + i + stride);
-        __builtin_nontemporal_store(v2, dst + i + 2 * stride);
-        __builtin_nontemporal_store(v3, dst + i + 3 * stride);
+      for (; i + 7 * stride < chunk_vecs; i += 8 * stride) {
+        u32x4 v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) v[u] = __builtin_nontemporal_load(src + i + u * stride);
+#pragma unroll
+        for (int u = 0; u < 8; ++u) __builtin_nontemporal_store(v[u], dst + i + u * stride);
       }
       for (; i < chunk_vecs; i += stride) {
         u32x4 v = __builtin_nontemporal_load(src + i);
@@ -64,6 +63,7 @@ __global__ __launch_bounds__(kGatherThreads) void all_gather_kernel(
         if (prev + 1u == (uint32_t)nwg) {
           __hip_atomic_store(&counters[idx], 0u, __ATOMIC_RELAXED, kScope);
           __hip_atomic_store(&progress[idx], 1u, __ATOMIC_RELEASE, kScope);
+          if (trace != nullptr && idx < kTraceProducerWords - 1) trace[idx] = wall_clock64();
         }
       }
     }
@@ -93,6 +93,6 @@ extern "C" int smr_all_gather_with_progress(const uint64_t* buffer_ptrs_dev, voi
   hipLaunchKernelGGL(all_gather_kernel, dim3(nwg), dim3(kGatherThreads), 0,
                      reinterpret_cast<hipStream_t>(stream), buffer_ptrs_dev,
                      reinterpret_cast<uint8_t*>(a_out_dev), progress_dev, counters_dev, rank,
-                     world_size, chunk_bytes / 16, splits_per_rank);
+                     world_size, chunk_bytes / 16, splits_per_rank, trace_buffer(kTraceProducerWords));
   return check_hip(hipGetLastError(), "smr_all_gather_with_progress launch");
 }

@@ -115,7 +115,8 @@ __global__ __launch_bounds__(kReduceMaxThreads) void one_shot_all_reduce_kernel(
     out += (size_t)rank * nvec;
   }
 
-  if (do_barrier) blockwise_barrier(signal_pad_ptrs, block, rank, WS, limit_ticks, status);
+  // the peers' buffers were written by earlier kernels: nothing of this kernel to publish
+  if (do_barrier) blockwise_barrier(signal_pad_ptrs, block, rank, WS, limit_ticks, status, false);
 
   GlobalVec* src[WS];
 #pragma unroll

@@ -15,6 +15,15 @@ void set_last_error(const char* msg);
 int fail(int code, const char* msg);            // records msg, returns code
 int check_hip(hipError_t e, const char* what);  // 0 or the hip error (recorded)
 uint64_t spin_limit_ticks();                    // current timeout in wall_clock64 ticks (0 = none)
+uint64_t* trace_buffer(int64_t min_words);      // the registered trace buffer if it is large enough
+
+// Layout of the optional trace buffer (uint64 words of the 100 MHz device clock):
+//   [0 .. 63]                       producer: word i = time flag i was raised, word 63 = start
+//   [64 + (wg*kTraceSteps + step)*4 + k]   GEMM workgroup wg, its step-th tile:
+//        k = 0 tile picked, 1 flag wait over, 2 K loop done, 3 tile stored
+constexpr int kTraceProducerWords = 64;
+constexpr int kTraceSteps = 16;
+constexpr int kTraceGemmWords = 256 * kTraceSteps * 4;
 
 // ---------------------------------------------------------------- bf16
 __device__ __forceinline__ float bf16_lo(uint32_t w) { return __uint_as_float(w << 16); }
@@ -92,6 +101,27 @@ __device__ __forceinline__ bool spin_cas(uint32_t* addr, uint32_t from, uint32_t
   }
 }
 
+// Wait-side variant: poll with plain atomic loads and attempt the CAS only once
+// the flag shows `from`, so that a waiting lane sends loads, not read-modify-write
+// traffic, to memory.  (The transition itself must stay a read-modify-write: a
+// plain store by the polling side would leave the line in its own L2, where its
+// later polls would keep hitting the stale copy.)
+__device__ __forceinline__ bool poll_then_cas(uint32_t* addr, uint32_t from, uint32_t to,
+                                              uint64_t limit_ticks) {
+  SpinClock clk(limit_ticks);
+  uint32_t level = 0;
+  for (;;) {
+    if (__hip_atomic_load(addr, __ATOMIC_RELAXED, kScope) == from) {
+      uint32_t expected = from;
+      if (__hip_atomic_compare_exchange_strong(addr, &expected, to, __ATOMIC_RELAXED,
+                                               __ATOMIC_RELAXED, kScope))
+        return true;
+    }
+    backoff_sleep(level);
+    if (clk.expired()) return false;
+  }
+}
+
 // Release-CAS 0 -> 1 until it succeeds: publishes everything the calling
 // thread (and, through a preceding workgroup barrier, its workgroup) wrote.
 __device__ __forceinline__ bool send_signal(uint32_t* addr, uint64_t limit_ticks) {
@@ -102,7 +132,7 @@ __device__ __forceinline__ bool send_signal(uint32_t* addr, uint64_t limit_ticks
 // CAS 1 -> 0 until it succeeds (consumes and resets the flag).  Relaxed: the
 // caller acquires afterwards, once, for the whole workgroup.
 __device__ __forceinline__ bool wait_signal_reset(uint32_t* addr, uint64_t limit_ticks) {
-  return spin_cas(addr, 1u, 0u, limit_ticks);
+  return poll_then_cas(addr, 1u, 0u, limit_ticks);
 }
 
 // Spin (one thread) until *addr == 1; the flag is left set.
@@ -134,30 +164,56 @@ __device__ __forceinline__ void wait_signal(const uint32_t* addr, uint64_t limit
 // The two halves are independent memory operations, so they run on different
 // lanes of the same wave and a round costs one atomic round trip, not two.  Pads
 // are all-zero again afterwards.
-// Writes made by this workgroup before the call are published to the peers
-// (every wave releases before the workgroup barrier that precedes the sends);
-// after the call every thread has acquired the peers' earlier writes.
+//
+// Only the first wave touches memory-ordering machinery: the workgroup barrier in
+// front collects every wave's earlier stores, then that one wave releases (when
+// `publish` is set: the workgroup wrote data inside this kernel that the peers
+// will read), flips the flags and acquires; the closing workgroup barrier hands
+// the acquired view to the other waves, which share its L1 and L2.  A cache
+// write-back and an invalidate per wave would otherwise dominate the round.
+// After the call every thread sees what the peers wrote before their call.
 // Needs at least 2*ws threads.  Returns false (to every thread of the workgroup
 // alike) when a spin timed out.
 __device__ __forceinline__ bool blockwise_barrier(const uint64_t* signal_pad_ptrs,
                                                   uint32_t block_id, int rank, int world_size,
-                                                  uint64_t limit_ticks, uint32_t* status) {
-  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+                                                  uint64_t limit_ticks, uint32_t* status,
+                                                  bool publish = true) {
   __syncthreads();
   const int lane = threadIdx.x;
   int bad = 0;
-  if (lane < 2 * world_size) {
-    const bool is_send = lane < world_size;
-    const int peer = is_send ? lane : lane - world_size;
-    uint32_t* pad = reinterpret_cast<uint32_t*>(signal_pad_ptrs[is_send ? peer : rank]);
-    uint32_t* slot = pad + (size_t)block_id * world_size + (is_send ? rank : peer);
-    if (!spin_cas(slot, is_send ? 0u : 1u, is_send ? 1u : 0u, limit_ticks)) {
-      report(status, is_send ? SMR_ST_SEND_TIMEOUT : SMR_ST_WAIT_TIMEOUT, rank, block_id, peer);
-      bad = 1;
+  if (lane < 64) {
+    if (publish) __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+    if (lane < 2 * world_size) {
+      const bool is_send = lane < world_size;
+      const int peer = is_send ? lane : lane - world_size;
+      uint32_t* pad = reinterpret_cast<uint32_t*>(signal_pad_ptrs[is_send ? peer : rank]);
+      uint32_t* slot = pad + (size_t)block_id * world_size + (is_send ? rank : peer);
+      // One loop for both kinds of lane: the wait lane of the rank's own slot
+      // depends on the send lane next to it, so neither may spin in a loop of its
+      // own while the other is masked off.  Wait lanes poll with a plain load and
+      // attempt the CAS only when the flag is up.
+      const uint32_t from = is_send ? 0u : 1u, to = is_send ? 1u : 0u;
+      SpinClock clk(limit_ticks);
+      uint32_t level = 0;
+      bool ok = false;
+      for (;;) {
+        if (is_send || __hip_atomic_load(slot, __ATOMIC_RELAXED, kScope) == from) {
+          uint32_t expected = from;
+          ok = __hip_atomic_compare_exchange_strong(slot, &expected, to, __ATOMIC_RELAXED,
+                                                    __ATOMIC_RELAXED, kScope);
+        }
+        if (ok) break;
+        backoff_sleep(level);
+        if (clk.expired()) break;
+      }
+      if (!ok) {
+        report(status, is_send ? SMR_ST_SEND_TIMEOUT : SMR_ST_WAIT_TIMEOUT, rank, block_id, peer);
+        bad = 1;
+      }
     }
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
   }
   bad = __syncthreads_or(bad);
-  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
   return bad == 0;
 }
 

@@ -30,6 +30,14 @@ int check_hip(hipError_t e, const char* what) {
   return (int)e;
 }
 
+static std::atomic<uint64_t*> g_trace{nullptr};
+static std::atomic<int64_t> g_trace_words{0};
+
+uint64_t* trace_buffer(int64_t min_words) {
+  uint64_t* p = g_trace.load(std::memory_order_relaxed);
+  return (p != nullptr && g_trace_words.load(std::memory_order_relaxed) >= min_words) ? p : nullptr;
+}
+
 uint64_t spin_limit_ticks() {
   int64_t us = g_spin_timeout_us.load(std::memory_order_relaxed);
   return us <= 0 ? 0 : (uint64_t)us * kTicksPerUs;
@@ -46,6 +54,14 @@ const char* smr_last_error_string(void) { return smr::g_err; }
 int smr_set_spin_timeout_us(int64_t us) {
   if (us < 0) return smr::fail(SMR_E_INVALID, "smr_set_spin_timeout_us: negative timeout");
   smr::g_spin_timeout_us.store(us, std::memory_order_relaxed);
+  return 0;
+}
+
+int smr_set_trace_buffer(uint64_t* trace_dev, int64_t words) {
+  if (words < 0 || (trace_dev == nullptr) != (words == 0))
+    return smr::fail(SMR_E_INVALID, "smr_set_trace_buffer: pointer and size must both be set or both be zero");
+  smr::g_trace.store(trace_dev, std::memory_order_relaxed);
+  smr::g_trace_words.store(words, std::memory_order_relaxed);
   return 0;
 }
 

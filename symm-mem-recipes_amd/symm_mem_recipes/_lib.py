@@ -34,6 +34,7 @@ SIGNATURES = {
     "smr_last_error_string": (C.c_char_p, []),
     "smr_set_spin_timeout_us": (_i, [_i64]),
     "smr_get_spin_timeout_us": (_i64, []),
+    "smr_set_trace_buffer": (_i, [_p, _i64]),
     "smr_one_shot_all_reduce": (_i, [_p, _p, _p, _i64, _i, _i, _i, _i, _i, _p, _p]),
     "smr_reduce_num_blocks": (_i, [_i64, _i]),
     "smr_set_reduce_launch": (_i, [_i, _i]),
