@@ -164,7 +164,7 @@ def bench_gemv(dev):
     res = []
     for batch in (1, 4, 8):
         xb = x[:batch].contiguous()
-        wsp = GemvWorkspace(batch, N, WS, dev)
+        wsp = GemvWorkspace(batch, N, WS, dev, K)
         out = torch.empty(batch, N, dtype=torch.bfloat16, device=dev)
         idx = [0]
 

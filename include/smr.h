@@ -183,15 +183,21 @@ int smr_ag_matmul_grid(int M, int N, int K, int world_size, int comm_block_m, in
 /* Split-K GEMV + rank-ordered combine through signal-pad flags.  No reference
  * code exists for it in symm_mem_recipes; it reuses the send/wait protocol of
  * triton_barrier.py:119-129 and triton_all_gather_matmul.py:72-95.
- *   x [batch,K] bf16, w [K,N] bf16 row-major, K split into ws shards;
- *   partials fp32 [ws, batch, N] scratch; flags uint32 [ws * flag_blocks] zero on
- *   entry and zero again on exit; out [batch,N] bf16 =
- *   bf16(((0 + p_0) + p_1) + ... + p_{ws-1}).  batch <= 8.
- *   smr_gemv_flag_blocks(N) gives flag_blocks. */
+ *   x [batch,K] bf16, w [K,N] bf16 row-major, K split into ws rank shards, each
+ *   cut further into sub-shards (one workgroup per column block and sub-shard);
+ *   S = smr_gemv_senders(N, K, ws) partial producers per column block.
+ *   partials fp32 [S, batch, N] scratch; flags uint32 [smr_gemv_flag_blocks(N) * S]
+ *   zero on entry and zero again on exit; out [batch,N] bf16 = the fp32 sum of the
+ *   S partials in sender order (rank-major), i.e.
+ *   bf16(((0 + p_0) + p_1) + ... + p_{ws-1}) when S == ws.  batch <= 8. */
 int smr_gemv_allreduce(const void* x_dev, const void* w_dev, float* partials_dev,
                        uint32_t* flags_dev, void* out_dev, int batch, int K, int N,
                        int world_size, uint32_t* status, void* stream);
 int smr_gemv_flag_blocks(int N);
+int smr_gemv_senders(int N, int K, int world_size);
+/* Tuning knob: threads per contiguous row segment (16 or 64; 0 = default 16) and
+ * sub-shards per rank (1..8; 0 = chosen so that at least 256 workgroups run). */
+int smr_set_gemv_launch(int threads_per_row, int sub_shards);
 
 #ifdef __cplusplus
 }

@@ -287,8 +287,7 @@ __global__ __launch_bounds__(kGemmThreads, 1) void ag_matmul_kernel(
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
 #pragma unroll
-    for (int w = 0; w < kWarmAhead; ++w)
-      if (2 + w < nk) warm_stage(2 + w);
+    for (int w = 0; w < kWarmAhead; ++w) warm_stage(2 + w < nk ? 2 + w : nk - 1);
 
     // Fragment double buffer: while the MFMAs of K step kk run, the fragments of
     // step kk+1 are read.  The workgroup barrier sits before the last K step of a
@@ -299,6 +298,52 @@ __global__ __launch_bounds__(kGemmThreads, 1) void ag_matmul_kernel(
     bf16x8 af0[FM], bf0[FN], af1[FM], bf1[FN];
     read_frags(af0, bf0, 0, 0);
 
+    // Last K step of a stage, issued right behind the barrier.  Its fragments are
+    // already in registers, so the MFMAs can start at once; the loads of stage
+    // kt+2, the first fragment reads of stage kt+1 and the warm-up touches are
+    // slotted in between them instead of standing in front of them.  There is
+    // one code path: past the end of K the loads are clamped to the last K-slab
+    // (they land in a stage nobody reads any more) rather than branched around,
+    // which keeps the accumulators in place across the whole loop body.
+    auto last_step = [&](auto stage_tag, int kt) {
+      constexpr int S = decltype(stage_tag)::value;
+      const int kl = kt + 2 < nk ? kt + 2 : nk - 1;
+      const uint8_t* ak = a_base + (int64_t)kl * kRowBytes;
+      const uint8_t* bk = b_base + (int64_t)kl * kRowBytes;
+      const uint32_t la = lds0 + S * T::kABytes + wave * (GA * 1024);
+      const uint32_t lb = lds0 + T::kBBase + S * T::kBBytes + wave * (GB * 1024);
+      constexpr int kMfma = FM * FN, kLoads = GA + GB, kReads = FM + FN;
+      // loads are spread over all MFMAs, fragment reads over the later ones
+      constexpr int kReadFrom = kMfma >= 2 * kReads ? kMfma / 4 : 0;
+      // (all loops below have constant trip counts so that they unroll fully and
+      // every array index is a compile-time constant)
+#pragma unroll
+      for (int ni = 0; ni < FN; ++ni) {
+#pragma unroll
+        for (int mi = 0; mi < FM; ++mi) {
+          const int slot = ni * FM + mi;
+          acc[ni][mi] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bf1[ni], af1[mi], acc[ni][mi], 0, 0, 0);
+#pragma unroll
+          for (int g = 0; g < GA; ++g)
+            if (g * kMfma / kLoads == slot) load_group(ak, a_off[g], la + g * 1024);
+#pragma unroll
+          for (int g = 0; g < GB; ++g)
+            if ((GA + g) * kMfma / kLoads == slot) load_group(bk, b_off[g], lb + g * 1024);
+#pragma unroll
+          for (int r = 0; r < FM; ++r)
+            if (kReadFrom + r * (kMfma - kReadFrom) / kReads == slot)
+              af0[r] = lds_read_frag(a_fr[(r & 1) << 1] + (S ^ 1) * T::kABytes + r * (32 * kRowBytes));
+#pragma unroll
+          for (int r = 0; r < FN; ++r)
+            if (kReadFrom + (FM + r) * (kMfma - kReadFrom) / kReads == slot)
+              bf0[r] = lds_read_frag(b_fr[(r & 1) << 1] + (S ^ 1) * T::kBBytes + r * (32 * kRowBytes));
+          if (slot == kMfma - 1) {
+            const int kw = kt + 2 + kWarmAhead;
+            warm_stage(kw < nk ? kw : nk - 1);
+          }
+        }
+      }
+    };
     auto stage_body = [&](auto stage_tag, int kt) {
       constexpr int S = decltype(stage_tag)::value;
       read_frags(af1, bf1, S, 1);
@@ -310,21 +355,14 @@ __global__ __launch_bounds__(kGemmThreads, 1) void ag_matmul_kernel(
       read_frags(af1, bf1, S, 3);
       mfma_all(af0, bf0);
       interleave_mfma_dsread<FM * FN, FM + FN>();
-      // The compiler does not track direct-to-LDS loads across the loop back
-      // edge: wait for this wave's own loads explicitly before the barrier.
-      // The warm-up loads issued after them (if any were) may stay in flight:
-      // loads return in order.
-      if (kWarmLoads > 0 && (kt == 0 || kt + 1 + kWarmAhead < nk)) {
-        if constexpr (kWarmLoads == 1) asm volatile("s_waitcnt vmcnt(1)" ::: "memory");
-        else asm volatile("s_waitcnt vmcnt(2)" ::: "memory");
-      } else {
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-      }
+      // Wait for this wave's own tile loads before the barrier; the compiler does
+      // not count them (see load_group).  The kWarmLoads warm-up loads issued
+      // behind them may stay in flight: loads return in order.
+      if constexpr (kWarmLoads == 0) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      else if constexpr (kWarmLoads == 1) asm volatile("s_waitcnt vmcnt(1)" ::: "memory");
+      else asm volatile("s_waitcnt vmcnt(2)" ::: "memory");
       __syncthreads();     // stage S fully read by everyone; the other stage has landed
-      if (kt + 2 < nk) load_stage(S, kt + 2);
-      if (kt + 2 + kWarmAhead < nk) warm_stage(kt + 2 + kWarmAhead);
-      if (kt + 1 < nk) read_frags(af0, bf0, S ^ 1, 0);
-      mfma_all(af1, bf1);
+      last_step(stage_tag, kt);
     };
     int kt = 0;
     for (; kt + 1 < nk; kt += 2) {

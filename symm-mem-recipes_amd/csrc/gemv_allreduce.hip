@@ -4,48 +4,72 @@
 //   p_r = x[:, shard r] @ W[shard r, :]   (fp32)
 //
 // The job is bound by reading W once (K*N*2 bytes).  W is row-major [K, N], so a
-// row is N contiguous bf16: 16 threads cover 128 columns with one 128-bit load
-// each, and the 16 thread groups of a workgroup stride over the shard's K rows,
-// 8 independent loads in flight per thread.  x (at most 8 rows) is staged in LDS
-// as fp32, transposed to [k][batch] so a k step reads its batch values with one
-// or two broadcast 128-bit LDS reads.
+// row is N contiguous bf16: TPR threads cover a row segment with one 128-bit load
+// each, and the 256/TPR thread groups of a workgroup stride over the K rows of
+// their share with 4 to 16 independent loads in flight per thread.  x (at most 8
+// rows) is staged in LDS as fp32, transposed to [k][batch].
 //
-// Workgroup id -> (column block = id / ws, rank = id % ws).  Every workgroup
-// writes its fp32 partial, releases, and raises flag[column block][rank]
-// (CAS 0 -> 1).  The workgroup of rank 0 then consumes the ws flags of its column
-// block (CAS 1 -> 0, so the flags are zero again on exit), acquires, and adds
-// the partials in rank order.
+// Workgroup id -> (sender = rank * sub + sub-shard, column block), column block
+// fastest.  Every workgroup writes its fp32 partial, waits until the stores are
+// acknowledged, and raises flag[column block][sender] (CAS 0 -> 1).  The first
+// workgroup of a column block then consumes all flags (CAS 1 -> 0, so the flags
+// are zero again on exit) and adds the partials in sender order, i.e. rank by
+// rank.  The partials travel with agent-coherent stores and loads, so no cache
+// write-back or invalidate surrounds the flags.
 #include "smr_device.hpp"
 
 namespace smr {
 
 constexpr int kGemvThreads = 256;
-constexpr int kGemvCols = 128;               // columns per workgroup
-constexpr int kGemvTpr = kGemvCols / 8;      // threads per row segment (16)
-constexpr int kGemvKGroups = kGemvThreads / kGemvTpr;   // 16
-constexpr int kGemvUnroll = 8;
 constexpr int kGemvKChunk = 1024;            // K rows of x staged in LDS at a time
+
+// Launch shape: TPR threads cover one row segment of TPR*8 columns (TPR*16
+// contiguous bytes); the K rows of a rank's shard may be split into `sub`
+// sub-shards, one workgroup each, when the column blocks alone do not fill the
+// chip.  Measured on MI355X at K = N = 8192: 16 threads per segment (512
+// workgroups, 64 of them combining) beat 64-thread segments at every batch size.
+// smr_set_gemv_launch overrides.
+static int g_gemv_tpr = 16;
+static int g_gemv_sub = 0;                   // 0 = pick so that >= 256 workgroups run
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef __attribute__((address_space(1))) u32x4 GlobalVec;
 
-template <int B>
+template <int B, int TPR>
 __global__ __launch_bounds__(kGemvThreads) void gemv_allreduce_kernel(
     const uint16_t* __restrict__ x, const uint8_t* __restrict__ w, float* __restrict__ partials,
     uint32_t* __restrict__ flags, uint16_t* __restrict__ out, int batch, int K, int N,
-    int world_size, uint64_t limit_ticks, uint32_t* status) {
-  __shared__ __attribute__((aligned(16))) float xs[kGemvKChunk][B];
-  __shared__ float red[kGemvThreads / 64][B][kGemvCols];
+    int world_size, int sub, uint64_t limit_ticks, uint32_t* status) {
+  // 128-bit loads in flight per thread: fewer for larger batches, whose 8*B
+  // accumulators would otherwise leave one wave per SIMD
+  constexpr int kGemvUnroll = B >= 8 ? 4 : (B >= 4 ? 8 : 16);
+  constexpr int kCols = TPR * 8;                         // columns per workgroup
+  constexpr int kKGroups = kGemvThreads / TPR;           // row groups per workgroup
+  constexpr int kKGroupsPerWave = 64 / TPR;
+  // x staging and the cross-wave reduction never live at the same time: one buffer
+  constexpr int kXsFloats = kGemvKChunk * B, kRedFloats = (kGemvThreads / 64) * B * kCols;
+  __shared__ __attribute__((aligned(16))) float smem[kXsFloats > kRedFloats ? kXsFloats : kRedFloats];
+  float (*xs)[B] = reinterpret_cast<float (*)[B]>(smem);
+  float (*red)[B][kCols] = reinterpret_cast<float (*)[B][kCols]>(smem);
 
-  const int cblk = blockIdx.x / world_size;
-  const int rank = blockIdx.x % world_size;
+  // Column block fastest: workgroups with neighbouring ids read neighbouring 1 KiB
+  // segments of the same rows, so the workgroups in flight together sweep whole
+  // rows of W instead of segments that lie a power-of-two stride apart.
+  const int senders = world_size * sub;
+  const int cblocks = gridDim.x / senders;
+  const int cblk = blockIdx.x % cblocks;
+  const int sender = blockIdx.x / cblocks;               // rank-major, sub-shard-minor
+  const int rank = sender / sub;
   const int tid = threadIdx.x;
-  const int col_t = tid % kGemvTpr;
-  const int kg = tid / kGemvTpr;
-  const int col0 = cblk * kGemvCols + col_t * 8;
+  const int col_t = tid % TPR;
+  const int kg = tid / TPR;
+  const int col0 = cblk * kCols + col_t * 8;
   const bool col_ok = col0 < N;
-  const int ks = K / world_size;
-  const int k_begin = rank * ks, k_end = k_begin + ks;
+  const int ks = K / world_size;                         // rows per rank
+  const int kss = (ks + sub - 1) / sub;                  // rows per sub-shard
+  const int k_begin = rank * ks + (sender % sub) * kss;
+  int k_end = k_begin + kss;
+  if (k_end > (rank + 1) * ks) k_end = (rank + 1) * ks;
   const int64_t row_bytes = (int64_t)N * 2;
 
   float acc[B][8];
@@ -56,28 +80,34 @@ __global__ __launch_bounds__(kGemvThreads) void gemv_allreduce_kernel(
 
   for (int k0 = k_begin; k0 < k_end; k0 += kGemvKChunk) {
     const int kc = (k_end - k0) < kGemvKChunk ? (k_end - k0) : kGemvKChunk;
-    for (int i = tid; i < kc * B; i += kGemvThreads) {
-      const int b = i / kc, k = i - b * kc;
-      xs[k][b] = b < batch ? bf16_lo((uint32_t)x[(int64_t)b * K + k0 + k]) : 0.0f;
+    // stage x[:, k0 .. k0+kc) as fp32, transposed to [k][batch]
+#pragma unroll
+    for (int b = 0; b < B; ++b) {
+#pragma unroll
+      for (int i = 0; i < kGemvKChunk / kGemvThreads; ++i) {
+        const int k = tid + i * kGemvThreads;
+        if (k < kc) xs[k][b] = b < batch ? bf16_lo((uint32_t)x[(int64_t)b * K + k0 + k]) : 0.0f;
+      }
     }
     __syncthreads();
     if (col_ok) {
-      const GlobalVec* wp = (const GlobalVec*)(uintptr_t)(w + (int64_t)k0 * row_bytes + (int64_t)col0 * 2);
-      for (int k = kg; k < kc; k += kGemvKGroups * kGemvUnroll) {
+      const __attribute__((address_space(1))) uint8_t* wp =
+          (const __attribute__((address_space(1))) uint8_t*)(uintptr_t)(w + (int64_t)k0 * row_bytes +
+                                                                      (int64_t)col0 * 2);
+      for (int k = kg; k < kc; k += kKGroups * kGemvUnroll) {
         u32x4 wv[kGemvUnroll];
 #pragma unroll
         for (int u = 0; u < kGemvUnroll; ++u) {
-          const int kk = k + u * kGemvKGroups;
-          if (kk < kc)
-            wv[u] = __builtin_nontemporal_load(
-                (const GlobalVec*)((const __attribute__((address_space(1))) uint8_t*)wp + (int64_t)kk * row_bytes));
-          else
-            wv[u] = u32x4{0u, 0u, 0u, 0u};
+          // rows past the end are re-read from the last valid row and weighted by 0
+          const int kk = k + u * kKGroups;
+          const int kr = kk < kc ? kk : kc - 1;
+          wv[u] = __builtin_nontemporal_load((const GlobalVec*)(wp + (int64_t)kr * row_bytes));
         }
 #pragma unroll
         for (int u = 0; u < kGemvUnroll; ++u) {
-          const int kk = k + u * kGemvKGroups;
-          const int ksafe = kk < kc ? kk : 0;      // wv is zero past the end
+          const int kk = k + u * kKGroups;
+          const bool live = kk < kc;
+          const int kr = live ? kk : kc - 1;
           float wf[8];
           wf[0] = bf16_lo(wv[u].x); wf[1] = bf16_hi(wv[u].x);
           wf[2] = bf16_lo(wv[u].y); wf[3] = bf16_hi(wv[u].y);
@@ -85,7 +115,7 @@ __global__ __launch_bounds__(kGemvThreads) void gemv_allreduce_kernel(
           wf[6] = bf16_lo(wv[u].w); wf[7] = bf16_hi(wv[u].w);
 #pragma unroll
           for (int b = 0; b < B; ++b) {
-            const float xb = xs[ksafe][b];
+            const float xb = live ? xs[kr][b] : 0.0f;
 #pragma unroll
             for (int j = 0; j < 8; ++j) acc[b][j] = __builtin_fmaf(xb, wf[j], acc[b][j]);
           }
@@ -95,62 +125,106 @@ __global__ __launch_bounds__(kGemvThreads) void gemv_allreduce_kernel(
     __syncthreads();
   }
 
-  // combine the 16 k groups: 4 per wave by lane shuffles, then 4 waves through LDS
+  // combine the row groups: those of one wave by lane shuffles, the waves through LDS
 #pragma unroll
   for (int b = 0; b < B; ++b)
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
       float v = acc[b][j];
-      v += __shfl_xor(v, 16, 64);
-      v += __shfl_xor(v, 32, 64);
+#pragma unroll
+      for (int off = TPR; off < 64; off <<= 1) v += __shfl_xor(v, off, 64);
       acc[b][j] = v;
     }
-  if ((tid & 63) < kGemvTpr) {
+  if ((tid & 63) < TPR) {
 #pragma unroll
     for (int b = 0; b < B; ++b)
 #pragma unroll
       for (int j = 0; j < 8; ++j) red[tid >> 6][b][col_t * 8 + j] = acc[b][j];
   }
   __syncthreads();
-  const int col = cblk * kGemvCols + tid;
-  if (tid < kGemvCols && col < N) {
-    for (int b = 0; b < batch; ++b) {
-      const float p = ((red[0][b][tid] + red[1][b][tid]) + red[2][b][tid]) + red[3][b][tid];
-      partials[((int64_t)rank * batch + b) * N + col] = p;
+  static_assert(kKGroupsPerWave * (kGemvThreads / 64) == kKGroups, "row groups = per wave x waves");
+  for (int c = tid; c < kCols; c += kGemvThreads) {
+    const int col = cblk * kCols + c;
+    if (col < N) {
+      for (int b = 0; b < batch; ++b) {
+        const float p = ((red[0][b][c] + red[1][b][c]) + red[2][b][c]) + red[3][b][c];
+        store_coherent(&partials[((int64_t)sender * batch + b) * N + col], p);
+      }
     }
   }
 
-  // publish the partial: every wave releases, the workgroup meets, one send
-  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+  // publish the partial: it was written through, so once every thread's stores
+  // are acknowledged and the workgroup has met, one thread raises the flag
+  wait_stores_acknowledged();
   __syncthreads();
-  uint32_t* my_flags = flags + (size_t)cblk * world_size;
-  if (tid == 0 && !send_signal(my_flags + rank, limit_ticks))
-    report(status, SMR_ST_SEND_TIMEOUT, rank, cblk, 0u);
-  if (rank != 0) return;
+  uint32_t* my_flags = flags + (size_t)cblk * senders;
+  if (tid == 0 && !send_signal_relaxed(my_flags + sender, limit_ticks))
+    report(status, SMR_ST_SEND_TIMEOUT, sender, cblk, 0u);
+  if (sender != 0) return;
 
-  // rank 0 of the column block: consume all ws flags, then add in rank order
+  // first workgroup of the column block: consume all flags, then add the partials
+  // in rank order (sub-shards of a rank in order inside it)
   int bad = 0;
-  if (tid < world_size && !wait_signal_reset(my_flags + tid, limit_ticks)) {
+  if (tid < senders && !wait_signal_reset(my_flags + tid, limit_ticks)) {
     report(status, SMR_ST_WAIT_TIMEOUT, tid, cblk, 0u);
     bad = 1;
   }
   bad = __syncthreads_or(bad);
-  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
   if (bad) return;
-  if (tid < kGemvCols && col < N) {
-    for (int b = 0; b < batch; ++b) {
-      float a = 0.0f;
-      for (int r = 0; r < world_size; ++r) a += partials[((int64_t)r * batch + b) * N + col];
-      out[(int64_t)b * N + col] = (uint16_t)f32_to_bf16_bits(a);
+  // 16 partials are fetched at a time (independent loads), then added strictly in
+  // sender order; the +0 terms that pad the last group cannot change a sum that
+  // starts from +0.
+  for (int idx = tid; idx < batch * kCols; idx += kGemvThreads) {
+    const int b = idx / kCols, c = idx % kCols;
+    const int col = cblk * kCols + c;
+    if (col >= N) continue;
+    const float* p = partials + (int64_t)b * N + col;
+    const int64_t plane = (int64_t)batch * N;
+    float a = 0.0f;
+    for (int r0 = 0; r0 < senders; r0 += 16) {
+      float v[16];
+#pragma unroll
+      for (int u = 0; u < 16; ++u) v[u] = r0 + u < senders ? load_coherent(p + (int64_t)(r0 + u) * plane) : 0.0f;
+#pragma unroll
+      for (int u = 0; u < 16; ++u) a += v[u];
     }
+    out[(int64_t)b * N + col] = (uint16_t)f32_to_bf16_bits(a);
   }
+}
+
+static int gemv_sub_for(int N, int K, int world_size) {
+  if (g_gemv_sub > 0) return g_gemv_sub;
+  const int cols = g_gemv_tpr * 8;
+  const int cblocks = (N + cols - 1) / cols;
+  int sub = 1;
+  while (sub < 8 && cblocks * world_size * sub < 256 && (K / world_size) / (sub * 2) >= 64) sub *= 2;
+  return sub;
 }
 
 }  // namespace smr
 
 extern "C" {
 
-int smr_gemv_flag_blocks(int N) { return N <= 0 ? 0 : (N + smr::kGemvCols - 1) / smr::kGemvCols; }
+int smr_set_gemv_launch(int threads_per_row, int sub_shards) {
+  using namespace smr;
+  if (threads_per_row == 0) threads_per_row = 16;
+  if (threads_per_row != 16 && threads_per_row != 64)
+    return fail(SMR_E_INVALID, "smr_set_gemv_launch: threads_per_row must be 16 or 64");
+  if (sub_shards < 0 || sub_shards > 8)
+    return fail(SMR_E_INVALID, "smr_set_gemv_launch: sub_shards must be 0..8");
+  g_gemv_tpr = threads_per_row;
+  g_gemv_sub = sub_shards;
+  return 0;
+}
+
+int smr_gemv_flag_blocks(int N) {
+  return N <= 0 ? 0 : (N + smr::g_gemv_tpr * 8 - 1) / (smr::g_gemv_tpr * 8);
+}
+
+int smr_gemv_senders(int N, int K, int world_size) {
+  if (N <= 0 || K <= 0 || world_size < 1 || world_size > SMR_MAX_WORLD_SIZE) return 0;
+  return world_size * smr::gemv_sub_for(N, K, world_size);
+}
 
 int smr_gemv_allreduce(const void* x_dev, const void* w_dev, float* partials_dev, uint32_t* flags_dev,
                        void* out_dev, int batch, int K, int N, int world_size, uint32_t* status,
@@ -166,7 +240,8 @@ int smr_gemv_allreduce(const void* x_dev, const void* w_dev, float* partials_dev
     return fail(SMR_E_INVALID, "smr_gemv_allreduce: K must split evenly over the ranks");
   if (N % 8 != 0 || (reinterpret_cast<uintptr_t>(w_dev) & 15u))
     return fail(SMR_E_UNSUPPORTED, "smr_gemv_allreduce: N must be a multiple of 8 and W 16-byte aligned");
-  const unsigned grid = (unsigned)smr_gemv_flag_blocks(N) * (unsigned)world_size;
+  const int sub = gemv_sub_for(N, K, world_size);
+  const unsigned grid = (unsigned)smr_gemv_flag_blocks(N) * (unsigned)world_size * (unsigned)sub;
   if (grid > 4096u)
     return fail(SMR_E_UNSUPPORTED, "smr_gemv_allreduce: more than 4096 workgroups cannot be co-resident");
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
@@ -174,13 +249,19 @@ int smr_gemv_allreduce(const void* x_dev, const void* w_dev, float* partials_dev
   const uint8_t* w = reinterpret_cast<const uint8_t*>(w_dev);
   uint16_t* out = reinterpret_cast<uint16_t*>(out_dev);
   const uint64_t lim = spin_limit_ticks();
-#define SMR_GEMV_LAUNCH(BP)                                                                        \
-  hipLaunchKernelGGL((gemv_allreduce_kernel<BP>), dim3(grid), dim3(kGemvThreads), 0, st, x, w,     \
-                     partials_dev, flags_dev, out, batch, K, N, world_size, lim, status)
-  if (batch == 1) SMR_GEMV_LAUNCH(1);
-  else if (batch == 2) SMR_GEMV_LAUNCH(2);
-  else if (batch <= 4) SMR_GEMV_LAUNCH(4);
-  else SMR_GEMV_LAUNCH(8);
+#define SMR_GEMV_LAUNCH(BP, TPR)                                                                   \
+  hipLaunchKernelGGL((gemv_allreduce_kernel<BP, TPR>), dim3(grid), dim3(kGemvThreads), 0, st, x, w, \
+                     partials_dev, flags_dev, out, batch, K, N, world_size, sub, lim, status)
+#define SMR_GEMV_BATCH(TPR)                                                                        \
+  do {                                                                                             \
+    if (batch == 1) SMR_GEMV_LAUNCH(1, TPR);                                                       \
+    else if (batch == 2) SMR_GEMV_LAUNCH(2, TPR);                                                  \
+    else if (batch <= 4) SMR_GEMV_LAUNCH(4, TPR);                                                  \
+    else SMR_GEMV_LAUNCH(8, TPR);                                                                  \
+  } while (0)
+  if (g_gemv_tpr == 16) SMR_GEMV_BATCH(16);
+  else SMR_GEMV_BATCH(64);
+#undef SMR_GEMV_BATCH
 #undef SMR_GEMV_LAUNCH
   return check_hip(hipGetLastError(), "smr_gemv_allreduce launch");
 }

@@ -27,8 +27,16 @@ enum ReduceLayout : int { kPlain = 0, kProxy = 1, kAllRanks = 2 };
 constexpr int kReduceMaxThreads = 1024;
 // Launch shape (threads per workgroup, cap on workgroups = barrier blocks per
 // rank); smr_set_reduce_launch overrides the defaults.
-static int g_reduce_threads = 256;
-static int g_reduce_max_blocks = 2048;   // 8 workgroups of 256 threads per CU on 256 CUs
+// Defaults from a sweep on MI355X: one workgroup per compute unit streams best
+// (8 contiguous read streams of 1 MiB-strided chunks keep the DRAM pages open);
+// 512 threads below 32 MiB per buffer, 256 above.  0 = pick by size.
+static int g_reduce_threads = 0;
+static int g_reduce_max_blocks = 256;
+
+static int reduce_threads_for(int64_t nvec) {
+  if (g_reduce_threads != 0) return g_reduce_threads;
+  return nvec >= (int64_t)(32 << 20) / 16 ? 256 : 512;
+}
 
 struct alignas(16) Vec16 {
   uint32_t w[4];
@@ -139,26 +147,26 @@ __global__ __launch_bounds__(kReduceMaxThreads) void one_shot_all_reduce_kernel(
 }
 
 template <bool BF16, int WS>
-static int launch_ws(bool write_all, dim3 grid, hipStream_t s, const uint64_t* bp, const uint64_t* sp,
+static int launch_ws(bool write_all, dim3 grid, int threads, hipStream_t s, const uint64_t* bp, const uint64_t* sp,
                      Vec16* out, int64_t nvec, int rank, int layout, int nblocks, int do_barrier,
                      uint32_t* status) {
   const uint64_t lim = spin_limit_ticks();
   if (write_all)
-    hipLaunchKernelGGL((one_shot_all_reduce_kernel<BF16, WS, true>), grid, dim3(g_reduce_threads), 0, s,
+    hipLaunchKernelGGL((one_shot_all_reduce_kernel<BF16, WS, true>), grid, dim3(threads), 0, s,
                        bp, sp, out, nvec, rank, layout, nblocks, do_barrier, lim, status);
   else
-    hipLaunchKernelGGL((one_shot_all_reduce_kernel<BF16, WS, false>), grid, dim3(g_reduce_threads), 0, s,
+    hipLaunchKernelGGL((one_shot_all_reduce_kernel<BF16, WS, false>), grid, dim3(threads), 0, s,
                        bp, sp, out, nvec, rank, layout, nblocks, do_barrier, lim, status);
   return check_hip(hipGetLastError(), "smr_one_shot_all_reduce launch");
 }
 
 template <bool BF16>
-static int launch_dtype(int ws, bool write_all, dim3 grid, hipStream_t s, const uint64_t* bp,
+static int launch_dtype(int ws, bool write_all, dim3 grid, int threads, hipStream_t s, const uint64_t* bp,
                         const uint64_t* sp, Vec16* out, int64_t nvec, int rank, int layout,
                         int nblocks, int do_barrier, uint32_t* status) {
 #define SMR_WS_CASE(W)                                                                          \
   case W:                                                                                       \
-    return launch_ws<BF16, W>(write_all, grid, s, bp, sp, out, nvec, rank, layout, nblocks,     \
+    return launch_ws<BF16, W>(write_all, grid, threads, s, bp, sp, out, nvec, rank, layout, nblocks,     \
                               do_barrier, status);
   switch (ws) {
     SMR_WS_CASE(1) SMR_WS_CASE(2) SMR_WS_CASE(3) SMR_WS_CASE(4)
@@ -173,9 +181,8 @@ static int launch_dtype(int ws, bool write_all, dim3 grid, hipStream_t s, const 
 extern "C" {
 
 int smr_set_reduce_launch(int threads, int max_blocks) {
-  if (threads == 0) threads = 256;
-  if (max_blocks == 0) max_blocks = 2048;
-  if (threads < 64 || threads > smr::kReduceMaxThreads || (threads & 63) != 0)
+  if (max_blocks == 0) max_blocks = 256;
+  if (threads != 0 && (threads < 64 || threads > smr::kReduceMaxThreads || (threads & 63) != 0))
     return smr::fail(SMR_E_INVALID, "smr_set_reduce_launch: threads must be a multiple of 64 in 64..1024");
   if (max_blocks < 1 || max_blocks > 4096)
     return smr::fail(SMR_E_INVALID, "smr_set_reduce_launch: max_blocks must be 1..4096");
@@ -188,7 +195,8 @@ int smr_reduce_num_blocks(int64_t numel, int dtype) {
   const int per_vec = dtype == SMR_DTYPE_BF16 ? 8 : 4;
   if (numel <= 0) return 0;
   const int64_t nvec = numel / per_vec;
-  int64_t nb = (nvec + smr::g_reduce_threads - 1) / smr::g_reduce_threads;
+  const int threads = smr::reduce_threads_for(nvec);
+  int64_t nb = (nvec + threads - 1) / threads;
   if (nb > smr::g_reduce_max_blocks) nb = smr::g_reduce_max_blocks;
   if (nb < 1) nb = 1;
   return (int)nb;
@@ -223,6 +231,7 @@ int smr_one_shot_all_reduce(const uint64_t* buffer_ptrs_dev, const uint64_t* sig
 
   const int64_t nvec = numel / per_vec;
   const int nblocks = smr_reduce_num_blocks(numel, dtype);
+  const int threads = reduce_threads_for(nvec);
   const int do_barrier = barrier_mode != SMR_BARRIER_NONE;
   int layout = kPlain;
   unsigned grid = (unsigned)nblocks;
@@ -231,15 +240,15 @@ int smr_one_shot_all_reduce(const uint64_t* buffer_ptrs_dev, const uint64_t* sig
     grid = (unsigned)nblocks * (unsigned)world_size;
   } else if (do_barrier) {
     layout = kProxy;
-    const int per_proxy = g_reduce_threads / 8;
+    const int per_proxy = threads / 8;
     grid = (unsigned)nblocks + (unsigned)((nblocks + per_proxy - 1) / per_proxy);
   }
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
   Vec16* o = reinterpret_cast<Vec16*>(out);
   if (dtype == SMR_DTYPE_BF16)
-    return launch_dtype<true>(world_size, write_all != 0, dim3(grid), s, buffer_ptrs_dev,
+    return launch_dtype<true>(world_size, write_all != 0, dim3(grid), threads, s, buffer_ptrs_dev,
                               signal_pad_ptrs_dev, o, nvec, rank, layout, nblocks, do_barrier, status);
-  return launch_dtype<false>(world_size, write_all != 0, dim3(grid), s, buffer_ptrs_dev,
+  return launch_dtype<false>(world_size, write_all != 0, dim3(grid), threads, s, buffer_ptrs_dev,
                              signal_pad_ptrs_dev, o, nvec, rank, layout, nblocks, do_barrier, status);
 }
 

@@ -59,6 +59,33 @@ __device__ __forceinline__ void report(uint32_t* status, uint32_t code, uint32_t
 // __HIP_MEMORY_SCOPE_SYSTEM on fine-grained peer mappings with the same code.
 constexpr int kScope = __HIP_MEMORY_SCOPE_AGENT;
 
+// ---------------------------------------------------------------- coherent data accesses
+// A release fence at agent scope writes back the whole L2 of the XCD and an
+// acquire fence invalidates it; with thousands of workgroups handing data over
+// through flags those two cache-wide operations queue up behind each other and
+// cost more than the hand-over itself.  Data that is handed over through a flag is
+// therefore written with agent-scope (write-through) stores and read with
+// agent-scope loads, which go to the level where all XCDs agree.  The producer
+// then only has to wait until its stores are acknowledged before it raises the
+// flag, and the consumer needs nothing but the flag: no write-back, no invalidate.
+__device__ __forceinline__ void store_coherent(float* p, float v) {
+  __hip_atomic_store(p, v, __ATOMIC_RELAXED, kScope);
+}
+__device__ __forceinline__ float load_coherent(const float* p) {
+  return __hip_atomic_load(p, __ATOMIC_RELAXED, kScope);
+}
+__device__ __forceinline__ void store_coherent(uint64_t* p, uint64_t v) {
+  __hip_atomic_store(p, v, __ATOMIC_RELAXED, kScope);
+}
+__device__ __forceinline__ uint64_t load_coherent(const uint64_t* p) {
+  return __hip_atomic_load(p, __ATOMIC_RELAXED, kScope);
+}
+// All of this thread's stores have been acknowledged (and nothing is moved across
+// by the compiler).
+__device__ __forceinline__ void wait_stores_acknowledged() {
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+}
+
 // Spin helper: true while the caller may keep spinning.
 struct SpinClock {
   uint64_t start, limit;
@@ -129,6 +156,12 @@ __device__ __forceinline__ bool send_signal(uint32_t* addr, uint64_t limit_ticks
   return spin_cas(addr, 0u, 1u, limit_ticks);
 }
 
+// The same without the release fence, for data written with store_coherent and
+// followed by wait_stores_acknowledged.
+__device__ __forceinline__ bool send_signal_relaxed(uint32_t* addr, uint64_t limit_ticks) {
+  return spin_cas(addr, 0u, 1u, limit_ticks);
+}
+
 // CAS 1 -> 0 until it succeeds (consumes and resets the flag).  Relaxed: the
 // caller acquires afterwards, once, for the whole workgroup.
 __device__ __forceinline__ bool wait_signal_reset(uint32_t* addr, uint64_t limit_ticks) {
@@ -177,7 +210,7 @@ __device__ __forceinline__ void wait_signal(const uint32_t* addr, uint64_t limit
 __device__ __forceinline__ bool blockwise_barrier(const uint64_t* signal_pad_ptrs,
                                                   uint32_t block_id, int rank, int world_size,
                                                   uint64_t limit_ticks, uint32_t* status,
-                                                  bool publish = true) {
+                                                  bool publish = true, bool acquire = true) {
   __syncthreads();
   const int lane = threadIdx.x;
   int bad = 0;
@@ -197,7 +230,10 @@ __device__ __forceinline__ bool blockwise_barrier(const uint64_t* signal_pad_ptr
       uint32_t level = 0;
       bool ok = false;
       for (;;) {
-        if (is_send || __hip_atomic_load(slot, __ATOMIC_RELAXED, kScope) == from) {
+        // attempt first (the flag is usually already there); after a failed
+        // attempt a wait lane polls with plain loads until the flag shows up
+        if (is_send || level == 0 ||
+            __hip_atomic_load(slot, __ATOMIC_RELAXED, kScope) == from) {
           uint32_t expected = from;
           ok = __hip_atomic_compare_exchange_strong(slot, &expected, to, __ATOMIC_RELAXED,
                                                     __ATOMIC_RELAXED, kScope);
@@ -211,7 +247,7 @@ __device__ __forceinline__ bool blockwise_barrier(const uint64_t* signal_pad_ptr
         bad = 1;
       }
     }
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+    if (acquire) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
   }
   bad = __syncthreads_or(bad);
   return bad == 0;

@@ -50,6 +50,8 @@ SIGNATURES = {
     "smr_ag_matmul_grid": (_i, [_i, _i, _i, _i, _i, _i]),
     "smr_gemv_allreduce": (_i, [_p, _p, _p, _p, _p, _i, _i, _i, _i, _p, _p]),
     "smr_gemv_flag_blocks": (_i, [_i]),
+    "smr_gemv_senders": (_i, [_i, _i, _i]),
+    "smr_set_gemv_launch": (_i, [_i, _i]),
 }
 
 _lib: Optional[C.CDLL] = None

@@ -4,7 +4,8 @@ the one of symm_mem_recipes/triton_barrier.py:119-129 and
 symm_mem_recipes/triton_all_gather_matmul.py:72-95.
 
 ``W`` ([K, N], row-major) is split along K into ``world_size`` shards, one per
-emulated rank; every rank multiplies its shard of ``x`` with its shard of ``W`` in
+emulated rank (the kernel may cut a shard further into sub-shards to fill the
+chip); every producer multiplies its share of ``x`` with its share of ``W`` in
 fp32, publishes the partial and raises a flag; the partials are added in rank
 order 0..world_size-1 in fp32 and rounded to bf16 once.
 """
@@ -21,11 +22,13 @@ class GemvWorkspace:
     """Scratch the kernel needs: fp32 partials, the flag array (zero between
     calls) and status words."""
 
-    def __init__(self, batch: int, N: int, world_size: int, device):
+    def __init__(self, batch: int, N: int, world_size: int, device, K: int = 0):
         lib = _lib.load()
         self.batch, self.N, self.world_size = batch, N, world_size
-        self.partials = torch.empty(world_size, batch, N, dtype=torch.float32, device=device)
-        self.flags = torch.zeros(lib.smr_gemv_flag_blocks(N) * world_size, dtype=torch.int32, device=device)
+        # partial producers per column block: the ranks, each possibly cut into K sub-shards
+        self.senders = lib.smr_gemv_senders(N, K, world_size) if K else 8 * world_size
+        self.partials = torch.empty(self.senders, batch, N, dtype=torch.float32, device=device)
+        self.flags = torch.zeros(lib.smr_gemv_flag_blocks(N) * self.senders, dtype=torch.int32, device=device)
         self.status = torch.zeros(_lib.STATUS_WORDS, dtype=torch.int32, device=device)
 
     def check_status(self) -> None:
@@ -48,8 +51,9 @@ def gemv_all_reduce(x: torch.Tensor, w: torch.Tensor, world_size: int = 8,
     assert 1 <= batch <= 8, "batch must be 1..8"
     assert K % world_size == 0, "K must split evenly over the ranks"
     if workspace is None:
-        workspace = GemvWorkspace(batch, N, world_size, x.device)
+        workspace = GemvWorkspace(batch, N, world_size, x.device, K)
     assert (workspace.batch, workspace.N, workspace.world_size) == (batch, N, world_size)
+    assert workspace.senders >= _lib.load().smr_gemv_senders(N, K, world_size)
     if out is None:
         out = torch.empty(batch, N, dtype=torch.bfloat16, device=x.device)
     rc = _lib.load().smr_gemv_allreduce(

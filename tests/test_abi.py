@@ -36,11 +36,16 @@ def test_version_and_timeout_roundtrip(lib):
 
 
 def test_reduce_grid(lib):
-    assert lib.smr_reduce_num_blocks(8192, 0) == 4          # 1024 slots / 256 threads
+    assert lib.smr_reduce_num_blocks(8192, 0) == 2          # 1024 slots / 512 threads
     assert lib.smr_reduce_num_blocks(8, 0) == 1
-    assert lib.smr_reduce_num_blocks(1 << 25, 0) == 2048    # capped
+    assert lib.smr_reduce_num_blocks(1 << 25, 0) == 256     # capped: one workgroup per compute unit
     assert lib.smr_reduce_num_blocks(0, 0) == 0
-    assert lib.smr_reduce_num_blocks(4096, 1) == 4
+    assert lib.smr_reduce_num_blocks(4096, 1) == 2
+    assert lib.smr_set_reduce_launch(256, 2048) == 0        # tuning knob
+    assert lib.smr_reduce_num_blocks(1 << 25, 0) == 2048
+    assert lib.smr_set_reduce_launch(100, 0) == -1
+    assert lib.smr_set_reduce_launch(0, 0) == 0
+    assert lib.smr_reduce_num_blocks(1 << 25, 0) == 256
 
 
 def test_reduce_argument_errors_before_launch(lib):

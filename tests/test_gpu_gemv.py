@@ -35,35 +35,48 @@ def _within_one_ulp(got, ref, term_sum):
     return np.all(np.abs(got - ref) <= tol)
 
 
+@pytest.fixture(params=[(0, 0), (64, 0), (64, 3)], ids=["default", "wide", "wide-3sub"])
+def launch_shape(request, lib):
+    tpr, sub = request.param
+    assert lib.smr_set_gemv_launch(tpr, sub) == 0
+    yield request.param
+    lib.smr_set_gemv_launch(0, 0)
+
+
 @pytest.mark.parametrize("batch,K,N,ws", [(1, 512, 128, 8), (4, 1024, 256, 8), (8, 2048, 1000, 8),
                                           (3, 768, 136, 4), (8, 8192, 384, 8), (5, 16384, 128, 8)])
-def test_gemv_parity(cuda, batch, K, N, ws):
+def test_gemv_parity(cuda, launch_shape, batch, K, N, ws):
     from symm_mem_recipes import gemv_all_reduce, GemvWorkspace
     x_bits = O.seeded_normal_bf16_bits(batch * K, seed=0).reshape(batch, K)
     w_bits = O.seeded_normal_bf16_bits(K * N, seed=1, std=0.02).reshape(K, N)
     x = _bits_t(x_bits).to(cuda)
     w = _bits_t(w_bits).to(cuda)
-    wsp = GemvWorkspace(batch, N, ws, cuda)
+    wsp = GemvWorkspace(batch, N, ws, cuda, K)
+    senders = wsp.senders
+    assert senders % ws == 0
+    sub = senders // ws                     # the kernel may cut a rank's K shard into sub-shards
     want, want_partials = O.gemv_allreduce_ref(x_bits, w_bits, ws, return_partials=True)
     for _ in range(2):                      # second call: flags must have returned to zero
         out = gemv_all_reduce(x, w, ws, wsp)
         wsp.check_status()
         assert int(wsp.flags.abs().sum().item()) == 0
-        got_p = wsp.partials.cpu().numpy()
+        got_p = wsp.partials.cpu().numpy()[:senders]
+        per_rank = got_p.reshape(ws, sub, batch, N).astype(np.float64).sum(axis=1)
         xf = np.abs(O.bf16_bits_to_f32(x_bits)).astype(np.float64)
         wf = np.abs(O.bf16_bits_to_f32(w_bits)).astype(np.float64)
         ks = K // ws
         for r in range(ws):
             bound = 1e-5 * (xf[:, r * ks:(r + 1) * ks] @ wf[r * ks:(r + 1) * ks]) + 1e-30
-            assert np.all(np.abs(got_p[r].astype(np.float64) - want_partials[r]) <= bound)
+            assert np.all(np.abs(per_rank[r] - want_partials[r]) <= bound)
         got = O.bf16_bits_to_f32(_t_bits(out)).astype(np.float64)
         ref = O.bf16_bits_to_f32(want).astype(np.float64)
         assert _within_one_ulp(got, ref, xf @ wf)
         rms = np.sqrt(np.mean(ref ** 2))
         assert np.all(np.abs(got - ref) <= 1e-2 * np.abs(ref) + 1e-2 * rms)
-        # the combine itself is exact: rank-ordered fp32 sum of the kernel's own partials
+        # the combine itself is exact: fp32 sum of the kernel's own partials in sender
+        # order (rank-major)
         acc = np.zeros_like(got_p[0])
-        for r in range(ws):
+        for r in range(senders):
             acc = (acc + got_p[r]).astype(np.float32)
         assert np.array_equal(_t_bits(out), O.f32_to_bf16_bits(acc))
 
@@ -78,7 +91,7 @@ def test_gemv_config4_full_size(cuda):
     want = O.gemv_allreduce_ref(x_bits, w_bits, 8)
     terms = np.abs(O.bf16_bits_to_f32(x_bits)).astype(np.float64) @ np.abs(O.bf16_bits_to_f32(w_bits)).astype(np.float64)
     for batch in (1, 4, 8):
-        wsp = GemvWorkspace(batch, N, 8, cuda)
+        wsp = GemvWorkspace(batch, N, 8, cuda, K)
         out = gemv_all_reduce(x[:batch].contiguous(), w, 8, wsp)
         wsp.check_status()
         got = O.bf16_bits_to_f32(_t_bits(out)).astype(np.float64)
