@@ -153,6 +153,12 @@ int smr_all_gather_with_progress(const uint64_t* buffer_ptrs_dev, void* a_out_de
                                  int world_size, int64_t shard_bytes, int splits_per_rank,
                                  int num_workgroups, void* stream);
 
+/* Pacing of the producer: the first `fast_chunks` chunks are copied by all
+ * workgroups, the remaining ones by `slow_workgroups` of them (0 = all, i.e. no
+ * pacing).  Default 2 and 12.  No reference counterpart (copy engines pace
+ * themselves by link speed). */
+int smr_set_gather_pacing(int fast_chunks, int slow_workgroups);
+
 /* Flag-gated bf16 GEMM.  Replaces matmul_kernel_tma_persistent and its launch
  * (symm_mem_recipes/triton_all_gather_matmul.py:98-193, :287-315).
  *   C[M,N] = A[M,K] * B[N,K]^T, fp32 accumulate, bf16 output, all row-major.

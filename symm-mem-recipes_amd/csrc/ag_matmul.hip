@@ -42,44 +42,77 @@ struct GemmSchedule {
   int rank, world_size, comm_block_m;
   int BM, BN;
   int grid;                      // persistent workgroups, a multiple of 8
+  // The comm blocks are visited in ring order starting at the local one.  The
+  // first `head` and the last `tail` ring positions (0 or 1 each) are cut into
+  // tiles of half the width: a pass over half tiles takes half as long, so with the
+  // local comm block in halves every workgroup starts on rows that need no flag,
+  // and the producer gets that half pass as a head start.
+  int head, tail;
 };
 
 struct TileRef {
   int row0, col0;                // output tile origin
+  int cols;                      // tile width: BN or BN / 2
   int comm_block;                // progress flag index
   int local;                     // rows come from the local shard, no wait
   int a_row;                     // first row inside the source (shard-relative when local)
 };
 
+__host__ __device__ inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
+
 // Tile visited by workgroup `wg` in its `step`-th trip; false when it has no more work.
+// Three phases: `head` ring positions in half tiles, the middle in full tiles, `tail`
+// in half tiles.  A phase is walked in passes of `grid` tiles; within a pass XCD x
+// (workgroups with id % 8 == x) takes a contiguous run of the tile order.  The tile
+// order inside a phase is comm block (ring order), then column tile, then row tile.
 __host__ __device__ inline bool tile_for(const GemmSchedule& s, int wg, int step, TileRef& t) {
-  const int tn = (s.N + s.BN - 1) / s.BN;
   const int cb_tiles_m = s.comm_block_m / s.BM;
   const int n_comm = s.M / s.comm_block_m;
   const int per_rank = n_comm / s.world_size;
-  const int tiles_per_cb = cb_tiles_m * tn;
-  const int total = n_comm * tiles_per_cb;
-  const int start = step * s.grid;
-  if (start >= total) return false;
-  const int cnt = (total - start) < s.grid ? (total - start) : s.grid;
-  const int per_xcd = (cnt + 7) >> 3;
-  const int slot = wg >> 3;
-  if (slot >= per_xcd) return false;
-  const int in_pass = (wg & 7) * per_xcd + slot;
-  if (in_pass >= cnt) return false;
-  const int lin = start + in_pass;
-  const int ring_pos = lin / tiles_per_cb;
-  const int rem = lin - ring_pos * tiles_per_cb;
-  const int tile_n = rem / cb_tiles_m;
-  const int tile_m = rem - tile_n * cb_tiles_m;
   const int first_local = s.rank * per_rank;
-  const int cb = (first_local + ring_pos) % n_comm;
-  t.comm_block = cb;
-  t.row0 = cb * s.comm_block_m + tile_m * s.BM;
-  t.col0 = tile_n * s.BN;
-  t.local = (cb / per_rank) == s.rank;
-  t.a_row = t.local ? t.row0 - first_local * s.comm_block_m : t.row0;
-  return true;
+  int ring0 = 0;                                   // first ring position of the phase
+  for (int phase = 0; phase < 3; ++phase) {
+    const int positions = phase == 0 ? s.head : (phase == 1 ? n_comm - s.head - s.tail : s.tail);
+    const int bn = phase == 1 ? s.BN : s.BN / 2;
+    const int tn = ceil_div(s.N, bn);
+    const int tiles_per_cb = cb_tiles_m * tn;
+    const int total = positions * tiles_per_cb;
+    const int passes = ceil_div(total, s.grid);
+    if (step < passes) {
+      const int start = step * s.grid;
+      const int cnt = (total - start) < s.grid ? (total - start) : s.grid;
+      const int per_xcd = (cnt + 7) >> 3;
+      const int slot = wg >> 3;
+      if (slot >= per_xcd) return false;
+      const int in_pass = (wg & 7) * per_xcd + slot;
+      if (in_pass >= cnt) return false;
+      const int lin = start + in_pass;
+      const int pos = lin / tiles_per_cb;
+      const int rem = lin - pos * tiles_per_cb;
+      const int tile_n = rem / cb_tiles_m;
+      const int tile_m = rem - tile_n * cb_tiles_m;
+      const int cb = (first_local + ring0 + pos) % n_comm;
+      t.comm_block = cb;
+      t.row0 = cb * s.comm_block_m + tile_m * s.BM;
+      t.col0 = tile_n * bn;
+      t.cols = bn;
+      t.local = (cb / per_rank) == s.rank;
+      t.a_row = t.local ? t.row0 - first_local * s.comm_block_m : t.row0;
+      return true;
+    }
+    step -= passes;
+    ring0 += positions;
+  }
+  return false;
+}
+
+// Number of trips of the busiest workgroup, in units of half a full-tile pass.
+__host__ __device__ inline int schedule_cost(const GemmSchedule& s) {
+  const int cb_tiles_m = s.comm_block_m / s.BM;
+  const int n_comm = s.M / s.comm_block_m;
+  const int full = cb_tiles_m * ceil_div(s.N, s.BN), half = cb_tiles_m * ceil_div(s.N, s.BN / 2);
+  return ceil_div(s.head * half, s.grid) + 2 * ceil_div((n_comm - s.head - s.tail) * full, s.grid) +
+         ceil_div(s.tail * half, s.grid);
 }
 
 // Position swizzle of an LDS row.
@@ -137,266 +170,299 @@ struct GemmTile {
 // How many stages ahead of its real load a K-slab is touched to pull it into L2.
 constexpr int kWarmAhead = 3;
 
+// Everything a tile needs that does not depend on the tile shape.
+struct TileContext {
+  int lane, wave;
+  uint32_t row_stride;           // bytes between rows of A and of B
+  int nk;                        // K-slabs
+  uint32_t lds0;                 // LDS byte offset of the tile buffer
+  int N;
+  uint8_t* c;
+  uint64_t* tr;                  // trace record of this tile or null
+};
+
+// One output tile: C[row0 .. +BM, col0 .. +BN] = A rows (at a_base) x B rows (at b_base)^T.
+template <int BM, int BN>
+__device__ __forceinline__ void run_tile(const TileContext& cx, const TileRef& tile,
+                                         const uint8_t* a_base, const uint8_t* b_base,
+                                         uint32_t& warm_scrap) {
+  using T = GemmTile<BM, BN>;
+  constexpr int WM = T::WM, WN = T::WN, FM = T::FM, FN = T::FN, GA = T::GA, GB = T::GB;
+  constexpr int kWarmLoads = GA / 8 + GB / 8;      // warm-up loads per wave and stage
+  const int lane = cx.lane, wave = cx.wave;
+  const int wm = wave >> 1, wn = wave & 1;
+  const int half = lane >> 5;
+  const uint32_t row_stride = cx.row_stride;
+  const int nk = cx.nk;
+  const uint32_t lds0 = cx.lds0;
+  uint64_t* tr = cx.tr;
+  uint8_t* c = cx.c;
+  struct { int N; } s = {cx.N};
+
+  // The per-lane addresses below are recomputed for every tile from a laundered
+  // copy of the lane id: kept loop-invariant they would stay live across the
+  // register-hungry epilogue, be spilled there, and be reloaded from scratch
+  // in the middle of the K loop.
+  int ln = lane;
+  asm volatile("" : "+v"(ln));
+  // ---- per-lane fragment read addresses (stage 0).  Row r = w*W + f*32 + (ln & 31)
+  // has swizzle ((lane & 7) ^ ((ln >> 3) & 3)) ^ ((f & 1) << 2); K step kk wants
+  // chunk 2*kk + half.  Hence position = t ^ (v << 1) with the per-lane constant
+  // t = half ^ (lane & 7) ^ ((ln >> 3) & 3) and v = kk ^ ((f & 1) << 1): four
+  // variants per operand, everything else is an immediate offset.
+  const int t = (ln >> 5) ^ (ln & 7) ^ ((ln >> 3) & 3);
+  uint32_t a_fr[4], b_fr[4];
+#pragma unroll
+  for (int v = 0; v < 4; ++v) {
+    a_fr[v] = lds0 + (uint32_t)((wm * WM + (ln & 31)) * kRowBytes + ((t ^ (v << 1)) << 4));
+    b_fr[v] = lds0 + T::kBBase + (uint32_t)((wn * WN + (ln & 31)) * kRowBytes + ((t ^ (v << 1)) << 4));
+  }
+
+  // ---- per-lane global offsets of the tile loads.  Load group q = wave*G + j holds
+  // rows q*8 .. q*8+7; lane l carries row q*8 + (l >> 3) and the chunk whose swizzled
+  // position is (l & 7): chunk = (l & 7) ^ (l >> 3) ^ (q & 7).
+  const int u = (ln & 7) ^ (ln >> 3);
+  uint32_t a_off[GA];
+#pragma unroll
+  for (int j = 0; j < GA; ++j) {
+    const int q = wave * GA + j;
+    a_off[j] = (uint32_t)(q * 8 + (ln >> 3)) * row_stride + (uint32_t)((u ^ (q & 7)) << 4);
+  }
+
+  // ---- L2 warm-up: one dword per 128-byte row segment, 64 rows per wave instruction
+  uint32_t a_warm[GA / 8 > 0 ? GA / 8 : 1];
+#pragma unroll
+  for (int j = 0; j < GA / 8; ++j) a_warm[j] = (uint32_t)(wave * (GA * 8) + j * 64 + ln) * row_stride;
+
+    // rows of B past the last column are clamped: they feed outputs that are never stored
+  const int b_last = s.N - 1 - tile.col0;
+  uint32_t b_off[GB];
+#pragma unroll
+  for (int j = 0; j < GB; ++j) {
+    const int q = wave * GB + j;
+    int r = q * 8 + (ln >> 3);
+    r = r < b_last ? r : b_last;
+    b_off[j] = (uint32_t)r * row_stride + (uint32_t)((u ^ (q & 7)) << 4);
+  }
+
+  uint32_t b_warm[GB / 8 > 0 ? GB / 8 : 1];
+#pragma unroll
+  for (int j = 0; j < GB / 8; ++j) {
+    int r = wave * (GB * 8) + j * 64 + ln;
+    r = r < b_last ? r : b_last;
+    b_warm[j] = (uint32_t)r * row_stride;
+  }
+
+  f32x16 acc[FN][FM];
+#pragma unroll
+  for (int ni = 0; ni < FN; ++ni)
+#pragma unroll
+    for (int mi = 0; mi < FM; ++mi)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[ni][mi][e] = 0.0f;
+
+  auto load_stage = [&](int stage, int kt) {
+    const uint8_t* ak = a_base + (int64_t)kt * kRowBytes;
+    const uint8_t* bk = b_base + (int64_t)kt * kRowBytes;
+    const uint32_t la = lds0 + stage * T::kABytes + wave * (GA * 1024);
+    const uint32_t lb = lds0 + T::kBBase + stage * T::kBBytes + wave * (GB * 1024);
+#pragma unroll
+    for (int j = 0; j < GA; ++j) load_group(ak, a_off[j], la + j * 1024);
+#pragma unroll
+    for (int j = 0; j < GB; ++j) load_group(bk, b_off[j], lb + j * 1024);
+  };
+  // Touch the K-slab of stage kt (one dword per row) so that its real load,
+  // kWarmAhead stages later, finds the lines in L2.  The loaded dwords go to a
+  // scrap register that is never read for its value.  Inline assembly on
+  // purpose: the compiler must not count these loads, or it would make the wave
+  // wait for them - they are meant to miss - before the next fragment reads.
+  // `warm_scrap` is threaded through every statement and consumed after the
+  // tile loop, so its register stays reserved while loads into it are in flight.
+  auto warm_stage = [&](int kt) {
+    const uint8_t* ak = a_base + (int64_t)kt * kRowBytes;
+    const uint8_t* bk = b_base + (int64_t)kt * kRowBytes;
+#pragma unroll
+    for (int j = 0; j < GA / 8; ++j)
+      asm volatile("global_load_dword %0, %1, %2" : "+v"(warm_scrap) : "v"(a_warm[j]), "s"(ak) : "memory");
+#pragma unroll
+    for (int j = 0; j < GB / 8; ++j)
+      asm volatile("global_load_dword %0, %1, %2" : "+v"(warm_scrap) : "v"(b_warm[j]), "s"(bk) : "memory");
+  };
+  auto read_frags = [&](bf16x8 (&af)[FM], bf16x8 (&bf)[FN], int stage, int kk) {
+#pragma unroll
+    for (int mi = 0; mi < FM; ++mi)
+      af[mi] = lds_read_frag(a_fr[kk ^ ((mi & 1) << 1)] + stage * T::kABytes + mi * (32 * kRowBytes));
+#pragma unroll
+    for (int ni = 0; ni < FN; ++ni)
+      bf[ni] = lds_read_frag(b_fr[kk ^ ((ni & 1) << 1)] + stage * T::kBBytes + ni * (32 * kRowBytes));
+  };
+  auto mfma_all = [&](const bf16x8 (&af)[FM], const bf16x8 (&bf)[FN]) {
+#pragma unroll
+    for (int ni = 0; ni < FN; ++ni)
+#pragma unroll
+      for (int mi = 0; mi < FM; ++mi)
+        acc[ni][mi] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bf[ni], af[mi], acc[ni][mi], 0, 0, 0);
+  };
+
+  // Prologue: both LDS stages in flight, then the first fragments.
+  load_stage(0, 0);
+  if (nk > 1) load_stage(1, 1);
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();
+#pragma unroll
+  for (int w = 0; w < kWarmAhead; ++w) warm_stage(2 + w < nk ? 2 + w : nk - 1);
+
+  // Fragment double buffer: while the MFMAs of K step kk run, the fragments of
+  // step kk+1 are read.  The workgroup barrier sits before the last K step of a
+  // stage, right after that stage's last fragment reads: from there on the stage
+  // is free, so the loads of stage kt+2 are issued into it and have a whole stage
+  // of MFMAs to land, and the first fragments of stage kt+1 are read under the
+  // MFMAs of the last K step.
+  bf16x8 af0[FM], bf0[FN], af1[FM], bf1[FN];
+  read_frags(af0, bf0, 0, 0);
+
+  // Last K step of a stage, issued right behind the barrier.  Its fragments are
+  // already in registers, so the MFMAs can start at once; the loads of stage
+  // kt+2, the first fragment reads of stage kt+1 and the warm-up touches are
+  // slotted in between them instead of standing in front of them.  There is
+  // one code path: past the end of K the loads are clamped to the last K-slab
+  // (they land in a stage nobody reads any more) rather than branched around,
+  // which keeps the accumulators in place across the whole loop body.
+  auto last_step = [&](auto stage_tag, int kt) {
+    constexpr int S = decltype(stage_tag)::value;
+    const int kl = kt + 2 < nk ? kt + 2 : nk - 1;
+    const uint8_t* ak = a_base + (int64_t)kl * kRowBytes;
+    const uint8_t* bk = b_base + (int64_t)kl * kRowBytes;
+    const uint32_t la = lds0 + S * T::kABytes + wave * (GA * 1024);
+    const uint32_t lb = lds0 + T::kBBase + S * T::kBBytes + wave * (GB * 1024);
+    constexpr int kMfma = FM * FN, kLoads = GA + GB, kReads = FM + FN;
+    // loads are spread over all MFMAs, fragment reads over the later ones
+    constexpr int kReadFrom = kMfma >= 2 * kReads ? kMfma / 4 : 0;
+    // (all loops below have constant trip counts so that they unroll fully and
+    // every array index is a compile-time constant)
+#pragma unroll
+    for (int ni = 0; ni < FN; ++ni) {
+#pragma unroll
+      for (int mi = 0; mi < FM; ++mi) {
+        const int slot = ni * FM + mi;
+        acc[ni][mi] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bf1[ni], af1[mi], acc[ni][mi], 0, 0, 0);
+#pragma unroll
+        for (int g = 0; g < GA; ++g)
+          if (g * kMfma / kLoads == slot) load_group(ak, a_off[g], la + g * 1024);
+#pragma unroll
+        for (int g = 0; g < GB; ++g)
+          if ((GA + g) * kMfma / kLoads == slot) load_group(bk, b_off[g], lb + g * 1024);
+#pragma unroll
+        for (int r = 0; r < FM; ++r)
+          if (kReadFrom + r * (kMfma - kReadFrom) / kReads == slot)
+            af0[r] = lds_read_frag(a_fr[(r & 1) << 1] + (S ^ 1) * T::kABytes + r * (32 * kRowBytes));
+#pragma unroll
+        for (int r = 0; r < FN; ++r)
+          if (kReadFrom + (FM + r) * (kMfma - kReadFrom) / kReads == slot)
+            bf0[r] = lds_read_frag(b_fr[(r & 1) << 1] + (S ^ 1) * T::kBBytes + r * (32 * kRowBytes));
+        if (slot == kMfma - 1) {
+          const int kw = kt + 2 + kWarmAhead;
+          warm_stage(kw < nk ? kw : nk - 1);
+        }
+      }
+    }
+  };
+  auto stage_body = [&](auto stage_tag, int kt) {
+    constexpr int S = decltype(stage_tag)::value;
+    read_frags(af1, bf1, S, 1);
+    mfma_all(af0, bf0);
+    interleave_mfma_dsread<FM * FN, FM + FN>();
+    read_frags(af0, bf0, S, 2);
+    mfma_all(af1, bf1);
+    interleave_mfma_dsread<FM * FN, FM + FN>();
+    read_frags(af1, bf1, S, 3);
+    mfma_all(af0, bf0);
+    interleave_mfma_dsread<FM * FN, FM + FN>();
+    // Wait for this wave's own tile loads before the barrier; the compiler does
+    // not count them (see load_group).  The kWarmLoads warm-up loads issued
+    // behind them may stay in flight: loads return in order.
+    if constexpr (kWarmLoads == 0) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    else if constexpr (kWarmLoads == 1) asm volatile("s_waitcnt vmcnt(1)" ::: "memory");
+    else asm volatile("s_waitcnt vmcnt(2)" ::: "memory");
+    __syncthreads();     // stage S fully read by everyone; the other stage has landed
+    last_step(stage_tag, kt);
+  };
+  int kt = 0;
+  for (; kt + 1 < nk; kt += 2) {
+    stage_body(std::integral_constant<int, 0>{}, kt);
+    stage_body(std::integral_constant<int, 1>{}, kt + 1);
+  }
+  if (kt < nk) stage_body(std::integral_constant<int, 0>{}, kt);
+  __syncthreads();       // the next tile's prologue overwrites both stages
+  if (tr != nullptr) tr[2] = wall_clock64();
+
+  // D[n][m]: lane holds row m = lane & 31 and, per group of 4 registers, the 4
+  // consecutive columns g*8 + (lane >> 5)*4 .. +3 of the 32x32 fragment.
+#pragma unroll
+  for (int mi = 0; mi < FM; ++mi) {
+    const int m = tile.row0 + wm * WM + mi * 32 + (lane & 31);
+    uint8_t* c_row = c + ((int64_t)m * s.N) * 2;
+#pragma unroll
+    for (int ni = 0; ni < FN; ++ni) {
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const int n = tile.col0 + wn * WN + ni * 32 + g * 8 + half * 4;
+        if (n < s.N) {
+          uint2 v;
+          v.x = pack_bf16x2(acc[ni][mi][g * 4 + 0], acc[ni][mi][g * 4 + 1]);
+          v.y = pack_bf16x2(acc[ni][mi][g * 4 + 2], acc[ni][mi][g * 4 + 3]);
+          *reinterpret_cast<uint2*>(c_row + (int64_t)n * 2) = v;
+        }
+      }
+      // one fragment at a time: keeps the accumulator read-out from flooding
+      // the vector registers
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  }
+}
+
 template <int BM, int BN>
 __global__ __launch_bounds__(kGemmThreads, 1) void ag_matmul_kernel(
     const uint8_t* __restrict__ a_shard, const uint8_t* __restrict__ a_out,
     const uint8_t* __restrict__ b_nk, uint8_t* __restrict__ c, const uint32_t* __restrict__ progress,
     GemmSchedule s, uint64_t limit_ticks, uint32_t* status, uint64_t* trace) {
-  using T = GemmTile<BM, BN>;
-  constexpr int WM = T::WM, WN = T::WN, FM = T::FM, FN = T::FN, GA = T::GA, GB = T::GB;
-  constexpr int kWarmLoads = GA / 8 + GB / 8;      // warm-up loads per wave and stage
-  __shared__ __attribute__((aligned(1024))) uint8_t lds[T::kLdsBytes];
+  __shared__ __attribute__((aligned(1024))) uint8_t lds[GemmTile<BM, BN>::kLdsBytes];
 
-  const int lane = threadIdx.x & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int wm = wave >> 1, wn = wave & 1;
-  const int half = lane >> 5;
-  const uint32_t row_stride = (uint32_t)s.K * 2u;
-  const int nk = s.K / kBK;
-  const uint32_t lds0 = lds_offset_of(lds);
-
+  TileContext cx;
+  cx.lane = threadIdx.x & 63;
+  cx.wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  cx.row_stride = (uint32_t)s.K * 2u;
+  cx.nk = s.K / kBK;
+  cx.lds0 = lds_offset_of(lds);
+  cx.N = s.N;
+  cx.c = c;
   uint32_t warm_scrap = 0;
 
   for (int step = 0;; ++step) {
     TileRef tile;
     if (!tile_for(s, blockIdx.x, step, tile)) break;
-
-    // The per-lane addresses below are recomputed for every tile from a laundered
-    // copy of the lane id: kept loop-invariant they would stay live across the
-    // register-hungry epilogue, be spilled there, and be reloaded from scratch
-    // in the middle of the K loop.
-    int ln = lane;
-    asm volatile("" : "+v"(ln));
-    // ---- per-lane fragment read addresses (stage 0).  Row r = w*W + f*32 + (ln & 31)
-    // has swizzle ((lane & 7) ^ ((ln >> 3) & 3)) ^ ((f & 1) << 2); K step kk wants
-    // chunk 2*kk + half.  Hence position = t ^ (v << 1) with the per-lane constant
-    // t = half ^ (lane & 7) ^ ((ln >> 3) & 3) and v = kk ^ ((f & 1) << 1): four
-    // variants per operand, everything else is an immediate offset.
-    const int t = (ln >> 5) ^ (ln & 7) ^ ((ln >> 3) & 3);
-    uint32_t a_fr[4], b_fr[4];
-  #pragma unroll
-    for (int v = 0; v < 4; ++v) {
-      a_fr[v] = lds0 + (uint32_t)((wm * WM + (ln & 31)) * kRowBytes + ((t ^ (v << 1)) << 4));
-      b_fr[v] = lds0 + T::kBBase + (uint32_t)((wn * WN + (ln & 31)) * kRowBytes + ((t ^ (v << 1)) << 4));
-    }
-
-    // ---- per-lane global offsets of the tile loads.  Load group q = wave*G + j holds
-    // rows q*8 .. q*8+7; lane l carries row q*8 + (l >> 3) and the chunk whose swizzled
-    // position is (l & 7): chunk = (l & 7) ^ (l >> 3) ^ (q & 7).
-    const int u = (ln & 7) ^ (ln >> 3);
-    uint32_t a_off[GA];
-  #pragma unroll
-    for (int j = 0; j < GA; ++j) {
-      const int q = wave * GA + j;
-      a_off[j] = (uint32_t)(q * 8 + (ln >> 3)) * row_stride + (uint32_t)((u ^ (q & 7)) << 4);
-    }
-
-    // ---- L2 warm-up: one dword per 128-byte row segment, 64 rows per wave instruction
-    uint32_t a_warm[GA / 8 > 0 ? GA / 8 : 1];
-  #pragma unroll
-    for (int j = 0; j < GA / 8; ++j) a_warm[j] = (uint32_t)(wave * (GA * 8) + j * 64 + ln) * row_stride;
-
-    uint64_t* tr = nullptr;
+    cx.tr = nullptr;
     if (trace != nullptr && step < kTraceSteps && blockIdx.x < 256 && threadIdx.x == 0) {
-      tr = trace + kTraceProducerWords + ((size_t)blockIdx.x * kTraceSteps + step) * 4;
-      tr[0] = wall_clock64();
+      cx.tr = trace + kTraceProducerWords + ((size_t)blockIdx.x * kTraceSteps + step) * 4;
+      cx.tr[0] = wall_clock64();
     }
     const uint8_t* a_base;
     if (tile.local) {
-      a_base = a_shard + (int64_t)tile.a_row * row_stride;
+      a_base = a_shard + (int64_t)tile.a_row * cx.row_stride;
     } else {
       if (progress != nullptr)
         wait_signal(progress + tile.comm_block, limit_ticks, status, tile.comm_block);
-      a_base = a_out + (int64_t)tile.a_row * row_stride;
+      a_base = a_out + (int64_t)tile.a_row * cx.row_stride;
     }
-    if (tr != nullptr) tr[1] = wall_clock64();
-    const uint8_t* b_base = b_nk + (int64_t)tile.col0 * row_stride;
-    // rows of B past the last column are clamped: they feed outputs that are never stored
-    const int b_last = s.N - 1 - tile.col0;
-    uint32_t b_off[GB];
-#pragma unroll
-    for (int j = 0; j < GB; ++j) {
-      const int q = wave * GB + j;
-      int r = q * 8 + (ln >> 3);
-      r = r < b_last ? r : b_last;
-      b_off[j] = (uint32_t)r * row_stride + (uint32_t)((u ^ (q & 7)) << 4);
+    if (cx.tr != nullptr) cx.tr[1] = wall_clock64();
+    const uint8_t* b_base = b_nk + (int64_t)tile.col0 * cx.row_stride;
+    if constexpr (BN == 256) {
+      if (tile.cols != BN) run_tile<BM, BN / 2>(cx, tile, a_base, b_base, warm_scrap);
+      else run_tile<BM, BN>(cx, tile, a_base, b_base, warm_scrap);
+    } else {
+      run_tile<BM, BN>(cx, tile, a_base, b_base, warm_scrap);
     }
-
-    uint32_t b_warm[GB / 8 > 0 ? GB / 8 : 1];
-#pragma unroll
-    for (int j = 0; j < GB / 8; ++j) {
-      int r = wave * (GB * 8) + j * 64 + ln;
-      r = r < b_last ? r : b_last;
-      b_warm[j] = (uint32_t)r * row_stride;
-    }
-
-    f32x16 acc[FN][FM];
-#pragma unroll
-    for (int ni = 0; ni < FN; ++ni)
-#pragma unroll
-      for (int mi = 0; mi < FM; ++mi)
-#pragma unroll
-        for (int e = 0; e < 16; ++e) acc[ni][mi][e] = 0.0f;
-
-    auto load_stage = [&](int stage, int kt) {
-      const uint8_t* ak = a_base + (int64_t)kt * kRowBytes;
-      const uint8_t* bk = b_base + (int64_t)kt * kRowBytes;
-      const uint32_t la = lds0 + stage * T::kABytes + wave * (GA * 1024);
-      const uint32_t lb = lds0 + T::kBBase + stage * T::kBBytes + wave * (GB * 1024);
-#pragma unroll
-      for (int j = 0; j < GA; ++j) load_group(ak, a_off[j], la + j * 1024);
-#pragma unroll
-      for (int j = 0; j < GB; ++j) load_group(bk, b_off[j], lb + j * 1024);
-    };
-    // Touch the K-slab of stage kt (one dword per row) so that its real load,
-    // kWarmAhead stages later, finds the lines in L2.  The loaded dwords go to a
-    // scrap register that is never read for its value.  Inline assembly on
-    // purpose: the compiler must not count these loads, or it would make the wave
-    // wait for them - they are meant to miss - before the next fragment reads.
-    // `warm_scrap` is threaded through every statement and consumed after the
-    // tile loop, so its register stays reserved while loads into it are in flight.
-    auto warm_stage = [&](int kt) {
-      const uint8_t* ak = a_base + (int64_t)kt * kRowBytes;
-      const uint8_t* bk = b_base + (int64_t)kt * kRowBytes;
-#pragma unroll
-      for (int j = 0; j < GA / 8; ++j)
-        asm volatile("global_load_dword %0, %1, %2" : "+v"(warm_scrap) : "v"(a_warm[j]), "s"(ak) : "memory");
-#pragma unroll
-      for (int j = 0; j < GB / 8; ++j)
-        asm volatile("global_load_dword %0, %1, %2" : "+v"(warm_scrap) : "v"(b_warm[j]), "s"(bk) : "memory");
-    };
-    auto read_frags = [&](bf16x8 (&af)[FM], bf16x8 (&bf)[FN], int stage, int kk) {
-#pragma unroll
-      for (int mi = 0; mi < FM; ++mi)
-        af[mi] = lds_read_frag(a_fr[kk ^ ((mi & 1) << 1)] + stage * T::kABytes + mi * (32 * kRowBytes));
-#pragma unroll
-      for (int ni = 0; ni < FN; ++ni)
-        bf[ni] = lds_read_frag(b_fr[kk ^ ((ni & 1) << 1)] + stage * T::kBBytes + ni * (32 * kRowBytes));
-    };
-    auto mfma_all = [&](const bf16x8 (&af)[FM], const bf16x8 (&bf)[FN]) {
-#pragma unroll
-      for (int ni = 0; ni < FN; ++ni)
-#pragma unroll
-        for (int mi = 0; mi < FM; ++mi)
-          acc[ni][mi] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bf[ni], af[mi], acc[ni][mi], 0, 0, 0);
-    };
-
-    // Prologue: both LDS stages in flight, then the first fragments.
-    load_stage(0, 0);
-    if (nk > 1) load_stage(1, 1);
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    __syncthreads();
-#pragma unroll
-    for (int w = 0; w < kWarmAhead; ++w) warm_stage(2 + w < nk ? 2 + w : nk - 1);
-
-    // Fragment double buffer: while the MFMAs of K step kk run, the fragments of
-    // step kk+1 are read.  The workgroup barrier sits before the last K step of a
-    // stage, right after that stage's last fragment reads: from there on the stage
-    // is free, so the loads of stage kt+2 are issued into it and have a whole stage
-    // of MFMAs to land, and the first fragments of stage kt+1 are read under the
-    // MFMAs of the last K step.
-    bf16x8 af0[FM], bf0[FN], af1[FM], bf1[FN];
-    read_frags(af0, bf0, 0, 0);
-
-    // Last K step of a stage, issued right behind the barrier.  Its fragments are
-    // already in registers, so the MFMAs can start at once; the loads of stage
-    // kt+2, the first fragment reads of stage kt+1 and the warm-up touches are
-    // slotted in between them instead of standing in front of them.  There is
-    // one code path: past the end of K the loads are clamped to the last K-slab
-    // (they land in a stage nobody reads any more) rather than branched around,
-    // which keeps the accumulators in place across the whole loop body.
-    auto last_step = [&](auto stage_tag, int kt) {
-      constexpr int S = decltype(stage_tag)::value;
-      const int kl = kt + 2 < nk ? kt + 2 : nk - 1;
-      const uint8_t* ak = a_base + (int64_t)kl * kRowBytes;
-      const uint8_t* bk = b_base + (int64_t)kl * kRowBytes;
-      const uint32_t la = lds0 + S * T::kABytes + wave * (GA * 1024);
-      const uint32_t lb = lds0 + T::kBBase + S * T::kBBytes + wave * (GB * 1024);
-      constexpr int kMfma = FM * FN, kLoads = GA + GB, kReads = FM + FN;
-      // loads are spread over all MFMAs, fragment reads over the later ones
-      constexpr int kReadFrom = kMfma >= 2 * kReads ? kMfma / 4 : 0;
-      // (all loops below have constant trip counts so that they unroll fully and
-      // every array index is a compile-time constant)
-#pragma unroll
-      for (int ni = 0; ni < FN; ++ni) {
-#pragma unroll
-        for (int mi = 0; mi < FM; ++mi) {
-          const int slot = ni * FM + mi;
-          acc[ni][mi] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bf1[ni], af1[mi], acc[ni][mi], 0, 0, 0);
-#pragma unroll
-          for (int g = 0; g < GA; ++g)
-            if (g * kMfma / kLoads == slot) load_group(ak, a_off[g], la + g * 1024);
-#pragma unroll
-          for (int g = 0; g < GB; ++g)
-            if ((GA + g) * kMfma / kLoads == slot) load_group(bk, b_off[g], lb + g * 1024);
-#pragma unroll
-          for (int r = 0; r < FM; ++r)
-            if (kReadFrom + r * (kMfma - kReadFrom) / kReads == slot)
-              af0[r] = lds_read_frag(a_fr[(r & 1) << 1] + (S ^ 1) * T::kABytes + r * (32 * kRowBytes));
-#pragma unroll
-          for (int r = 0; r < FN; ++r)
-            if (kReadFrom + (FM + r) * (kMfma - kReadFrom) / kReads == slot)
-              bf0[r] = lds_read_frag(b_fr[(r & 1) << 1] + (S ^ 1) * T::kBBytes + r * (32 * kRowBytes));
-          if (slot == kMfma - 1) {
-            const int kw = kt + 2 + kWarmAhead;
-            warm_stage(kw < nk ? kw : nk - 1);
-          }
-        }
-      }
-    };
-    auto stage_body = [&](auto stage_tag, int kt) {
-      constexpr int S = decltype(stage_tag)::value;
-      read_frags(af1, bf1, S, 1);
-      mfma_all(af0, bf0);
-      interleave_mfma_dsread<FM * FN, FM + FN>();
-      read_frags(af0, bf0, S, 2);
-      mfma_all(af1, bf1);
-      interleave_mfma_dsread<FM * FN, FM + FN>();
-      read_frags(af1, bf1, S, 3);
-      mfma_all(af0, bf0);
-      interleave_mfma_dsread<FM * FN, FM + FN>();
-      // Wait for this wave's own tile loads before the barrier; the compiler does
-      // not count them (see load_group).  The kWarmLoads warm-up loads issued
-      // behind them may stay in flight: loads return in order.
-      if constexpr (kWarmLoads == 0) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-      else if constexpr (kWarmLoads == 1) asm volatile("s_waitcnt vmcnt(1)" ::: "memory");
-      else asm volatile("s_waitcnt vmcnt(2)" ::: "memory");
-      __syncthreads();     // stage S fully read by everyone; the other stage has landed
-      last_step(stage_tag, kt);
-    };
-    int kt = 0;
-    for (; kt + 1 < nk; kt += 2) {
-      stage_body(std::integral_constant<int, 0>{}, kt);
-      stage_body(std::integral_constant<int, 1>{}, kt + 1);
-    }
-    if (kt < nk) stage_body(std::integral_constant<int, 0>{}, kt);
-    __syncthreads();       // the next tile's prologue overwrites both stages
-    if (tr != nullptr) tr[2] = wall_clock64();
-
-    // D[n][m]: lane holds row m = lane & 31 and, per group of 4 registers, the 4
-    // consecutive columns g*8 + (lane >> 5)*4 .. +3 of the 32x32 fragment.
-#pragma unroll
-    for (int mi = 0; mi < FM; ++mi) {
-      const int m = tile.row0 + wm * WM + mi * 32 + (lane & 31);
-      uint8_t* c_row = c + ((int64_t)m * s.N) * 2;
-#pragma unroll
-      for (int ni = 0; ni < FN; ++ni) {
-#pragma unroll
-        for (int g = 0; g < 4; ++g) {
-          const int n = tile.col0 + wn * WN + ni * 32 + g * 8 + half * 4;
-          if (n < s.N) {
-            uint2 v;
-            v.x = pack_bf16x2(acc[ni][mi][g * 4 + 0], acc[ni][mi][g * 4 + 1]);
-            v.y = pack_bf16x2(acc[ni][mi][g * 4 + 2], acc[ni][mi][g * 4 + 3]);
-            *reinterpret_cast<uint2*>(c_row + (int64_t)n * 2) = v;
-          }
-        }
-        // one fragment at a time: keeps the accumulator read-out from flooding
-        // the vector registers
-        __builtin_amdgcn_sched_barrier(0);
-      }
-    }
-    if (tr != nullptr) tr[3] = wall_clock64();
+    if (cx.tr != nullptr) cx.tr[3] = wall_clock64();
   }
   // Drain the warm-up loads and give the scrap register a use the compiler
   // cannot remove (K is never negative).
@@ -461,6 +527,7 @@ static GemmSchedule make_schedule(int M, int N, int K, int rank, int world_size,
   GemmSchedule s;
   s.M = M; s.N = N; s.K = K;
   s.rank = rank; s.world_size = world_size; s.comm_block_m = comm_block_m;
+  s.head = s.tail = 0;
   pick_tile(M, N, comm_block_m, s.BM, s.BN);
   const int tn = (N + s.BN - 1) / s.BN;
   const int total = (M / s.BM) * tn;
@@ -469,7 +536,26 @@ static GemmSchedule make_schedule(int M, int N, int K, int rank, int world_size,
   const int passes = (total + max_grid - 1) / max_grid;
   const int need = ((total + passes - 1) / passes + 7) / 8 * 8;
   s.grid = need < max_grid ? need : max_grid;
+  // Gated launches: cut the local comm block (and, if that is what balances the
+  // passes, the last one too) into half-width tiles when it costs no extra time.
+  const int n_comm = M / comm_block_m;
+  if (gated && s.BN == 256 && n_comm >= 3) {
+    const int base = schedule_cost(s);
+    GemmSchedule both = s, head = s;
+    both.head = both.tail = 1;
+    head.head = 1;
+    if (schedule_cost(both) <= base) s = both;
+    else if (schedule_cost(head) <= base) s = head;
+  }
   return s;
+}
+
+static int total_steps(const GemmSchedule& s) {
+  const int cb_tiles_m = s.comm_block_m / s.BM;
+  const int n_comm = s.M / s.comm_block_m;
+  const int full = cb_tiles_m * ceil_div(s.N, s.BN), half = cb_tiles_m * ceil_div(s.N, s.BN / 2);
+  return ceil_div(s.head * half, s.grid) + ceil_div((n_comm - s.head - s.tail) * full, s.grid) +
+         ceil_div(s.tail * half, s.grid);
 }
 
 }  // namespace smr
@@ -522,11 +608,10 @@ int smr_ag_matmul_schedule(int M, int N, int K, int rank, int world_size, int co
   // host-only: the schedule of a 256-CU part, the one the kernels are tuned for
   const GemmSchedule s = make_schedule(M, N, K, rank, world_size, comm_block_m, 256, gated != 0);
   int count = 0;
+  const int steps = total_steps(s);
   for (int wg = 0; wg < s.grid; ++wg) {
-    for (int step = 0;; ++step) {
+    for (int step = 0; step < steps; ++step) {
       TileRef t;
-      const int tn = (s.N + s.BN - 1) / s.BN;
-      if (step * s.grid >= (s.M / s.BM) * tn) break;
       if (!tile_for(s, wg, step, t)) continue;
       if (out_records != nullptr && count < max_tiles) {
         int32_t* rec = out_records + (size_t)count * 8;
@@ -535,7 +620,7 @@ int smr_ag_matmul_schedule(int M, int N, int K, int rank, int world_size, int co
         rec[2] = t.row0;
         rec[3] = t.col0;
         rec[4] = s.BM;
-        rec[5] = s.BN;
+        rec[5] = t.cols;
         rec[6] = t.comm_block;
         rec[7] = t.local;
       }

@@ -9,9 +9,12 @@
 // "Last" is decided by a per-chunk arrival counter, so the flag is raised once
 // all of the chunk's bytes have been written and released.
 //
-// The grid is small on purpose: the consumer GEMM owns the compute units; the
-// producer only needs enough workgroups in flight to move 32 MiB chunks faster
-// than the GEMM consumes them.
+// The grid is small on purpose: the consumer GEMM owns the compute units.  It is
+// also paced: a copy that streams faster than about 0.25 TB/s slows the GEMM next
+// to it more than proportionally (measured: +20 % GEMM time at 0.5 TB/s, nothing
+// at 0.2 TB/s), so only the first chunks - the ones the consumer is about to ask
+// for - are copied by all workgroups; after them all but a few workgroups leave
+// and the rest of the gather trickles in just ahead of the consumer.
 #include "smr_device.hpp"
 
 namespace smr {
@@ -21,6 +24,10 @@ namespace smr {
 // whichever of the two kernels is dispatched first.
 constexpr int kGatherThreads = 1024;
 constexpr int kGatherDefaultWorkgroups = 8;
+// Pacing (smr_set_gather_pacing): chunks copied at full width, workgroups that stay
+// for the rest.
+static int g_gather_fast_chunks = 2;
+static int g_gather_slow_workgroups = 12;
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef __attribute__((address_space(1))) u32x4 GlobalVec;
@@ -28,13 +35,16 @@ typedef __attribute__((address_space(1))) u32x4 GlobalVec;
 __global__ __launch_bounds__(kGatherThreads) void all_gather_kernel(
     const uint64_t* __restrict__ buffer_ptrs, uint8_t* __restrict__ a_out,
     uint32_t* __restrict__ progress, uint32_t* __restrict__ counters, int rank, int world_size,
-    int64_t chunk_vecs, int splits_per_rank, uint64_t* trace) {
-  const int nwg = gridDim.x;
+    int64_t chunk_vecs, int splits_per_rank, uint64_t* trace, int fast_chunks, int slow_wgs) {
+  int done_chunks = 0;
   if (trace != nullptr && blockIdx.x == 0 && threadIdx.x == 0) trace[kTraceProducerWords - 1] = wall_clock64();
   for (int step = 0; step < world_size; ++step) {
     const int src_rank = (rank + step + 1) % world_size;
     for (int split = 0; split < splits_per_rank; ++split) {
       const int idx = src_rank * splits_per_rank + split;
+      // workgroups taking part in this chunk
+      const int nwg = done_chunks++ < fast_chunks ? (int)gridDim.x : slow_wgs;
+      if ((int)blockIdx.x >= nwg) continue;
       const GlobalVec* src =
           (const GlobalVec*)(uintptr_t)buffer_ptrs[src_rank] + (int64_t)split * chunk_vecs;
       GlobalVec* dst = (GlobalVec*)(uintptr_t)a_out + (int64_t)idx * chunk_vecs;
@@ -72,6 +82,14 @@ __global__ __launch_bounds__(kGatherThreads) void all_gather_kernel(
 
 }  // namespace smr
 
+extern "C" int smr_set_gather_pacing(int fast_chunks, int slow_workgroups) {
+  if (fast_chunks < 0 || slow_workgroups < 0 || slow_workgroups > 1024)
+    return smr::fail(SMR_E_INVALID, "smr_set_gather_pacing: negative or too large");
+  smr::g_gather_fast_chunks = fast_chunks;
+  smr::g_gather_slow_workgroups = slow_workgroups == 0 ? 1024 : slow_workgroups;
+  return 0;
+}
+
 extern "C" int smr_all_gather_with_progress(const uint64_t* buffer_ptrs_dev, void* a_out_dev,
                                             uint32_t* progress_dev, uint32_t* counters_dev,
                                             int rank, int world_size, int64_t shard_bytes,
@@ -93,6 +111,7 @@ extern "C" int smr_all_gather_with_progress(const uint64_t* buffer_ptrs_dev, voi
   hipLaunchKernelGGL(all_gather_kernel, dim3(nwg), dim3(kGatherThreads), 0,
                      reinterpret_cast<hipStream_t>(stream), buffer_ptrs_dev,
                      reinterpret_cast<uint8_t*>(a_out_dev), progress_dev, counters_dev, rank,
-                     world_size, chunk_bytes / 16, splits_per_rank, trace_buffer(kTraceProducerWords));
+                     world_size, chunk_bytes / 16, splits_per_rank, trace_buffer(kTraceProducerWords),
+                     g_gather_fast_chunks, g_gather_slow_workgroups < nwg ? g_gather_slow_workgroups : nwg);
   return check_hip(hipGetLastError(), "smr_all_gather_with_progress launch");
 }

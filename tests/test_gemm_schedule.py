@@ -16,35 +16,66 @@ def _by_wg(s):
     return by
 
 
+def _covers_exactly(s, M, N):
+    """The tiles are disjoint rectangles whose union is the whole output."""
+    cells = set()
+    for t in s:
+        assert t["row0"] % 128 == 0 and t["col0"] % 64 == 0
+        for r in range(t["row0"], t["row0"] + t["rows"], 128):
+            for c in range(t["col0"], min(t["col0"] + t["cols"], (N + 63) // 64 * 64), 64):
+                assert (r, c) not in cells, "tile overlap"
+                cells.add((r, c))
+    assert len(cells) == (M // 128) * ((N + 63) // 64)
+
+
 @pytest.mark.parametrize("rank", [0, 3, 7])
-def test_schedule_config5(rank):
+def test_schedule_config5_ungated(rank):
     M, N, K, ws = 16384, 3584, 8192, 8
-    s = gemm_schedule(M, N, K, rank, ws, M // ws)
+    s = gemm_schedule(M, N, K, rank, ws, M // ws, gated=False)
     assert len(s) == 64 * 14
     assert {(t["rows"], t["cols"]) for t in s} == {(256, 256)}
-    assert len({(t["row0"], t["col0"]) for t in s}) == len(s)              # bijection
-    assert {t["row0"] for t in s} == set(range(0, M, 256))
-    assert {t["col0"] for t in s} == set(range(0, N, 256))
+    _covers_exactly(s, M, N)
     for t in s:
         assert t["comm_block"] == t["row0"] // 2048
         assert t["local"] == int(t["comm_block"] == rank)                  # only local tiles skip the wait
     by = _by_wg(s)
-    # 896 tiles finish in 4 passes on 224 workgroups as on 256: the balanced grid
-    # leaves 32 compute units to the producer at no cost
+    # 896 tiles finish in 4 passes on 224 workgroups as on 256
     assert len(by) == 224 and all(len(v) == 4 for v in by.values())
     for wg, tiles in by.items():
         assert [t["step"] for t in tiles] == list(range(len(tiles)))
         ring = [(t["comm_block"] - rank) % ws for t in tiles]
         assert ring == sorted(ring)                                        # ready order of the gather
-    # the whole local comm block is scheduled in the first pass
     first = [t for t in s if t["step"] == 0]
     assert sum(t["local"] for t in first) == 8 * 14
-    # XCD locality: the 32 tiles an XCD holds in the first pass share few A/B slabs
+    # XCD locality: the 28 tiles an XCD holds in the first pass share few A/B slabs
     for x in range(8):
         mine = [t for t in first if t["wg"] % 8 == x]
         assert len(mine) == 28
         slabs = len({t["row0"] for t in mine}) + len({t["col0"] for t in mine})
         assert slabs <= 20                                                 # 56 when unrelated
+
+
+@pytest.mark.parametrize("rank", [0, 3, 7])
+def test_schedule_config5_gated(rank):
+    """Gated: the local comm block and the last one are cut into 256x128 half tiles
+    (half pass + 3 passes + half pass = the same 4 passes), so that every
+    workgroup starts on rows that need no flag."""
+    M, N, K, ws = 16384, 3584, 8192, 8
+    s = gemm_schedule(M, N, K, rank, ws, M // ws, gated=True)
+    _covers_exactly(s, M, N)
+    by = _by_wg(s)
+    assert len(by) == 224
+    for wg, tiles in by.items():
+        assert [t["cols"] for t in tiles] == [128, 256, 256, 256, 128]
+        assert tiles[0]["local"] == 1 and tiles[0]["comm_block"] == rank   # nobody starts with a wait
+        assert all(t["local"] == 0 for t in tiles[1:])
+        ring = [(t["comm_block"] - rank) % ws for t in tiles]
+        assert ring == sorted(ring) and ring[-1] == ws - 1
+    for t in s:
+        assert t["comm_block"] == t["row0"] // 2048
+        assert t["local"] == int(t["comm_block"] == rank)
+    # the first full pass only needs the next two comm blocks
+    assert {(t["comm_block"] - rank) % ws for t in s if t["step"] == 1} == {1, 2}
 
 
 @pytest.mark.parametrize("M,N,K,ws,splits", [(1024, 256, 256, 8, 1), (2048, 384, 512, 8, 1),
@@ -54,10 +85,8 @@ def test_schedule_other_shapes(M, N, K, ws, splits):
     comm = M // ws // splits
     for rank in range(ws):
         s = gemm_schedule(M, N, K, rank, ws, comm)
-        bm, bn = s[0]["rows"], s[0]["cols"]
-        assert comm % bm == 0
-        want = {(r, c) for r in range(0, M, bm) for c in range(0, N, bn)}
-        assert {(t["row0"], t["col0"]) for t in s} == want and len(s) == len(want)
+        assert comm % s[0]["rows"] == 0
+        _covers_exactly(s, M, N)
         for t in s:
             owner = t["comm_block"] // splits
             assert t["local"] == int(owner == rank)
