@@ -54,6 +54,24 @@ def _time_events(fn, iters, warm, pre=None):
     return _median(ts)
 
 
+def _time_batched(fn, calls, warm):
+    """Mean device time per call in microseconds over `calls` back-to-back launches
+    between one event pair: for kernels of a few tens of microseconds, where a
+    synchronise after every call would time the launch path instead."""
+    import torch
+    for _ in range(warm):
+        fn()
+    torch.cuda.synchronize()
+    a = torch.cuda.Event(enable_timing=True)
+    b = torch.cuda.Event(enable_timing=True)
+    a.record()
+    for _ in range(calls):
+        fn()
+    b.record()
+    torch.cuda.synchronize()
+    return a.elapsed_time(b) * 1e3 / calls
+
+
 def bench_reduce(size_mib, steps, warmup, dev):
     import torch
     from symm_mem_recipes import EmulatedSymmetricMemory as SM, one_shot_all_reduce
@@ -112,7 +130,7 @@ def bench_reduce_rotating(size_mib, dev, dtype_name="bf16"):
     def call():
         one_shot_all_reduce(sets[idx[0] % nsets], barrier=False)
         idx[0] += 1
-    us = _time_events(call, 40, nsets)
+    us = _time_batched(call, 10 * nsets, nsets)
     SM.release()
     return dict(size_mib=size_mib, dtype=dtype_name, us=us, gbs=(WS + 1) * nbytes / us / 1e3,
                 frac=(WS + 1) * nbytes / us / 1e3 / HBM_PEAK_GBS, buffer_sets=nsets)
@@ -171,7 +189,7 @@ def bench_gemv(dev):
         def call():
             gemv_all_reduce(xb, ws_[idx[0] % nw], WS, wsp, out)
             idx[0] += 1
-        us = _time_events(call, 40, nw)
+        us = _time_batched(call, 5 * nw, nw)
         wsp.check_status()
         nbytes = K * N * 2 + batch * K * 2 + batch * N * 2
         res.append(dict(batch=batch, us=us, gbs=nbytes / us / 1e3, frac=nbytes / us / 1e3 / HBM_PEAK_GBS))

@@ -181,11 +181,48 @@ struct TileContext {
   uint64_t* tr;                  // trace record of this tile or null
 };
 
-// One output tile: C[row0 .. +BM, col0 .. +BN] = A rows (at a_base) x B rows (at b_base)^T.
+// The first two K-slabs of a tile, global -> LDS stages 0 and 1 (no wait).  Issued
+// either at the start of the tile or, for every tile but a workgroup's first, by
+// the previous tile between its K loop and its epilogue, so that the loads fly
+// while the previous tile's results are being stored.
 template <int BM, int BN>
+__device__ __forceinline__ void issue_prologue(const TileContext& cx, const uint8_t* a_base,
+                                               const uint8_t* b_base, int b_last) {
+  using T = GemmTile<BM, BN>;
+  constexpr int GA = T::GA, GB = T::GB;
+  int ln = cx.lane;
+  asm volatile("" : "+v"(ln));
+  const int u = (ln & 7) ^ (ln >> 3);
+  const int stages = cx.nk > 1 ? 2 : 1;
+  for (int st = 0; st < stages; ++st) {
+    const uint8_t* ak = a_base + (int64_t)st * kRowBytes;
+    const uint8_t* bk = b_base + (int64_t)st * kRowBytes;
+    const uint32_t la = cx.lds0 + st * T::kABytes + cx.wave * (GA * 1024);
+    const uint32_t lb = cx.lds0 + T::kBBase + st * T::kBBytes + cx.wave * (GB * 1024);
+#pragma unroll
+    for (int j = 0; j < GA; ++j) {
+      const int q = cx.wave * GA + j;
+      load_group(ak, (uint32_t)(q * 8 + (ln >> 3)) * cx.row_stride + (uint32_t)((u ^ (q & 7)) << 4),
+                 la + j * 1024);
+    }
+#pragma unroll
+    for (int j = 0; j < GB; ++j) {
+      const int q = cx.wave * GB + j;
+      int r = q * 8 + (ln >> 3);
+      r = r < b_last ? r : b_last;
+      load_group(bk, (uint32_t)r * cx.row_stride + (uint32_t)((u ^ (q & 7)) << 4), lb + j * 1024);
+    }
+  }
+}
+
+// One output tile: C[row0 .. +BM, col0 .. +BN] = A rows (at a_base) x B rows (at b_base)^T.
+// `preloaded`: the tile's first two K-slabs are already on their way into LDS.
+// `between` runs after the K loop, when LDS is free again, and before the results
+// are stored: the place to start the next tile's loads.
+template <int BM, int BN, typename Between>
 __device__ __forceinline__ void run_tile(const TileContext& cx, const TileRef& tile,
                                          const uint8_t* a_base, const uint8_t* b_base,
-                                         uint32_t& warm_scrap) {
+                                         uint32_t& warm_scrap, bool preloaded, Between&& between) {
   using T = GemmTile<BM, BN>;
   constexpr int WM = T::WM, WN = T::WN, FM = T::FM, FN = T::FN, GA = T::GA, GB = T::GB;
   constexpr int kWarmLoads = GA / 8 + GB / 8;      // warm-up loads per wave and stage
@@ -305,8 +342,10 @@ __device__ __forceinline__ void run_tile(const TileContext& cx, const TileRef& t
   };
 
   // Prologue: both LDS stages in flight, then the first fragments.
-  load_stage(0, 0);
-  if (nk > 1) load_stage(1, 1);
+  if (!preloaded) {
+    load_stage(0, 0);
+    if (nk > 1) load_stage(1, 1);
+  }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
 #pragma unroll
@@ -395,6 +434,7 @@ __device__ __forceinline__ void run_tile(const TileContext& cx, const TileRef& t
   if (kt < nk) stage_body(std::integral_constant<int, 0>{}, kt);
   __syncthreads();       // the next tile's prologue overwrites both stages
   if (tr != nullptr) tr[2] = wall_clock64();
+  between();
 
   // D[n][m]: lane holds row m = lane & 31 and, per group of 4 registers, the 4
   // consecutive columns g*8 + (lane >> 5)*4 .. +3 of the 32x32 fragment.
@@ -438,31 +478,60 @@ __global__ __launch_bounds__(kGemmThreads, 1) void ag_matmul_kernel(
   cx.c = c;
   uint32_t warm_scrap = 0;
 
-  for (int step = 0;; ++step) {
-    TileRef tile;
-    if (!tile_for(s, blockIdx.x, step, tile)) break;
+  // Source rows of a tile: the local shard, or the gathered buffer once the comm
+  // block's flag is up.
+  auto a_rows_of = [&](const TileRef& t) -> const uint8_t* {
+    if (t.local) return a_shard + (int64_t)t.a_row * cx.row_stride;
+    if (progress != nullptr) wait_signal(progress + t.comm_block, limit_ticks, status, t.comm_block);
+    return a_out + (int64_t)t.a_row * cx.row_stride;
+  };
+
+  TileRef tile;
+  bool have = tile_for(s, blockIdx.x, 0, tile);
+  const uint8_t* a_base = nullptr;
+  const uint8_t* b_base = nullptr;
+  if (have) {
+    a_base = a_rows_of(tile);
+    b_base = b_nk + (int64_t)tile.col0 * cx.row_stride;
+  }
+  bool preloaded = false;
+  for (int step = 0; have; ++step) {
     cx.tr = nullptr;
     if (trace != nullptr && step < kTraceSteps && blockIdx.x < 256 && threadIdx.x == 0) {
       cx.tr = trace + kTraceProducerWords + ((size_t)blockIdx.x * kTraceSteps + step) * 4;
-      cx.tr[0] = wall_clock64();
+      cx.tr[0] = cx.tr[1] = wall_clock64();
     }
-    const uint8_t* a_base;
-    if (tile.local) {
-      a_base = a_shard + (int64_t)tile.a_row * cx.row_stride;
-    } else {
-      if (progress != nullptr)
-        wait_signal(progress + tile.comm_block, limit_ticks, status, tile.comm_block);
-      a_base = a_out + (int64_t)tile.a_row * cx.row_stride;
-    }
-    if (cx.tr != nullptr) cx.tr[1] = wall_clock64();
-    const uint8_t* b_base = b_nk + (int64_t)tile.col0 * cx.row_stride;
+    TileRef next;
+    bool have_next = false;
+    const uint8_t* a_next = nullptr;
+    const uint8_t* b_next = nullptr;
+    // Between this tile's K loop and its stores: pick the next tile, wait for its
+    // flag if it has one, and start its first loads.
+    auto between = [&]() {
+      have_next = tile_for(s, blockIdx.x, step + 1, next);
+      if (!have_next) return;
+      a_next = a_rows_of(next);
+      b_next = b_nk + (int64_t)next.col0 * cx.row_stride;
+      const int b_last = s.N - 1 - next.col0;
+      if constexpr (BN == 256) {
+        if (next.cols != BN) issue_prologue<BM, BN / 2>(cx, a_next, b_next, b_last);
+        else issue_prologue<BM, BN>(cx, a_next, b_next, b_last);
+      } else {
+        issue_prologue<BM, BN>(cx, a_next, b_next, b_last);
+      }
+    };
     if constexpr (BN == 256) {
-      if (tile.cols != BN) run_tile<BM, BN / 2>(cx, tile, a_base, b_base, warm_scrap);
-      else run_tile<BM, BN>(cx, tile, a_base, b_base, warm_scrap);
+      if (tile.cols != BN) run_tile<BM, BN / 2>(cx, tile, a_base, b_base, warm_scrap, preloaded, between);
+      else run_tile<BM, BN>(cx, tile, a_base, b_base, warm_scrap, preloaded, between);
     } else {
-      run_tile<BM, BN>(cx, tile, a_base, b_base, warm_scrap);
+      run_tile<BM, BN>(cx, tile, a_base, b_base, warm_scrap, preloaded, between);
     }
     if (cx.tr != nullptr) cx.tr[3] = wall_clock64();
+    have = have_next;
+    tile = next;
+    a_base = a_next;
+    b_base = b_next;
+    preloaded = true;
   }
   // Drain the warm-up loads and give the scrap register a use the compiler
   // cannot remove (K is never negative).

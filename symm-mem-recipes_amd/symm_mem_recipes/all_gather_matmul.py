@@ -18,6 +18,10 @@ import torch
 from . import _lib
 from .symm_mem import EmulatedSymmetricMemory, _get_backend_stream
 
+#: Upper bound on the producer's workgroups (it never gets more than the compute
+#: units the GEMM's grid leaves free).
+MAX_PRODUCER_WORKGROUPS = 24
+
 
 def all_gather_with_progress(output: torch.Tensor, inp: torch.Tensor, progress: torch.Tensor,
                              splits_per_rank: int, num_workgroups: int = 0) -> None:
@@ -103,7 +107,7 @@ def all_gather_matmul_tma_persistent(a_shard: torch.Tensor, b: torch.Tensor, a_o
         if grid < 0:
             _lib.check(grid, "all_gather_matmul")
         cus = torch.cuda.get_device_properties(device).multi_processor_count
-        producer_wgs = max(8, min(32, cus - grid))
+        producer_wgs = max(8, min(MAX_PRODUCER_WORKGROUPS, cus - grid))
         with torch.cuda.stream(backend):
             all_gather_with_progress(a_out, a_shard, progress, splits_per_rank, producer_wgs)
 
