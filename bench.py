@@ -207,6 +207,7 @@ def bench_barrier(dev):
     h = SM.rendezvous(t)
     rounds = 10000
     us_flags = _time_events(lambda: blockwise_barrier(h, blocks, rounds), 3, 1) / rounds
+    us_flags_only = _time_events(lambda: blockwise_barrier(h, blocks, rounds, order_memory=False), 3, 1) / rounds
     h.check_status()
     src = (torch.rand(WS, blocks, words * 2, device=dev) * 2 - 1).to(torch.bfloat16).view(torch.int32)
     src = src.reshape(WS, blocks, words).contiguous()
@@ -229,6 +230,7 @@ def bench_barrier(dev):
     SM.release()
     written = WS * blocks * chunk
     return dict(workgroups=WS * blocks, rounds_flags=rounds, us_per_round_flags=us_flags,
+                us_per_round_flags_no_cache_maintenance=us_flags_only,
                 rounds_payload=prounds, us_per_round_payload=us_payload,
                 payload_written_mib=written / 2 ** 20, payload_read_mib=WS * written / 2 ** 20,
                 payload_gbs=(written + WS * written) / us_payload / 1e3)

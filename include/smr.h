@@ -104,9 +104,13 @@ int smr_set_reduce_launch(int threads, int max_blocks);
  * around the device function blockwise_barrier (:50-153).
  *   rank -1: all ws emulated ranks in one launch (ws*num_blocks workgroups)
  *   rank >= 0: only that rank's num_blocks workgroups; its peers must be running
- *              concurrently on other streams or the spins time out. */
+ *              concurrently on other streams or the spins time out.
+ *   order_memory 1: every round releases the workgroup's earlier writes before the
+ *              sends and acquires after the waits, as the reference's barrier does
+ *              (release CAS :119-122, acquire loads :145-153).  0: flags only,
+ *              for data handed over with coherent accesses. */
 int smr_barrier(const uint64_t* signal_pad_ptrs_dev, int rank, int world_size, int num_blocks,
-                int rounds, uint32_t* status, void* stream);
+                int rounds, int order_memory, uint32_t* status, void* stream);
 
 /* Host-callable halves of the flag protocol, one workgroup each.
  * smr_send_signal: release-CAS 0->1 (triton_barrier.py:119-122).

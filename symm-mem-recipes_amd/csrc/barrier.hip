@@ -37,7 +37,7 @@ __device__ __forceinline__ bool any_failure(uint32_t* status, uint32_t* lds_flag
 
 __global__ __launch_bounds__(kBarrierThreads) void barrier_kernel(
     const uint64_t* __restrict__ signal_pad_ptrs, int rank, int world_size, int rounds,
-    uint64_t limit_ticks, uint32_t* status) {
+    int order_memory, uint64_t limit_ticks, uint32_t* status) {
   __shared__ uint32_t failed;
   int block = blockIdx.x;
   if (rank < 0) {
@@ -45,7 +45,9 @@ __global__ __launch_bounds__(kBarrierThreads) void barrier_kernel(
     rank = blockIdx.x % world_size;
   }
   for (int r = 0; r < rounds; ++r) {
-    if (!blockwise_barrier(signal_pad_ptrs, block, rank, world_size, limit_ticks, status)) break;
+    if (!blockwise_barrier(signal_pad_ptrs, block, rank, world_size, limit_ticks, status,
+                           order_memory != 0, order_memory != 0))
+      break;
     if ((r & 63) == 63 && any_failure(status, &failed)) break;
   }
 }
@@ -78,11 +80,17 @@ __global__ __launch_bounds__(kRoundThreads) void signal_round_kernel(
       for (int64_t i = threadIdx.x; i < chunk_vecs; i += kRoundThreads) {
         u32x4 v = my_src[i];
         v.x += tag; v.y += tag; v.z += tag; v.w += tag;
-        dst[i] = v;
+        uint64_t* d = reinterpret_cast<uint64_t*>(dst + i);
+        store_coherent(d, ((uint64_t)v.y << 32) | v.x);
+        store_coherent(d + 1, ((uint64_t)v.w << 32) | v.z);
       }
+      wait_stores_acknowledged();
     }
-    // publish + wait for all peers' chunks of this block
-    if (!blockwise_barrier(signal_pad_ptrs, block, rank, world_size, limit_ticks, status)) break;
+    // Publish + wait for all peers' chunks of this block.  The payload travels
+    // with agent-coherent stores and loads, so the handshake itself needs no
+    // cache write-back or invalidate.
+    if (!blockwise_barrier(signal_pad_ptrs, block, rank, world_size, limit_ticks, status, false, false))
+      break;
     // consume
     if (chunk_vecs) {
       uint32_t s = 0u;
@@ -90,8 +98,9 @@ __global__ __launch_bounds__(kRoundThreads) void signal_round_kernel(
         const u32x4* peer = reinterpret_cast<const u32x4*>(
             reinterpret_cast<const uint32_t*>(buffer_ptrs[p]) + half + (size_t)block * chunk_words);
         for (int64_t i = threadIdx.x; i < chunk_vecs; i += kRoundThreads) {
-          const u32x4 v = peer[i];
-          s += v.x + v.y + v.z + v.w;
+          const uint64_t* q = reinterpret_cast<const uint64_t*>(peer + i);
+          const uint64_t lo = load_coherent(q), hi = load_coherent(q + 1);
+          s += (uint32_t)lo + (uint32_t)(lo >> 32) + (uint32_t)hi + (uint32_t)(hi >> 32);
         }
       }
 #pragma unroll
@@ -139,7 +148,7 @@ __global__ void write_value32_kernel(uint32_t* addr, uint32_t value) {
 extern "C" {
 
 int smr_barrier(const uint64_t* signal_pad_ptrs_dev, int rank, int world_size, int num_blocks,
-                int rounds, uint32_t* status, void* stream) {
+                int rounds, int order_memory, uint32_t* status, void* stream) {
   using namespace smr;
   if (signal_pad_ptrs_dev == nullptr) return fail(SMR_E_INVALID, "smr_barrier: signal pads are NULL");
   if (world_size < 1 || world_size > SMR_MAX_WORLD_SIZE)
@@ -152,7 +161,7 @@ int smr_barrier(const uint64_t* signal_pad_ptrs_dev, int rank, int world_size, i
   const unsigned grid = rank < 0 ? (unsigned)num_blocks * world_size : (unsigned)num_blocks;
   hipLaunchKernelGGL(barrier_kernel, dim3(grid), dim3(kBarrierThreads), 0,
                      reinterpret_cast<hipStream_t>(stream), signal_pad_ptrs_dev, rank, world_size,
-                     rounds, spin_limit_ticks(), status);
+                     rounds, order_memory, spin_limit_ticks(), status);
   return check_hip(hipGetLastError(), "smr_barrier launch");
 }
 

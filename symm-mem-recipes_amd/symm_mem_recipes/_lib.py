@@ -38,7 +38,7 @@ SIGNATURES = {
     "smr_one_shot_all_reduce": (_i, [_p, _p, _p, _i64, _i, _i, _i, _i, _i, _p, _p]),
     "smr_reduce_num_blocks": (_i, [_i64, _i]),
     "smr_set_reduce_launch": (_i, [_i, _i]),
-    "smr_barrier": (_i, [_p, _i, _i, _i, _i, _p, _p]),
+    "smr_barrier": (_i, [_p, _i, _i, _i, _i, _i, _p, _p]),
     "smr_send_signal": (_i, [_p, _p, _p]),
     "smr_wait_signal": (_i, [_p, _p, _p]),
     "smr_wait_signal_reset": (_i, [_p, _p, _p]),

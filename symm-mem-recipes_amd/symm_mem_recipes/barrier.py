@@ -20,14 +20,16 @@ def _stream(device) -> int:
 
 
 def blockwise_barrier(symm_mem: EmulatedSymmetricMemory, num_blocks: int, rounds: int = 1,
-                      all_ranks: bool = True) -> None:
+                      all_ranks: bool = True, order_memory: bool = True) -> None:
     """Run ``rounds`` barrier rounds on ``num_blocks`` blocks.  With
     ``all_ranks`` every emulated rank takes part in one launch; otherwise only
-    ``symm_mem.rank`` runs and its peers must be running on other streams."""
+    ``symm_mem.rank`` runs and its peers must be running on other streams.
+    ``order_memory`` keeps the reference's release/acquire around every round;
+    without it only the flags are exchanged."""
     assert num_blocks * symm_mem.world_size * 4 <= symm_mem.signal_pad_size, "signal pad too small"
     lib = _lib.load()
     rc = lib.smr_barrier(symm_mem.signal_pad_ptrs_dev, -1 if all_ranks else symm_mem.rank,
-                         symm_mem.world_size, int(num_blocks), int(rounds),
+                         symm_mem.world_size, int(num_blocks), int(rounds), int(order_memory),
                          symm_mem.status.data_ptr(), _stream(symm_mem.device))
     _lib.check(rc, "blockwise_barrier")
 

@@ -66,10 +66,10 @@ def test_reduce_argument_errors_before_launch(lib):
 
 
 def test_barrier_argument_errors(lib):
-    assert lib.smr_barrier(None, 0, 8, 1, 1, None, None) == -1
-    assert lib.smr_barrier(0x1000, 0, 8, 0, 1, None, None) == -1
-    assert lib.smr_barrier(0x1000, 9, 8, 1, 1, None, None) == -1
-    assert lib.smr_barrier(0x1000, -1, 8, 2000, 1, None, None) == -2
+    assert lib.smr_barrier(None, 0, 8, 1, 1, 1, None, None) == -1
+    assert lib.smr_barrier(0x1000, 0, 8, 0, 1, 1, None, None) == -1
+    assert lib.smr_barrier(0x1000, 9, 8, 1, 1, 1, None, None) == -1
+    assert lib.smr_barrier(0x1000, -1, 8, 2000, 1, 1, None, None) == -2
     assert lib.smr_signal_round(None, None, 0x1000, None, 0x1000, 0x1000, 8, 304, 24, 1, None, None) == -1
     assert lib.smr_send_signal(None, None, None) == -1
     assert lib.smr_wait_signal(None, None, None) == -1

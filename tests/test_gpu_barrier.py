@@ -36,10 +36,11 @@ def test_barrier_test_terminates_and_resets(handle):
     assert _pads_zero(handle)
 
 
+@pytest.mark.parametrize("order_memory", [True, False])
 @pytest.mark.parametrize("blocks,rounds", [(1, 1), (32, 100), (304, 1000)])
-def test_many_rounds(handle, blocks, rounds):
+def test_many_rounds(handle, blocks, rounds, order_memory):
     from symm_mem_recipes import blockwise_barrier
-    blockwise_barrier(handle, blocks, rounds)
+    blockwise_barrier(handle, blocks, rounds, order_memory=order_memory)
     handle.check_status()
     assert _pads_zero(handle)
 
