@@ -161,3 +161,22 @@ def test_full_size_config5(cuda):
     c_rms = float(c_out.float().pow(2).mean().sqrt())
     tol = 8 * (N ** 0.5) * 2.0 ** -9 * c_rms + 1e-3
     assert torch.all((got - rowsum).abs() <= tol), float((got - rowsum).abs().max())
+
+
+def test_golden_vectors(cuda):
+    """tests/golden/ag_matmul.npz: 4 shards of [128, 64], B [72, 64]."""
+    import os
+    from symm_mem_recipes import EmulatedSymmetricMemory as SM, all_gather_matmul_tma_persistent
+    g = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "ag_matmul.npz"))
+    ws, rows, K = g["shards"].shape
+    N = g["b_nk"].shape[0]
+    for rank in range(ws):
+        a_shard = SM.empty_strided_p2p((rows, K), (K, 1), torch.bfloat16, cuda, world_size=ws, rank=rank)
+        h = SM.rendezvous(a_shard)
+        for r in range(ws):
+            h.get_buffer(r, (rows, K), torch.bfloat16).copy_(_bits_t(g["shards"][r]))
+        a_out = torch.zeros(ws * rows, K, dtype=torch.bfloat16, device=cuda)
+        c_out = torch.full((ws * rows, N), float("nan"), dtype=torch.bfloat16, device=cuda)
+        all_gather_matmul_tma_persistent(a_shard, _bits_t(g["b_nk"]).to(cuda), a_out, c_out, None)
+        h.check_status()
+        _check(_t_bits(c_out), g["c"])

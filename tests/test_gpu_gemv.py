@@ -111,3 +111,16 @@ def test_gemv_validation(cuda):
         gemv_all_reduce(x[:2, :60].contiguous(), w[:60].contiguous())
     with pytest.raises(AssertionError):
         gemv_all_reduce(x[:2].contiguous(), w[:, :100].contiguous())       # N % 8
+
+
+def test_golden_vectors(cuda):
+    """tests/golden/gemv.npz: x [4, 256], W [256, 128], 8 K-shards."""
+    import os
+    from symm_mem_recipes import gemv_all_reduce
+    g = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "gemv.npz"))
+    out = gemv_all_reduce(_bits_t(g["x"]).to(cuda), _bits_t(g["w"]).to(cuda), 8)
+    torch.cuda.synchronize()
+    got = O.bf16_bits_to_f32(_t_bits(out)).astype(np.float64)
+    ref = O.bf16_bits_to_f32(g["out"]).astype(np.float64)
+    terms = np.abs(O.bf16_bits_to_f32(g["x"])).astype(np.float64) @ np.abs(O.bf16_bits_to_f32(g["w"])).astype(np.float64)
+    assert _within_one_ulp(got, ref, terms)

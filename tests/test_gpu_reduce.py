@@ -189,3 +189,19 @@ def test_full_size_properties_64mib(cuda, dtype):
     for s in starts:
         want = O.reduce_ref(bufs[s], "bf16" if dtype == torch.bfloat16 else "fp32")
         assert _same(_bits(out[s:s + win]), want)
+
+
+def test_golden_vectors(cuda):
+    """The committed vectors (tests/golden/reduce.npz), independent of the oracle's code."""
+    import os
+    from symm_mem_recipes import one_shot_all_reduce
+    g = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "reduce.npz"))
+    t, h = _alloc(256, torch.bfloat16, cuda)
+    for r in range(WS):
+        h.get_buffer(r, (256,), torch.int16).copy_(torch.from_numpy(g["bf16_in"][r].view(np.int16)))
+    assert np.array_equal(_bits(one_shot_all_reduce(t)), g["bf16_out"])
+    t, h = _alloc(256, torch.float32, cuda)
+    for r in range(WS):
+        h.get_buffer(r, (256,), torch.float32).copy_(torch.from_numpy(g["fp32_in"][r]))
+    assert np.array_equal(_bits(one_shot_all_reduce(t)).view(np.uint32), g["fp32_out"].view(np.uint32))
+    h.check_status()
