@@ -133,8 +133,7 @@ __device__ __forceinline__ bf16x8 lds_read_frag(uint32_t addr) {
 //
 // Issued through inline assembly so that the compiler does not count these loads:
 // it cannot tell which LDS bytes they write, so it would make every later
-// fragment read wait for all of them - and for the L2 warm-up loads issued
-// behind them.  All waits on these loads are explicit s_waitcnt vmcnt in the
+// fragment read wait for all of them.  All waits on these loads are explicit s_waitcnt vmcnt in the
 // kernel (loads return in order, so "vmcnt(n)" leaves the n youngest in flight).
 __device__ __forceinline__ void load_group(const uint8_t* base, uint32_t voff, uint32_t lds_dst) {
   // scalar base + 32-bit per-lane offset: no 64-bit address arithmetic per lane
@@ -155,36 +154,39 @@ __device__ __forceinline__ void interleave_mfma_dsread() {
   }
 }
 
+// LDS holds a ring of five slots.  A K-slab of A and a K-slab of B take one slot each,
+// in the order A0 B0 A1 B1 A2 ..., so slab number i lives in slot i % 5: the two slabs
+// of the K step being multiplied, and up to three slabs that are landing.
+constexpr int kRingSlots = 5;
+
 template <int BM, int BN>
 struct GemmTile {
   static constexpr int WM = BM / 2, WN = BN / 2;        // wave tile (2 x 2 waves)
   static constexpr int FM = WM / 32, FN = WN / 32;      // 32x32 fragments per wave tile
-  static constexpr int GA = BM / 32, GB = BN / 32;      // 8-row load groups per wave and stage
-  static constexpr int kABytes = BM * kRowBytes, kBBytes = BN * kRowBytes;
-  // LDS map: A stage 0 | A stage 1 | B stage 0 | B stage 1.  The second stage of an
-  // operand is a 16-bit immediate away from the first.
-  static constexpr int kBBase = 2 * kABytes;
-  static constexpr int kLdsBytes = 2 * (kABytes + kBBytes);
+  static constexpr int GA = BM / 32, GB = BN / 32;      // 8-row load groups per wave and slab
+  // BN <= BM in every configuration; a slot takes the larger slab, which also lets a
+  // half-width tile share the ring (and the next tile's early loads) with a full one.
+  static constexpr int kSlotBytes = BM * kRowBytes;
+  static constexpr int kLdsBytes = kRingSlots * kSlotBytes;
+  static_assert(BN <= BM, "slot size is the A slab");
 };
-
-// How many stages ahead of its real load a K-slab is touched to pull it into L2.
-constexpr int kWarmAhead = 3;
 
 // Everything a tile needs that does not depend on the tile shape.
 struct TileContext {
   int lane, wave;
   uint32_t row_stride;           // bytes between rows of A and of B
   int nk;                        // K-slabs
-  uint32_t lds0;                 // LDS byte offset of the tile buffer
+  uint32_t lds0;                 // LDS byte offset of the ring
   int N;
   uint8_t* c;
   uint64_t* tr;                  // trace record of this tile or null
 };
 
-// The first two K-slabs of a tile, global -> LDS stages 0 and 1 (no wait).  Issued
-// either at the start of the tile or, for every tile but a workgroup's first, by
-// the previous tile between its K loop and its epilogue, so that the loads fly
-// while the previous tile's results are being stored.
+// The first five slabs of a tile (A0 B0 A1 B1 A2), global -> ring slots 0..4, no wait.
+// Issued either at the start of the tile or, for every tile but a workgroup's first,
+// by the previous tile between its K loop and its epilogue, so that the loads fly
+// while the previous tile's results are being stored.  Slabs past the end of K repeat
+// the last one; nobody reads them.
 template <int BM, int BN>
 __device__ __forceinline__ void issue_prologue(const TileContext& cx, const uint8_t* a_base,
                                                const uint8_t* b_base, int b_last) {
@@ -193,39 +195,42 @@ __device__ __forceinline__ void issue_prologue(const TileContext& cx, const uint
   int ln = cx.lane;
   asm volatile("" : "+v"(ln));
   const int u = (ln & 7) ^ (ln >> 3);
-  const int stages = cx.nk > 1 ? 2 : 1;
-  for (int st = 0; st < stages; ++st) {
-    const uint8_t* ak = a_base + (int64_t)st * kRowBytes;
-    const uint8_t* bk = b_base + (int64_t)st * kRowBytes;
-    const uint32_t la = cx.lds0 + st * T::kABytes + cx.wave * (GA * 1024);
-    const uint32_t lb = cx.lds0 + T::kBBase + st * T::kBBytes + cx.wave * (GB * 1024);
 #pragma unroll
-    for (int j = 0; j < GA; ++j) {
-      const int q = cx.wave * GA + j;
-      load_group(ak, (uint32_t)(q * 8 + (ln >> 3)) * cx.row_stride + (uint32_t)((u ^ (q & 7)) << 4),
-                 la + j * 1024);
-    }
+  for (int idx = 0; idx < kRingSlots; ++idx) {
+    const int k = (idx >> 1) < cx.nk ? (idx >> 1) : cx.nk - 1;
+    const uint32_t dst = cx.lds0 + idx * T::kSlotBytes;
+    if ((idx & 1) == 0) {
+      const uint8_t* ak = a_base + (int64_t)k * kRowBytes;
 #pragma unroll
-    for (int j = 0; j < GB; ++j) {
-      const int q = cx.wave * GB + j;
-      int r = q * 8 + (ln >> 3);
-      r = r < b_last ? r : b_last;
-      load_group(bk, (uint32_t)r * cx.row_stride + (uint32_t)((u ^ (q & 7)) << 4), lb + j * 1024);
+      for (int j = 0; j < GA; ++j) {
+        const int q = cx.wave * GA + j;
+        load_group(ak, (uint32_t)(q * 8 + (ln >> 3)) * cx.row_stride + (uint32_t)((u ^ (q & 7)) << 4),
+                   dst + q * 1024);
+      }
+    } else {
+      const uint8_t* bk = b_base + (int64_t)k * kRowBytes;
+#pragma unroll
+      for (int j = 0; j < GB; ++j) {
+        const int q = cx.wave * GB + j;
+        int r = q * 8 + (ln >> 3);
+        r = r < b_last ? r : b_last;
+        load_group(bk, (uint32_t)r * cx.row_stride + (uint32_t)((u ^ (q & 7)) << 4), dst + q * 1024);
+      }
     }
   }
 }
 
 // One output tile: C[row0 .. +BM, col0 .. +BN] = A rows (at a_base) x B rows (at b_base)^T.
-// `preloaded`: the tile's first two K-slabs are already on their way into LDS.
+// `preloaded`: the tile's first five slabs are already on their way into LDS.
 // `between` runs after the K loop, when LDS is free again, and before the results
 // are stored: the place to start the next tile's loads.
 template <int BM, int BN, typename Between>
 __device__ __forceinline__ void run_tile(const TileContext& cx, const TileRef& tile,
                                          const uint8_t* a_base, const uint8_t* b_base,
-                                         uint32_t& warm_scrap, bool preloaded, Between&& between) {
+                                         bool preloaded, Between&& between) {
   using T = GemmTile<BM, BN>;
   constexpr int WM = T::WM, WN = T::WN, FM = T::FM, FN = T::FN, GA = T::GA, GB = T::GB;
-  constexpr int kWarmLoads = GA / 8 + GB / 8;      // warm-up loads per wave and stage
+  constexpr uint32_t kSlot = T::kSlotBytes;
   const int lane = cx.lane, wave = cx.wave;
   const int wm = wave >> 1, wn = wave & 1;
   const int half = lane >> 5;
@@ -242,18 +247,21 @@ __device__ __forceinline__ void run_tile(const TileContext& cx, const TileRef& t
   // in the middle of the K loop.
   int ln = lane;
   asm volatile("" : "+v"(ln));
-  // ---- per-lane fragment read addresses (stage 0).  Row r = w*W + f*32 + (ln & 31)
+  // ---- per-lane fragment read addresses.  Row r = w*W + f*32 + (ln & 31)
   // has swizzle ((lane & 7) ^ ((ln >> 3) & 3)) ^ ((f & 1) << 2); K step kk wants
   // chunk 2*kk + half.  Hence position = t ^ (v << 1) with the per-lane constant
   // t = half ^ (lane & 7) ^ ((ln >> 3) & 3) and v = kk ^ ((f & 1) << 1): four
-  // variants per operand, everything else is an immediate offset.
+  // variants per operand, the fragment row is an immediate offset.  The addresses
+  // point into the slots of the slab pair being read (slots 0 and 1 at first) and
+  // move around the ring by a uniform amount once per slab pair.
   const int t = (ln >> 5) ^ (ln & 7) ^ ((ln >> 3) & 3);
   uint32_t a_fr[4], b_fr[4];
 #pragma unroll
   for (int v = 0; v < 4; ++v) {
     a_fr[v] = lds0 + (uint32_t)((wm * WM + (ln & 31)) * kRowBytes + ((t ^ (v << 1)) << 4));
-    b_fr[v] = lds0 + T::kBBase + (uint32_t)((wn * WN + (ln & 31)) * kRowBytes + ((t ^ (v << 1)) << 4));
+    b_fr[v] = lds0 + kSlot + (uint32_t)((wn * WN + (ln & 31)) * kRowBytes + ((t ^ (v << 1)) << 4));
   }
+  uint32_t a_at = 0, b_at = kSlot;       // ring offsets of the slab pair being read
 
   // ---- per-lane global offsets of the tile loads.  Load group q = wave*G + j holds
   // rows q*8 .. q*8+7; lane l carries row q*8 + (l >> 3) and the chunk whose swizzled
@@ -265,13 +273,7 @@ __device__ __forceinline__ void run_tile(const TileContext& cx, const TileRef& t
     const int q = wave * GA + j;
     a_off[j] = (uint32_t)(q * 8 + (ln >> 3)) * row_stride + (uint32_t)((u ^ (q & 7)) << 4);
   }
-
-  // ---- L2 warm-up: one dword per 128-byte row segment, 64 rows per wave instruction
-  uint32_t a_warm[GA / 8 > 0 ? GA / 8 : 1];
-#pragma unroll
-  for (int j = 0; j < GA / 8; ++j) a_warm[j] = (uint32_t)(wave * (GA * 8) + j * 64 + ln) * row_stride;
-
-    // rows of B past the last column are clamped: they feed outputs that are never stored
+  // rows of B past the last column are clamped: they feed outputs that are never stored
   const int b_last = s.N - 1 - tile.col0;
   uint32_t b_off[GB];
 #pragma unroll
@@ -282,14 +284,6 @@ __device__ __forceinline__ void run_tile(const TileContext& cx, const TileRef& t
     b_off[j] = (uint32_t)r * row_stride + (uint32_t)((u ^ (q & 7)) << 4);
   }
 
-  uint32_t b_warm[GB / 8 > 0 ? GB / 8 : 1];
-#pragma unroll
-  for (int j = 0; j < GB / 8; ++j) {
-    int r = wave * (GB * 8) + j * 64 + ln;
-    r = r < b_last ? r : b_last;
-    b_warm[j] = (uint32_t)r * row_stride;
-  }
-
   f32x16 acc[FN][FM];
 #pragma unroll
   for (int ni = 0; ni < FN; ++ni)
@@ -298,40 +292,13 @@ __device__ __forceinline__ void run_tile(const TileContext& cx, const TileRef& t
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[ni][mi][e] = 0.0f;
 
-  auto load_stage = [&](int stage, int kt) {
-    const uint8_t* ak = a_base + (int64_t)kt * kRowBytes;
-    const uint8_t* bk = b_base + (int64_t)kt * kRowBytes;
-    const uint32_t la = lds0 + stage * T::kABytes + wave * (GA * 1024);
-    const uint32_t lb = lds0 + T::kBBase + stage * T::kBBytes + wave * (GB * 1024);
-#pragma unroll
-    for (int j = 0; j < GA; ++j) load_group(ak, a_off[j], la + j * 1024);
-#pragma unroll
-    for (int j = 0; j < GB; ++j) load_group(bk, b_off[j], lb + j * 1024);
-  };
-  // Touch the K-slab of stage kt (one dword per row) so that its real load,
-  // kWarmAhead stages later, finds the lines in L2.  The loaded dwords go to a
-  // scrap register that is never read for its value.  Inline assembly on
-  // purpose: the compiler must not count these loads, or it would make the wave
-  // wait for them - they are meant to miss - before the next fragment reads.
-  // `warm_scrap` is threaded through every statement and consumed after the
-  // tile loop, so its register stays reserved while loads into it are in flight.
-  auto warm_stage = [&](int kt) {
-    const uint8_t* ak = a_base + (int64_t)kt * kRowBytes;
-    const uint8_t* bk = b_base + (int64_t)kt * kRowBytes;
-#pragma unroll
-    for (int j = 0; j < GA / 8; ++j)
-      asm volatile("global_load_dword %0, %1, %2" : "+v"(warm_scrap) : "v"(a_warm[j]), "s"(ak) : "memory");
-#pragma unroll
-    for (int j = 0; j < GB / 8; ++j)
-      asm volatile("global_load_dword %0, %1, %2" : "+v"(warm_scrap) : "v"(b_warm[j]), "s"(bk) : "memory");
-  };
-  auto read_frags = [&](bf16x8 (&af)[FM], bf16x8 (&bf)[FN], int stage, int kk) {
+  auto read_frags = [&](bf16x8 (&af)[FM], bf16x8 (&bf)[FN], int kk) {
 #pragma unroll
     for (int mi = 0; mi < FM; ++mi)
-      af[mi] = lds_read_frag(a_fr[kk ^ ((mi & 1) << 1)] + stage * T::kABytes + mi * (32 * kRowBytes));
+      af[mi] = lds_read_frag(a_fr[kk ^ ((mi & 1) << 1)] + mi * (32 * kRowBytes));
 #pragma unroll
     for (int ni = 0; ni < FN; ++ni)
-      bf[ni] = lds_read_frag(b_fr[kk ^ ((ni & 1) << 1)] + stage * T::kBBytes + ni * (32 * kRowBytes));
+      bf[ni] = lds_read_frag(b_fr[kk ^ ((ni & 1) << 1)] + ni * (32 * kRowBytes));
   };
   auto mfma_all = [&](const bf16x8 (&af)[FM], const bf16x8 (&bf)[FN]) {
 #pragma unroll
@@ -341,39 +308,48 @@ __device__ __forceinline__ void run_tile(const TileContext& cx, const TileRef& t
         acc[ni][mi] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bf[ni], af[mi], acc[ni][mi], 0, 0, 0);
   };
 
-  // Prologue: both LDS stages in flight, then the first fragments.
-  if (!preloaded) {
-    load_stage(0, 0);
-    if (nk > 1) load_stage(1, 1);
-  }
+  // Prologue: five slabs in flight, then the first fragments.  The wait is for
+  // everything: loads and the previous tile's stores do not retire in one order.
+  if (!preloaded) issue_prologue<BM, BN>(cx, a_base, b_base, b_last);
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
-#pragma unroll
-  for (int w = 0; w < kWarmAhead; ++w) warm_stage(2 + w < nk ? 2 + w : nk - 1);
 
   // Fragment double buffer: while the MFMAs of K step kk run, the fragments of
   // step kk+1 are read.  The workgroup barrier sits before the last K step of a
-  // stage, right after that stage's last fragment reads: from there on the stage
-  // is free, so the loads of stage kt+2 are issued into it and have a whole stage
-  // of MFMAs to land, and the first fragments of stage kt+1 are read under the
-  // MFMAs of the last K step.
+  // slab pair, right after its last fragment reads: from there on both of its
+  // slots are free.
   bf16x8 af0[FM], bf0[FN], af1[FM], bf1[FN];
-  read_frags(af0, bf0, 0, 0);
+  read_frags(af0, bf0, 0);
 
-  // Last K step of a stage, issued right behind the barrier.  Its fragments are
-  // already in registers, so the MFMAs can start at once; the loads of stage
-  // kt+2, the first fragment reads of stage kt+1 and the warm-up touches are
-  // slotted in between them instead of standing in front of them.  There is
-  // one code path: past the end of K the loads are clamped to the last K-slab
-  // (they land in a stage nobody reads any more) rather than branched around,
+  // Last K step of slab pair kt, issued right behind the barrier.  Its
+  // fragments are already in registers, so the MFMAs start at once; slotted in
+  // between them are
+  //   * the loads of B slab kt+2 into the slot A slab kt just left: they must
+  //     have landed by the next barrier, one slab pair (64 MFMAs) from now;
+  //   * the loads of A slab kt+3 into the slot of B slab kt: two slab pairs of
+  //     time.  Only half of a K step's bytes are ever on the short deadline,
+  //     which the 2.5 slab pairs of LDS buy;
+  //   * the first fragment reads of slab pair kt+1.
+  // There is one code path: past the end of K the loads repeat the last slab
+  // (into a slot nobody reads any more) rather than being branched around,
   // which keeps the accumulators in place across the whole loop body.
-  auto last_step = [&](auto stage_tag, int kt) {
-    constexpr int S = decltype(stage_tag)::value;
-    const int kl = kt + 2 < nk ? kt + 2 : nk - 1;
-    const uint8_t* ak = a_base + (int64_t)kl * kRowBytes;
-    const uint8_t* bk = b_base + (int64_t)kl * kRowBytes;
-    const uint32_t la = lds0 + S * T::kABytes + wave * (GA * 1024);
-    const uint32_t lb = lds0 + T::kBBase + S * T::kBBytes + wave * (GB * 1024);
+  auto last_step = [&](int kt) {
+    const int kb = kt + 2 < nk ? kt + 2 : nk - 1;
+    const int ka = kt + 3 < nk ? kt + 3 : nk - 1;
+    const uint8_t* bk = b_base + (int64_t)kb * kRowBytes;
+    const uint8_t* ak = a_base + (int64_t)ka * kRowBytes;
+    const uint32_t lb = lds0 + a_at + wave * (GB * 1024);
+    const uint32_t la = lds0 + b_at + wave * (GA * 1024);
+    // the next slab pair sits two slots further round the ring
+    const uint32_t a_to = a_at + 2 * kSlot < kRingSlots * kSlot ? a_at + 2 * kSlot : a_at + 2 * kSlot - kRingSlots * kSlot;
+    const uint32_t b_to = b_at + 2 * kSlot < kRingSlots * kSlot ? b_at + 2 * kSlot : b_at + 2 * kSlot - kRingSlots * kSlot;
+#pragma unroll
+    for (int v = 0; v < 4; ++v) {
+      a_fr[v] += a_to - a_at;
+      b_fr[v] += b_to - b_at;
+    }
+    a_at = a_to;
+    b_at = b_to;
     constexpr int kMfma = FM * FN, kLoads = GA + GB, kReads = FM + FN;
     // loads are spread over all MFMAs, fragment reads over the later ones
     constexpr int kReadFrom = kMfma >= 2 * kReads ? kMfma / 4 : 0;
@@ -386,53 +362,45 @@ __device__ __forceinline__ void run_tile(const TileContext& cx, const TileRef& t
         const int slot = ni * FM + mi;
         acc[ni][mi] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bf1[ni], af1[mi], acc[ni][mi], 0, 0, 0);
 #pragma unroll
-        for (int g = 0; g < GA; ++g)
-          if (g * kMfma / kLoads == slot) load_group(ak, a_off[g], la + g * 1024);
-#pragma unroll
         for (int g = 0; g < GB; ++g)
-          if ((GA + g) * kMfma / kLoads == slot) load_group(bk, b_off[g], lb + g * 1024);
+          if (g * kMfma / kLoads == slot) load_group(bk, b_off[g], lb + g * 1024);
+#pragma unroll
+        for (int g = 0; g < GA; ++g)
+          if ((GB + g) * kMfma / kLoads == slot) load_group(ak, a_off[g], la + g * 1024);
 #pragma unroll
         for (int r = 0; r < FM; ++r)
           if (kReadFrom + r * (kMfma - kReadFrom) / kReads == slot)
-            af0[r] = lds_read_frag(a_fr[(r & 1) << 1] + (S ^ 1) * T::kABytes + r * (32 * kRowBytes));
+            af0[r] = lds_read_frag(a_fr[(r & 1) << 1] + r * (32 * kRowBytes));
 #pragma unroll
         for (int r = 0; r < FN; ++r)
           if (kReadFrom + (FM + r) * (kMfma - kReadFrom) / kReads == slot)
-            bf0[r] = lds_read_frag(b_fr[(r & 1) << 1] + (S ^ 1) * T::kBBytes + r * (32 * kRowBytes));
-        if (slot == kMfma - 1) {
-          const int kw = kt + 2 + kWarmAhead;
-          warm_stage(kw < nk ? kw : nk - 1);
-        }
+            bf0[r] = lds_read_frag(b_fr[(r & 1) << 1] + r * (32 * kRowBytes));
       }
     }
   };
-  auto stage_body = [&](auto stage_tag, int kt) {
-    constexpr int S = decltype(stage_tag)::value;
-    read_frags(af1, bf1, S, 1);
+  for (int kt = 0; kt < nk; ++kt) {
+    read_frags(af1, bf1, 1);
     mfma_all(af0, bf0);
     interleave_mfma_dsread<FM * FN, FM + FN>();
-    read_frags(af0, bf0, S, 2);
+    read_frags(af0, bf0, 2);
     mfma_all(af1, bf1);
     interleave_mfma_dsread<FM * FN, FM + FN>();
-    read_frags(af1, bf1, S, 3);
+    read_frags(af1, bf1, 3);
     mfma_all(af0, bf0);
     interleave_mfma_dsread<FM * FN, FM + FN>();
-    // Wait for this wave's own tile loads before the barrier; the compiler does
-    // not count them (see load_group).  The kWarmLoads warm-up loads issued
-    // behind them may stay in flight: loads return in order.
-    if constexpr (kWarmLoads == 0) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    else if constexpr (kWarmLoads == 1) asm volatile("s_waitcnt vmcnt(1)" ::: "memory");
-    else asm volatile("s_waitcnt vmcnt(2)" ::: "memory");
-    __syncthreads();     // stage S fully read by everyone; the other stage has landed
-    last_step(stage_tag, kt);
-  };
-  int kt = 0;
-  for (; kt + 1 < nk; kt += 2) {
-    stage_body(std::integral_constant<int, 0>{}, kt);
-    stage_body(std::integral_constant<int, 1>{}, kt + 1);
+    // Wait for this wave's own loads of slab pair kt+1 before the barrier; the
+    // compiler does not count them (see load_group).  The GA loads of A slab
+    // kt+2, issued last, may stay in flight: loads return in order.
+    static_assert(GA == 8 || GA == 4, "explicit vmcnt below");
+    if constexpr (GA == 8) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+    else asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+    __syncthreads();     // slab pair kt fully read by everyone; pair kt+1 has landed
+    last_step(kt);
   }
-  if (kt < nk) stage_body(std::integral_constant<int, 0>{}, kt);
-  __syncthreads();       // the next tile's prologue overwrites both stages
+  // The repeated loads of the last K steps must not land on top of the next
+  // tile's first slabs.
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();       // the next tile's prologue overwrites the ring
   if (tr != nullptr) tr[2] = wall_clock64();
   between();
 
@@ -476,7 +444,6 @@ __global__ __launch_bounds__(kGemmThreads, 1) void ag_matmul_kernel(
   cx.lds0 = lds_offset_of(lds);
   cx.N = s.N;
   cx.c = c;
-  uint32_t warm_scrap = 0;
 
   // Source rows of a tile: the local shard, or the gathered buffer once the comm
   // block's flag is up.
@@ -521,10 +488,10 @@ __global__ __launch_bounds__(kGemmThreads, 1) void ag_matmul_kernel(
       }
     };
     if constexpr (BN == 256) {
-      if (tile.cols != BN) run_tile<BM, BN / 2>(cx, tile, a_base, b_base, warm_scrap, preloaded, between);
-      else run_tile<BM, BN>(cx, tile, a_base, b_base, warm_scrap, preloaded, between);
+      if (tile.cols != BN) run_tile<BM, BN / 2>(cx, tile, a_base, b_base, preloaded, between);
+      else run_tile<BM, BN>(cx, tile, a_base, b_base, preloaded, between);
     } else {
-      run_tile<BM, BN>(cx, tile, a_base, b_base, warm_scrap, preloaded, between);
+      run_tile<BM, BN>(cx, tile, a_base, b_base, preloaded, between);
     }
     if (cx.tr != nullptr) cx.tr[3] = wall_clock64();
     have = have_next;
@@ -533,10 +500,6 @@ __global__ __launch_bounds__(kGemmThreads, 1) void ag_matmul_kernel(
     b_base = b_next;
     preloaded = true;
   }
-  // Drain the warm-up loads and give the scrap register a use the compiler
-  // cannot remove (K is never negative).
-  asm volatile("s_waitcnt vmcnt(0)" : "+v"(warm_scrap) : : "memory");
-  if (s.K < 0) status[3] = warm_scrap;
 }
 
 static int pick_tile(int M, int N, int comm_block_m, int& BM, int& BN) {
