@@ -143,17 +143,6 @@ __device__ __forceinline__ void load_group(const uint8_t* base, uint32_t voff, u
                : "memory", "m0");
 }
 
-// Scheduling hint: spread NDS LDS reads evenly under NMFMA matrix instructions.
-template <int NMFMA, int NDS>
-__device__ __forceinline__ void interleave_mfma_dsread() {
-  constexpr int kPer = NMFMA / NDS;     // MFMAs ahead of each LDS read
-#pragma unroll
-  for (int i = 0; i < NDS; ++i) {
-    __builtin_amdgcn_sched_group_barrier(0x008, kPer, 0);   // MFMA
-    __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);      // DS read
-  }
-}
-
 // LDS holds a ring of five slots.  A K-slab of A and a K-slab of B take one slot each,
 // in the order A0 B0 A1 B1 A2 ..., so slab number i lives in slot i % 5: the two slabs
 // of the K step being multiplied, and up to three slabs that are landing.
@@ -182,7 +171,7 @@ struct TileContext {
   uint64_t* tr;                  // trace record of this tile or null
 };
 
-// The first five slabs of a tile (A0 B0 A1 B1 A2), global -> ring slots 0..4, no wait.
+// The first four slabs of a tile (A0 B0 A1 B1), global -> ring slots 0..3, no wait.
 // Issued either at the start of the tile or, for every tile but a workgroup's first,
 // by the previous tile between its K loop and its epilogue, so that the loads fly
 // while the previous tile's results are being stored.  Slabs past the end of K repeat
@@ -196,7 +185,7 @@ __device__ __forceinline__ void issue_prologue(const TileContext& cx, const uint
   asm volatile("" : "+v"(ln));
   const int u = (ln & 7) ^ (ln >> 3);
 #pragma unroll
-  for (int idx = 0; idx < kRingSlots; ++idx) {
+  for (int idx = 0; idx < 4; ++idx) {
     const int k = (idx >> 1) < cx.nk ? (idx >> 1) : cx.nk - 1;
     const uint32_t dst = cx.lds0 + idx * T::kSlotBytes;
     if ((idx & 1) == 0) {
@@ -221,7 +210,7 @@ __device__ __forceinline__ void issue_prologue(const TileContext& cx, const uint
 }
 
 // One output tile: C[row0 .. +BM, col0 .. +BN] = A rows (at a_base) x B rows (at b_base)^T.
-// `preloaded`: the tile's first five slabs are already on their way into LDS.
+// `preloaded`: the tile's first four slabs are already on their way into LDS.
 // `between` runs after the K loop, when LDS is free again, and before the results
 // are stored: the place to start the next tile's loads.
 template <int BM, int BN, typename Between>
@@ -300,15 +289,7 @@ __device__ __forceinline__ void run_tile(const TileContext& cx, const TileRef& t
     for (int ni = 0; ni < FN; ++ni)
       bf[ni] = lds_read_frag(b_fr[kk ^ ((ni & 1) << 1)] + ni * (32 * kRowBytes));
   };
-  auto mfma_all = [&](const bf16x8 (&af)[FM], const bf16x8 (&bf)[FN]) {
-#pragma unroll
-    for (int ni = 0; ni < FN; ++ni)
-#pragma unroll
-      for (int mi = 0; mi < FM; ++mi)
-        acc[ni][mi] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bf[ni], af[mi], acc[ni][mi], 0, 0, 0);
-  };
-
-  // Prologue: five slabs in flight, then the first fragments.  The wait is for
+  // Prologue: four slabs in flight, then the first fragments.  The wait is for
   // everything: loads and the previous tile's stores do not retire in one order.
   if (!preloaded) issue_prologue<BM, BN>(cx, a_base, b_base, b_last);
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -321,25 +302,50 @@ __device__ __forceinline__ void run_tile(const TileContext& cx, const TileRef& t
   bf16x8 af0[FM], bf0[FN], af1[FM], bf1[FN];
   read_frags(af0, bf0, 0);
 
-  // Last K step of slab pair kt, issued right behind the barrier.  Its
-  // fragments are already in registers, so the MFMAs start at once; slotted in
-  // between them are
-  //   * the loads of B slab kt+2 into the slot A slab kt just left: they must
-  //     have landed by the next barrier, one slab pair (64 MFMAs) from now;
-  //   * the loads of A slab kt+3 into the slot of B slab kt: two slab pairs of
-  //     time.  Only half of a K step's bytes are ever on the short deadline,
-  //     which the 2.5 slab pairs of LDS buy;
-  //   * the first fragment reads of slab pair kt+1.
-  // There is one code path: past the end of K the loads repeat the last slab
-  // (into a slot nobody reads any more) rather than being branched around,
-  // which keeps the accumulators in place across the whole loop body.
+  // The loads of a K step's 64 KiB are spread over all of its MFMAs: a burst
+  // would fill the memory pipeline's queue, and a wave that cannot issue its
+  // load cannot issue the MFMA behind it either.
+  //   * K steps 0-2 of slab pair kt carry the loads of A slab kt+2, into the
+  //     slot that B slab kt-1 left at the previous barrier (slot 4 at kt = 0):
+  //     they have until the barrier of pair kt+1, more than a slab pair away;
+  //   * the last K step, behind the barrier, carries the loads of B slab kt+2
+  //     into the slot A slab kt has just left: due at the next barrier, one
+  //     slab pair (64 MFMAs) from now.  Only half of a K step's bytes are ever
+  //     on that short deadline, which the 2.5 slab pairs of LDS buy.
+  // Past the end of K the loads repeat the last slab (into a slot nobody reads
+  // any more) rather than being branched around: one code path keeps the
+  // accumulators in place across the whole loop body.  All loops below have
+  // constant trip counts, so they unroll fully and every array index is a
+  // compile-time constant; the instruction order is the program order.
+  constexpr int kMfma = FM * FN, kReads = FM + FN;
+  auto early_step = [&](auto step_tag, const bf16x8 (&ua)[FM], const bf16x8 (&ub)[FN],
+                        bf16x8 (&fa)[FM], bf16x8 (&fb)[FN], const uint8_t* ak, uint32_t la) {
+    constexpr int J = decltype(step_tag)::value;      // K step 0, 1 or 2 of the slab pair
+#pragma unroll
+    for (int ni = 0; ni < FN; ++ni) {
+#pragma unroll
+      for (int mi = 0; mi < FM; ++mi) {
+        const int slot = ni * FM + mi;
+        acc[ni][mi] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ub[ni], ua[mi], acc[ni][mi], 0, 0, 0);
+#pragma unroll
+        for (int r = 0; r < FM; ++r)
+          if (r * kMfma / kReads == slot)
+            fa[r] = lds_read_frag(a_fr[(J + 1) ^ ((r & 1) << 1)] + r * (32 * kRowBytes));
+#pragma unroll
+        for (int r = 0; r < FN; ++r)
+          if ((FM + r) * kMfma / kReads == slot)
+            fb[r] = lds_read_frag(b_fr[(J + 1) ^ ((r & 1) << 1)] + r * (32 * kRowBytes));
+#pragma unroll
+        for (int g = 0; g < GA; ++g)
+          if (g * (3 * kMfma) / GA == J * kMfma + slot) load_group(ak, a_off[g], la + g * 1024);
+        __builtin_amdgcn_sched_barrier(0);     // keep this interleaving
+      }
+    }
+  };
   auto last_step = [&](int kt) {
     const int kb = kt + 2 < nk ? kt + 2 : nk - 1;
-    const int ka = kt + 3 < nk ? kt + 3 : nk - 1;
     const uint8_t* bk = b_base + (int64_t)kb * kRowBytes;
-    const uint8_t* ak = a_base + (int64_t)ka * kRowBytes;
     const uint32_t lb = lds0 + a_at + wave * (GB * 1024);
-    const uint32_t la = lds0 + b_at + wave * (GA * 1024);
     // the next slab pair sits two slots further round the ring
     const uint32_t a_to = a_at + 2 * kSlot < kRingSlots * kSlot ? a_at + 2 * kSlot : a_at + 2 * kSlot - kRingSlots * kSlot;
     const uint32_t b_to = b_at + 2 * kSlot < kRingSlots * kSlot ? b_at + 2 * kSlot : b_at + 2 * kSlot - kRingSlots * kSlot;
@@ -350,11 +356,9 @@ __device__ __forceinline__ void run_tile(const TileContext& cx, const TileRef& t
     }
     a_at = a_to;
     b_at = b_to;
-    constexpr int kMfma = FM * FN, kLoads = GA + GB, kReads = FM + FN;
-    // loads are spread over all MFMAs, fragment reads over the later ones
-    constexpr int kReadFrom = kMfma >= 2 * kReads ? kMfma / 4 : 0;
-    // (all loops below have constant trip counts so that they unroll fully and
-    // every array index is a compile-time constant)
+    // the fragment reads of the next slab pair go under the first three quarters
+    // of the MFMAs, so that the last of them has returned when the next K step starts
+    constexpr int kReadSpan = kMfma >= 2 * kReads ? kMfma * 3 / 4 : kMfma;
 #pragma unroll
     for (int ni = 0; ni < FN; ++ni) {
 #pragma unroll
@@ -363,34 +367,31 @@ __device__ __forceinline__ void run_tile(const TileContext& cx, const TileRef& t
         acc[ni][mi] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bf1[ni], af1[mi], acc[ni][mi], 0, 0, 0);
 #pragma unroll
         for (int g = 0; g < GB; ++g)
-          if (g * kMfma / kLoads == slot) load_group(bk, b_off[g], lb + g * 1024);
-#pragma unroll
-        for (int g = 0; g < GA; ++g)
-          if ((GB + g) * kMfma / kLoads == slot) load_group(ak, a_off[g], la + g * 1024);
+          if (g * kMfma / GB == slot) load_group(bk, b_off[g], lb + g * 1024);
 #pragma unroll
         for (int r = 0; r < FM; ++r)
-          if (kReadFrom + r * (kMfma - kReadFrom) / kReads == slot)
+          if (r * kReadSpan / kReads == slot)
             af0[r] = lds_read_frag(a_fr[(r & 1) << 1] + r * (32 * kRowBytes));
 #pragma unroll
         for (int r = 0; r < FN; ++r)
-          if (kReadFrom + (FM + r) * (kMfma - kReadFrom) / kReads == slot)
+          if ((FM + r) * kReadSpan / kReads == slot)
             bf0[r] = lds_read_frag(b_fr[(r & 1) << 1] + r * (32 * kRowBytes));
+        __builtin_amdgcn_sched_barrier(0);
       }
     }
   };
   for (int kt = 0; kt < nk; ++kt) {
-    read_frags(af1, bf1, 1);
-    mfma_all(af0, bf0);
-    interleave_mfma_dsread<FM * FN, FM + FN>();
-    read_frags(af0, bf0, 2);
-    mfma_all(af1, bf1);
-    interleave_mfma_dsread<FM * FN, FM + FN>();
-    read_frags(af1, bf1, 3);
-    mfma_all(af0, bf0);
-    interleave_mfma_dsread<FM * FN, FM + FN>();
-    // Wait for this wave's own loads of slab pair kt+1 before the barrier; the
-    // compiler does not count them (see load_group).  The GA loads of A slab
-    // kt+2, issued last, may stay in flight: loads return in order.
+    const int ka = kt + 2 < nk ? kt + 2 : nk - 1;
+    const uint8_t* ak = a_base + (int64_t)ka * kRowBytes;
+    // four slots on from A slab kt = one slot back = where B slab kt-1 was
+    const uint32_t a_dst = a_at >= kSlot ? a_at - kSlot : a_at + (kRingSlots - 1) * kSlot;
+    const uint32_t la = lds0 + a_dst + wave * (GA * 1024);
+    early_step(std::integral_constant<int, 0>{}, af0, bf0, af1, bf1, ak, la);
+    early_step(std::integral_constant<int, 1>{}, af1, bf1, af0, bf0, ak, la);
+    early_step(std::integral_constant<int, 2>{}, af0, bf0, af1, bf1, ak, la);
+    // Wait for this wave's own loads of B slab kt+1 (and everything older) before
+    // the barrier; the compiler does not count them (see load_group).  The GA
+    // loads of A slab kt+2, issued last, may stay in flight: loads return in order.
     static_assert(GA == 8 || GA == 4, "explicit vmcnt below");
     if constexpr (GA == 8) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
     else asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
