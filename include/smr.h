@@ -159,7 +159,7 @@ int smr_all_gather_with_progress(const uint64_t* buffer_ptrs_dev, void* a_out_de
 
 /* Pacing of the producer: the first `fast_chunks` chunks are copied by all
  * workgroups, the remaining ones by `slow_workgroups` of them (0 = all, i.e. no
- * pacing).  Default 2 and 14.  No reference counterpart (copy engines pace
+ * pacing).  Default 3 and 16.  No reference counterpart (copy engines pace
  * themselves by link speed). */
 int smr_set_gather_pacing(int fast_chunks, int slow_workgroups);
 

@@ -126,6 +126,23 @@ __device__ __forceinline__ uint32_t lds_offset_of(const void* p) {
 __device__ __forceinline__ bf16x8 lds_read_frag(uint32_t addr) {
   return *reinterpret_cast<LdsFrag*>((uintptr_t)addr);
 }
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ void lds_write_b64(uint32_t addr, u32x2 v) {
+  *reinterpret_cast<__attribute__((address_space(3))) u32x2*>((uintptr_t)addr) = v;
+}
+__device__ __forceinline__ u32x4 lds_read_b128(uint32_t addr) {
+  return *reinterpret_cast<__attribute__((address_space(3))) const u32x4*>((uintptr_t)addr);
+}
+
+// A pointer that is the same in every lane, said so that it is kept in scalar
+// registers (the tile loads take their base address from there).
+__device__ __forceinline__ const uint8_t* uniform_ptr(const uint8_t* p) {
+  const uint64_t v = (uint64_t)(uintptr_t)p;
+  const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v);
+  const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+  return (const uint8_t*)(uintptr_t)(((uint64_t)hi << 32) | lo);
+}
 
 // One wave instruction of a direct-to-LDS tile load: 64 lanes x 16 B land at
 // lds_dst + lane*16 (one 8-row group, 1 KiB); `voff` is the lane's byte offset
@@ -177,9 +194,11 @@ struct TileContext {
 // while the previous tile's results are being stored.  Slabs past the end of K repeat
 // the last one; nobody reads them.
 template <int BM, int BN>
-__device__ __forceinline__ void issue_prologue(const TileContext& cx, const uint8_t* a_base,
-                                               const uint8_t* b_base, int b_last) {
+__device__ __forceinline__ void issue_prologue(const TileContext& cx, const uint8_t* a_rows,
+                                               const uint8_t* b_rows, int b_last) {
   using T = GemmTile<BM, BN>;
+  const uint8_t* a_base = uniform_ptr(a_rows);
+  const uint8_t* b_base = uniform_ptr(b_rows);
   constexpr int GA = T::GA, GB = T::GB;
   int ln = cx.lane;
   asm volatile("" : "+v"(ln));
@@ -215,9 +234,11 @@ __device__ __forceinline__ void issue_prologue(const TileContext& cx, const uint
 // are stored: the place to start the next tile's loads.
 template <int BM, int BN, typename Between>
 __device__ __forceinline__ void run_tile(const TileContext& cx, const TileRef& tile,
-                                         const uint8_t* a_base, const uint8_t* b_base,
+                                         const uint8_t* a_rows, const uint8_t* b_rows,
                                          bool preloaded, Between&& between) {
   using T = GemmTile<BM, BN>;
+  const uint8_t* a_base = uniform_ptr(a_rows);
+  const uint8_t* b_base = uniform_ptr(b_rows);
   constexpr int WM = T::WM, WN = T::WN, FM = T::FM, FN = T::FN, GA = T::GA, GB = T::GB;
   constexpr uint32_t kSlot = T::kSlotBytes;
   const int lane = cx.lane, wave = cx.wave;
@@ -405,28 +426,44 @@ __device__ __forceinline__ void run_tile(const TileContext& cx, const TileRef& t
   if (tr != nullptr) tr[2] = wall_clock64();
   between();
 
-  // D[n][m]: lane holds row m = lane & 31 and, per group of 4 registers, the 4
-  // consecutive columns g*8 + (lane >> 5)*4 .. +3 of the 32x32 fragment.
+  // Epilogue.  D[n][m]: a lane holds row m = lane & 31 of a 32x32 fragment and, per
+  // group g of 4 registers, the 4 consecutive columns g*8 + (lane >> 5)*4 .. +3.
+  // Stored from there, a wave instruction would touch 32 rows with 16 bytes each.
+  // Instead each wave turns 32 rows of its tile at a time through its own quarter of
+  // ring slot 4 (the only slot the next tile's early loads leave alone) and stores
+  // whole rows: 16 bytes per lane, WN*2 contiguous bytes per row.  Chunk c of row r
+  // sits at position c ^ (r mod chunks-per-row), so neither side has more than
+  // two-way bank conflicts.  The region is private to the wave and a wave's LDS
+  // operations execute in order, so no barrier is needed.
+  constexpr int kChunks = WN / 8;                 // 16-byte chunks per wave-tile row
+  constexpr int kRowsPerStore = 64 / kChunks;
+  const uint32_t turn = lds0 + (kRingSlots - 1) * kSlot + wave * (32 * WN * 2);
+  const int wr_row = ln & 31;
+  const int rd_row = ln / kChunks, rd_chunk = ln % kChunks;
 #pragma unroll
   for (int mi = 0; mi < FM; ++mi) {
-    const int m = tile.row0 + wm * WM + mi * 32 + (lane & 31);
-    uint8_t* c_row = c + ((int64_t)m * s.N) * 2;
 #pragma unroll
     for (int ni = 0; ni < FN; ++ni) {
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
-        const int n = tile.col0 + wn * WN + ni * 32 + g * 8 + half * 4;
-        if (n < s.N) {
-          uint2 v;
-          v.x = pack_bf16x2(acc[ni][mi][g * 4 + 0], acc[ni][mi][g * 4 + 1]);
-          v.y = pack_bf16x2(acc[ni][mi][g * 4 + 2], acc[ni][mi][g * 4 + 3]);
-          *reinterpret_cast<uint2*>(c_row + (int64_t)n * 2) = v;
-        }
+        u32x2 v;
+        v.x = pack_bf16x2(acc[ni][mi][g * 4 + 0], acc[ni][mi][g * 4 + 1]);
+        v.y = pack_bf16x2(acc[ni][mi][g * 4 + 2], acc[ni][mi][g * 4 + 3]);
+        const int chunk = ni * 4 + g;
+        lds_write_b64(turn + wr_row * (WN * 2) + (((chunk ^ wr_row) & (kChunks - 1)) << 4) + half * 8, v);
       }
-      // one fragment at a time: keeps the accumulator read-out from flooding
-      // the vector registers
-      __builtin_amdgcn_sched_barrier(0);
     }
+#pragma unroll
+    for (int i = 0; i < 32 / kRowsPerStore; ++i) {
+      const int r = i * kRowsPerStore + rd_row;
+      const u32x4 v = lds_read_b128(turn + r * (WN * 2) + (((rd_chunk ^ r) & (kChunks - 1)) << 4));
+      const int m = tile.row0 + wm * WM + mi * 32 + r;
+      const int n = tile.col0 + wn * WN + rd_chunk * 8;
+      if (n < s.N) *reinterpret_cast<u32x4*>(c + ((int64_t)m * s.N + n) * 2) = v;
+    }
+    // one 32-row band at a time: keeps the accumulator read-out from flooding
+    // the vector registers
+    __builtin_amdgcn_sched_barrier(0);
   }
 }
 

@@ -26,8 +26,8 @@ constexpr int kGatherThreads = 1024;
 constexpr int kGatherDefaultWorkgroups = 8;
 // Pacing (smr_set_gather_pacing): chunks copied at full width, workgroups that stay
 // for the rest.
-static int g_gather_fast_chunks = 2;
-static int g_gather_slow_workgroups = 14;
+static int g_gather_fast_chunks = 3;
+static int g_gather_slow_workgroups = 16;
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef __attribute__((address_space(1))) u32x4 GlobalVec;

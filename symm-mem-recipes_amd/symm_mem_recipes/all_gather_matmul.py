@@ -108,14 +108,17 @@ def all_gather_matmul_tma_persistent(a_shard: torch.Tensor, b: torch.Tensor, a_o
             _lib.check(grid, "all_gather_matmul")
         cus = torch.cuda.get_device_properties(device).multi_processor_count
         producer_wgs = max(8, min(MAX_PRODUCER_WORKGROUPS, cus - grid))
-        with torch.cuda.stream(backend):
-            all_gather_with_progress(a_out, a_shard, progress, splits_per_rank, producer_wgs)
 
+    # The GEMM goes first: its first tiles are local rows and need no flag, so the
+    # producer's launch latency is hidden behind them instead of delaying the GEMM.
+    # (The backend stream waits for what preceded the GEMM, not for the GEMM.)
     rc = lib.smr_ag_matmul(a_shard.data_ptr(), a_out.data_ptr(), b.data_ptr(), c_out.data_ptr(),
                            progress_ptr, M, N, K, rank, world_size, COMM_BLOCK_SIZE_M, status_ptr,
                            current.cuda_stream)
     _lib.check(rc, "all_gather_matmul")
     if not mm_only:
+        with torch.cuda.stream(backend):
+            all_gather_with_progress(a_out, a_shard, progress, splits_per_rank, producer_wgs)
         current.wait_stream(backend)
     return c_out
 
