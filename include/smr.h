@@ -183,6 +183,11 @@ int smr_ag_matmul(const void* a_shard_dev, const void* a_out_dev, const void* b_
 int smr_ag_matmul_schedule(int M, int N, int K, int rank, int world_size, int comm_block_m,
                            int gated, int32_t* out_records, int max_tiles);
 
+/* Tuning knob of the gated schedule: the first `head` and the last `tail` comm blocks
+ * of the ring order are computed in tiles of half the width.  Both -1 (the default)
+ * lets the library choose.  No reference counterpart. */
+int smr_set_ag_matmul_halves(int head, int tail);
+
 /* Workgroups smr_ag_matmul launches on the current device for this shape; a
  * gated launch (progress_dev != NULL) keeps at least 8 compute units free for the
  * producer, whose workgroup count should not exceed the number left free.

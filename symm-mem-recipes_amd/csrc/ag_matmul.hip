@@ -4,7 +4,8 @@
 //   * persistent grid, one 256-thread workgroup per CU; a workgroup computes
 //     BM x BN output tiles (256x256 by default), 4 waves in a 2x2 arrangement, so
 //     a wave owns a (BM/2)x(BN/2) block held in fp32 accumulators and built from
-//     v_mfma_f32_32x32x16_bf16;
+//     v_mfma_f32_16x16x32_bf16 (the 32x32x16 form computes the same in as many cycles
+//     but draws more power, and the clock of a GEMM this size is power-limited);
 //   * both operands are K-contiguous, so a tile's K-slab (rows x 64 bf16 = 128 B
 //     per row) is brought straight from global memory into LDS with 128-bit
 //     direct-to-LDS loads (no staging registers), two stages deep: the loads of
@@ -29,7 +30,7 @@
 namespace smr {
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
-typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef __attribute__((address_space(3))) void LdsVoid;
 typedef __attribute__((address_space(1))) void GlobalVoid;
 
@@ -168,7 +169,7 @@ constexpr int kRingSlots = 5;
 template <int BM, int BN>
 struct GemmTile {
   static constexpr int WM = BM / 2, WN = BN / 2;        // wave tile (2 x 2 waves)
-  static constexpr int FM = WM / 32, FN = WN / 32;      // 32x32 fragments per wave tile
+  static constexpr int FM = WM / 16, FN = WN / 16;      // 16x16 fragments per wave tile
   static constexpr int GA = BM / 32, GB = BN / 32;      // 8-row load groups per wave and slab
   // BN <= BM in every configuration; a slot takes the larger slab, which also lets a
   // half-width tile share the ring (and the next tile's early loads) with a full one.
@@ -243,7 +244,6 @@ __device__ __forceinline__ void run_tile(const TileContext& cx, const TileRef& t
   constexpr uint32_t kSlot = T::kSlotBytes;
   const int lane = cx.lane, wave = cx.wave;
   const int wm = wave >> 1, wn = wave & 1;
-  const int half = lane >> 5;
   const uint32_t row_stride = cx.row_stride;
   const int nk = cx.nk;
   const uint32_t lds0 = cx.lds0;
@@ -257,19 +257,21 @@ __device__ __forceinline__ void run_tile(const TileContext& cx, const TileRef& t
   // in the middle of the K loop.
   int ln = lane;
   asm volatile("" : "+v"(ln));
-  // ---- per-lane fragment read addresses.  Row r = w*W + f*32 + (ln & 31)
-  // has swizzle ((lane & 7) ^ ((ln >> 3) & 3)) ^ ((f & 1) << 2); K step kk wants
-  // chunk 2*kk + half.  Hence position = t ^ (v << 1) with the per-lane constant
-  // t = half ^ (lane & 7) ^ ((ln >> 3) & 3) and v = kk ^ ((f & 1) << 1): four
-  // variants per operand, the fragment row is an immediate offset.  The addresses
-  // point into the slots of the slab pair being read (slots 0 and 1 at first) and
+  // ---- per-lane fragment read addresses.  A 16x16x32 MFMA operand is 16 rows x 32
+  // K: lane l holds row l & 15 and the 8 K values (one 16-byte chunk) number
+  // l >> 4 of the four.  Row r = w*W + f*16 + (l & 15) of the slab has swizzle
+  // (l & 7) ^ ((l >> 3) & 1) ^ ((f & 3) << 1); K step kk (0 or 1) wants chunk
+  // 4*kk + (l >> 4).  Hence position = t ^ (v << 1) with the per-lane constant
+  // t = (l >> 4) ^ (l & 7) ^ ((l >> 3) & 1) and v = 2*kk ^ (f & 3): four variants
+  // per operand, the fragment row is an immediate offset.  The addresses point
+  // into the slots of the slab pair being read (slots 0 and 1 at first) and
   // move around the ring by a uniform amount once per slab pair.
-  const int t = (ln >> 5) ^ (ln & 7) ^ ((ln >> 3) & 3);
+  const int t = (ln >> 4) ^ (ln & 7) ^ ((ln >> 3) & 1);
   uint32_t a_fr[4], b_fr[4];
 #pragma unroll
   for (int v = 0; v < 4; ++v) {
-    a_fr[v] = lds0 + (uint32_t)((wm * WM + (ln & 31)) * kRowBytes + ((t ^ (v << 1)) << 4));
-    b_fr[v] = lds0 + kSlot + (uint32_t)((wn * WN + (ln & 31)) * kRowBytes + ((t ^ (v << 1)) << 4));
+    a_fr[v] = lds0 + (uint32_t)((wm * WM + (ln & 15)) * kRowBytes + ((t ^ (v << 1)) << 4));
+    b_fr[v] = lds0 + kSlot + (uint32_t)((wn * WN + (ln & 15)) * kRowBytes + ((t ^ (v << 1)) << 4));
   }
   uint32_t a_at = 0, b_at = kSlot;       // ring offsets of the slab pair being read
 
@@ -294,76 +296,77 @@ __device__ __forceinline__ void run_tile(const TileContext& cx, const TileRef& t
     b_off[j] = (uint32_t)r * row_stride + (uint32_t)((u ^ (q & 7)) << 4);
   }
 
-  f32x16 acc[FN][FM];
+  f32x4 acc[FN][FM];
 #pragma unroll
   for (int ni = 0; ni < FN; ++ni)
 #pragma unroll
     for (int mi = 0; mi < FM; ++mi)
 #pragma unroll
-      for (int e = 0; e < 16; ++e) acc[ni][mi][e] = 0.0f;
+      for (int e = 0; e < 4; ++e) acc[ni][mi][e] = 0.0f;
 
   auto read_frags = [&](bf16x8 (&af)[FM], bf16x8 (&bf)[FN], int kk) {
 #pragma unroll
     for (int mi = 0; mi < FM; ++mi)
-      af[mi] = lds_read_frag(a_fr[kk ^ ((mi & 1) << 1)] + mi * (32 * kRowBytes));
+      af[mi] = lds_read_frag(a_fr[(2 * kk) ^ (mi & 3)] + mi * (16 * kRowBytes));
 #pragma unroll
     for (int ni = 0; ni < FN; ++ni)
-      bf[ni] = lds_read_frag(b_fr[kk ^ ((ni & 1) << 1)] + ni * (32 * kRowBytes));
+      bf[ni] = lds_read_frag(b_fr[(2 * kk) ^ (ni & 3)] + ni * (16 * kRowBytes));
   };
+
   // Prologue: four slabs in flight, then the first fragments.  The wait is for
   // everything: loads and the previous tile's stores do not retire in one order.
   if (!preloaded) issue_prologue<BM, BN>(cx, a_base, b_base, b_last);
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
 
-  // Fragment double buffer: while the MFMAs of K step kk run, the fragments of
-  // step kk+1 are read.  The workgroup barrier sits before the last K step of a
-  // slab pair, right after its last fragment reads: from there on both of its
-  // slots are free.
+  // A slab pair is two K steps of 32.  Fragment double buffer: while the MFMAs
+  // of one K step run, the fragments of the next are read.  The workgroup
+  // barrier sits between the two K steps of a slab pair, right after its last
+  // fragment reads: from there on both of its slots are free.
   bf16x8 af0[FM], bf0[FN], af1[FM], bf1[FN];
   read_frags(af0, bf0, 0);
 
-  // The loads of a K step's 64 KiB are spread over all of its MFMAs: a burst
-  // would fill the memory pipeline's queue, and a wave that cannot issue its
-  // load cannot issue the MFMA behind it either.
-  //   * K steps 0-2 of slab pair kt carry the loads of A slab kt+2, into the
-  //     slot that B slab kt-1 left at the previous barrier (slot 4 at kt = 0):
-  //     they have until the barrier of pair kt+1, more than a slab pair away;
-  //   * the last K step, behind the barrier, carries the loads of B slab kt+2
-  //     into the slot A slab kt has just left: due at the next barrier, one
-  //     slab pair (64 MFMAs) from now.  Only half of a K step's bytes are ever
-  //     on that short deadline, which the 2.5 slab pairs of LDS buy.
+  // The loads of a slab pair's 64 KiB are spread over its MFMAs: a burst would
+  // fill the memory pipeline's queue, and a wave that cannot issue its load
+  // cannot issue the MFMA behind it either.
+  //   * the first K step of slab pair kt carries the loads of A slab kt+2, into
+  //     the slot that B slab kt-1 left at the previous barrier (slot 4 at
+  //     kt = 0): they have until the barrier of pair kt+1, more than a slab
+  //     pair away;
+  //   * the first half of the second K step, behind the barrier, carries the
+  //     loads of B slab kt+2 into the slot A slab kt has just left: due at the
+  //     next barrier, three quarters of a slab pair from now at the least.
+  //     Only half of a slab pair's bytes are ever on that short deadline,
+  //     which the 2.5 slab pairs of LDS buy.
   // Past the end of K the loads repeat the last slab (into a slot nobody reads
   // any more) rather than being branched around: one code path keeps the
   // accumulators in place across the whole loop body.  All loops below have
   // constant trip counts, so they unroll fully and every array index is a
   // compile-time constant; the instruction order is the program order.
   constexpr int kMfma = FM * FN, kReads = FM + FN;
-  auto early_step = [&](auto step_tag, const bf16x8 (&ua)[FM], const bf16x8 (&ub)[FN],
-                        bf16x8 (&fa)[FM], bf16x8 (&fb)[FN], const uint8_t* ak, uint32_t la) {
-    constexpr int J = decltype(step_tag)::value;      // K step 0, 1 or 2 of the slab pair
+  auto first_step = [&](const uint8_t* ak, uint32_t la) {
 #pragma unroll
     for (int ni = 0; ni < FN; ++ni) {
 #pragma unroll
       for (int mi = 0; mi < FM; ++mi) {
         const int slot = ni * FM + mi;
-        acc[ni][mi] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ub[ni], ua[mi], acc[ni][mi], 0, 0, 0);
+        acc[ni][mi] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(bf0[ni], af0[mi], acc[ni][mi], 0, 0, 0);
 #pragma unroll
         for (int r = 0; r < FM; ++r)
           if (r * kMfma / kReads == slot)
-            fa[r] = lds_read_frag(a_fr[(J + 1) ^ ((r & 1) << 1)] + r * (32 * kRowBytes));
+            af1[r] = lds_read_frag(a_fr[2 ^ (r & 3)] + r * (16 * kRowBytes));
 #pragma unroll
         for (int r = 0; r < FN; ++r)
           if ((FM + r) * kMfma / kReads == slot)
-            fb[r] = lds_read_frag(b_fr[(J + 1) ^ ((r & 1) << 1)] + r * (32 * kRowBytes));
+            bf1[r] = lds_read_frag(b_fr[2 ^ (r & 3)] + r * (16 * kRowBytes));
 #pragma unroll
         for (int g = 0; g < GA; ++g)
-          if (g * (3 * kMfma) / GA == J * kMfma + slot) load_group(ak, a_off[g], la + g * 1024);
+          if (g * kMfma / GA == slot) load_group(ak, a_off[g], la + g * 1024);
         __builtin_amdgcn_sched_barrier(0);     // keep this interleaving
       }
     }
   };
-  auto last_step = [&](int kt) {
+  auto second_step = [&](int kt) {
     const int kb = kt + 2 < nk ? kt + 2 : nk - 1;
     const uint8_t* bk = b_base + (int64_t)kb * kRowBytes;
     const uint32_t lb = lds0 + a_at + wave * (GB * 1024);
@@ -379,24 +382,24 @@ __device__ __forceinline__ void run_tile(const TileContext& cx, const TileRef& t
     b_at = b_to;
     // the fragment reads of the next slab pair go under the first three quarters
     // of the MFMAs, so that the last of them has returned when the next K step starts
-    constexpr int kReadSpan = kMfma >= 2 * kReads ? kMfma * 3 / 4 : kMfma;
+    constexpr int kReadSpan = kMfma * 3 / 4;
 #pragma unroll
     for (int ni = 0; ni < FN; ++ni) {
 #pragma unroll
       for (int mi = 0; mi < FM; ++mi) {
         const int slot = ni * FM + mi;
-        acc[ni][mi] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bf1[ni], af1[mi], acc[ni][mi], 0, 0, 0);
+        acc[ni][mi] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(bf1[ni], af1[mi], acc[ni][mi], 0, 0, 0);
 #pragma unroll
         for (int g = 0; g < GB; ++g)
-          if (g * kMfma / GB == slot) load_group(bk, b_off[g], lb + g * 1024);
+          if (g * (kMfma / 2) / GB == slot) load_group(bk, b_off[g], lb + g * 1024);
 #pragma unroll
         for (int r = 0; r < FM; ++r)
           if (r * kReadSpan / kReads == slot)
-            af0[r] = lds_read_frag(a_fr[(r & 1) << 1] + r * (32 * kRowBytes));
+            af0[r] = lds_read_frag(a_fr[r & 3] + r * (16 * kRowBytes));
 #pragma unroll
         for (int r = 0; r < FN; ++r)
           if ((FM + r) * kReadSpan / kReads == slot)
-            bf0[r] = lds_read_frag(b_fr[(r & 1) << 1] + r * (32 * kRowBytes));
+            bf0[r] = lds_read_frag(b_fr[r & 3] + r * (16 * kRowBytes));
         __builtin_amdgcn_sched_barrier(0);
       }
     }
@@ -406,10 +409,7 @@ __device__ __forceinline__ void run_tile(const TileContext& cx, const TileRef& t
     const uint8_t* ak = a_base + (int64_t)ka * kRowBytes;
     // four slots on from A slab kt = one slot back = where B slab kt-1 was
     const uint32_t a_dst = a_at >= kSlot ? a_at - kSlot : a_at + (kRingSlots - 1) * kSlot;
-    const uint32_t la = lds0 + a_dst + wave * (GA * 1024);
-    early_step(std::integral_constant<int, 0>{}, af0, bf0, af1, bf1, ak, la);
-    early_step(std::integral_constant<int, 1>{}, af1, bf1, af0, bf0, ak, la);
-    early_step(std::integral_constant<int, 2>{}, af0, bf0, af1, bf1, ak, la);
+    first_step(ak, lds0 + a_dst + wave * (GA * 1024));
     // Wait for this wave's own loads of B slab kt+1 (and everything older) before
     // the barrier; the compiler does not count them (see load_group).  The GA
     // loads of A slab kt+2, issued last, may stay in flight: loads return in order.
@@ -417,7 +417,7 @@ __device__ __forceinline__ void run_tile(const TileContext& cx, const TileRef& t
     if constexpr (GA == 8) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
     else asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
     __syncthreads();     // slab pair kt fully read by everyone; pair kt+1 has landed
-    last_step(kt);
+    second_step(kt);
   }
   // The repeated loads of the last K steps must not land on top of the next
   // tile's first slabs.
@@ -426,38 +426,39 @@ __device__ __forceinline__ void run_tile(const TileContext& cx, const TileRef& t
   if (tr != nullptr) tr[2] = wall_clock64();
   between();
 
-  // Epilogue.  D[n][m]: a lane holds row m = lane & 31 of a 32x32 fragment and, per
-  // group g of 4 registers, the 4 consecutive columns g*8 + (lane >> 5)*4 .. +3.
-  // Stored from there, a wave instruction would touch 32 rows with 16 bytes each.
-  // Instead each wave turns 32 rows of its tile at a time through its own quarter of
-  // ring slot 4 (the only slot the next tile's early loads leave alone) and stores
-  // whole rows: 16 bytes per lane, WN*2 contiguous bytes per row.  Chunk c of row r
-  // sits at position c ^ (r mod chunks-per-row), so neither side has more than
-  // two-way bank conflicts.  The region is private to the wave and a wave's LDS
-  // operations execute in order, so no barrier is needed.
+  // Epilogue.  D[n][m]: a lane holds row m = lane & 15 of a 16x16 fragment and the 4
+  // consecutive columns (lane >> 4)*4 .. +3.  Stored from there, a wave instruction
+  // would touch 16 rows with 32 bytes each.  Instead each wave turns 32 rows of its
+  // tile at a time through its own quarter of ring slot 4 (the only slot the next
+  // tile's early loads leave alone) and stores whole rows: 16 bytes per lane, WN*2
+  // contiguous bytes per row.  Chunk c of row r sits at position
+  // c ^ (r mod chunks-per-row), which keeps both sides free of bank conflicts.
+  // The region is private to the wave and a wave's LDS operations execute in
+  // order, so no barrier is needed.
   constexpr int kChunks = WN / 8;                 // 16-byte chunks per wave-tile row
   constexpr int kRowsPerStore = 64 / kChunks;
   const uint32_t turn = lds0 + (kRingSlots - 1) * kSlot + wave * (32 * WN * 2);
-  const int wr_row = ln & 31;
   const int rd_row = ln / kChunks, rd_chunk = ln % kChunks;
 #pragma unroll
-  for (int mi = 0; mi < FM; ++mi) {
+  for (int band = 0; band < FM / 2; ++band) {
 #pragma unroll
-    for (int ni = 0; ni < FN; ++ni) {
+    for (int sub = 0; sub < 2; ++sub) {
+      const int wr_row = sub * 16 + (ln & 15);
 #pragma unroll
-      for (int g = 0; g < 4; ++g) {
+      for (int ni = 0; ni < FN; ++ni) {
+        const f32x4 d = acc[ni][band * 2 + sub];
         u32x2 v;
-        v.x = pack_bf16x2(acc[ni][mi][g * 4 + 0], acc[ni][mi][g * 4 + 1]);
-        v.y = pack_bf16x2(acc[ni][mi][g * 4 + 2], acc[ni][mi][g * 4 + 3]);
-        const int chunk = ni * 4 + g;
-        lds_write_b64(turn + wr_row * (WN * 2) + (((chunk ^ wr_row) & (kChunks - 1)) << 4) + half * 8, v);
+        v.x = pack_bf16x2(d[0], d[1]);
+        v.y = pack_bf16x2(d[2], d[3]);
+        const int chunk = ni * 2 + (ln >> 5);
+        lds_write_b64(turn + wr_row * (WN * 2) + (((chunk ^ wr_row) & (kChunks - 1)) << 4) + ((ln >> 4) & 1) * 8, v);
       }
     }
 #pragma unroll
     for (int i = 0; i < 32 / kRowsPerStore; ++i) {
       const int r = i * kRowsPerStore + rd_row;
       const u32x4 v = lds_read_b128(turn + r * (WN * 2) + (((rd_chunk ^ r) & (kChunks - 1)) << 4));
-      const int m = tile.row0 + wm * WM + mi * 32 + r;
+      const int m = tile.row0 + wm * WM + band * 32 + r;
       const int n = tile.col0 + wn * WN + rd_chunk * 8;
       if (n < s.N) *reinterpret_cast<u32x4*>(c + ((int64_t)m * s.N + n) * 2) = v;
     }
@@ -592,6 +593,10 @@ static int cu_count() {
 // find no room while the consumers spin on its flags.
 constexpr int kReservedCus = 8;
 
+// smr_set_ag_matmul_halves: ring positions cut into half tiles at either end of a
+// gated launch, or -1 to let make_schedule choose.
+static int g_force_head = -1, g_force_tail = -1;
+
 static GemmSchedule make_schedule(int M, int N, int K, int rank, int world_size, int comm_block_m,
                                   int cus, bool gated) {
   GemmSchedule s;
@@ -616,6 +621,10 @@ static GemmSchedule make_schedule(int M, int N, int K, int rank, int world_size,
     head.head = 1;
     if (schedule_cost(both) <= base) s = both;
     else if (schedule_cost(head) <= base) s = head;
+    if (g_force_head >= 0 && g_force_tail >= 0 && g_force_head + g_force_tail <= n_comm) {
+      s.head = g_force_head;
+      s.tail = g_force_tail;
+    }
   }
   return s;
 }
@@ -661,6 +670,13 @@ int smr_ag_matmul(const void* a_shard_dev, const void* a_out_dev, const void* b_
     hipLaunchKernelGGL((ag_matmul_kernel<128, 128>), dim3(s.grid), dim3(kGemmThreads), 0, st, a0, a1, b,
                        c, progress_dev, s, lim, status, tb);
   return check_hip(hipGetLastError(), "smr_ag_matmul launch");
+}
+
+int smr_set_ag_matmul_halves(int head, int tail) {
+  if ((head < 0) != (tail < 0)) return smr::fail(SMR_E_INVALID, "smr_set_ag_matmul_halves: both or neither negative");
+  smr::g_force_head = head;
+  smr::g_force_tail = tail;
+  return 0;
 }
 
 int smr_ag_matmul_grid(int M, int N, int K, int world_size, int comm_block_m, int gated) {
