@@ -11,8 +11,8 @@
 //     direct-to-LDS loads (no staging registers), two stages deep: the loads of
 //     slab k+1 are in flight while slab k is multiplied;
 //   * an LDS row is 8 chunks of 16 B; chunk c of row r is stored at position
-//     c ^ s(r), s(r) = (r ^ (r >> 3)) & 7, which makes the 128-bit fragment reads
-//     of 32 consecutive rows hit distinct banks;
+//     c ^ row_swizzle(r), which keeps the 128-bit fragment reads free of bank
+//     conflicts;
 //   * the MFMA is issued with the B fragment as its first operand, so a lane
 //     ends up with 4 consecutive output columns of one row and stores 8 bytes
 //     at a time;
@@ -116,8 +116,16 @@ __host__ __device__ inline int schedule_cost(const GemmSchedule& s) {
          ceil_div(s.tail * half, s.grid);
 }
 
-// Position swizzle of an LDS row.
-__host__ __device__ inline int row_swizzle(int r) { return (r ^ (r >> 3)) & 7; }
+// Position swizzle of an LDS row: chunk c of slab row r is stored at position
+// c ^ row_swizzle(r).  A 128-bit LDS read is served 16 lanes at a time, lanes
+// 8g..8g+7 together with lanes 32+8g..32+8g+7, and those 16 lanes must fall into 16
+// different 16-byte columns of the 256-byte bank row (two slab rows).  In a fragment
+// read they are 8 consecutive rows at two chunks that differ by 2, so the 4 rows of
+// equal parity must differ in swizzle bits 0 and 2: bits 0,1 = row bits 1,2 and
+// bit 2 = row bit 2 ^ row bit 3.
+__host__ __device__ inline int row_swizzle(int r) {
+  return ((r >> 1) & 3) | ((((r >> 2) ^ (r >> 3)) & 1) << 2);
+}
 
 typedef __attribute__((address_space(3))) const bf16x8 LdsFrag;
 
@@ -203,7 +211,7 @@ __device__ __forceinline__ void issue_prologue(const TileContext& cx, const uint
   constexpr int GA = T::GA, GB = T::GB;
   int ln = cx.lane;
   asm volatile("" : "+v"(ln));
-  const int u = (ln & 7) ^ (ln >> 3);
+  const int u = (ln & 7) ^ row_swizzle(ln >> 3);
 #pragma unroll
   for (int idx = 0; idx < 4; ++idx) {
     const int k = (idx >> 1) < cx.nk ? (idx >> 1) : cx.nk - 1;
@@ -213,7 +221,7 @@ __device__ __forceinline__ void issue_prologue(const TileContext& cx, const uint
 #pragma unroll
       for (int j = 0; j < GA; ++j) {
         const int q = cx.wave * GA + j;
-        load_group(ak, (uint32_t)(q * 8 + (ln >> 3)) * cx.row_stride + (uint32_t)((u ^ (q & 7)) << 4),
+        load_group(ak, (uint32_t)(q * 8 + (ln >> 3)) * cx.row_stride + (uint32_t)((u ^ ((q & 1) << 2)) << 4),
                    dst + q * 1024);
       }
     } else {
@@ -223,7 +231,7 @@ __device__ __forceinline__ void issue_prologue(const TileContext& cx, const uint
         const int q = cx.wave * GB + j;
         int r = q * 8 + (ln >> 3);
         r = r < b_last ? r : b_last;
-        load_group(bk, (uint32_t)r * cx.row_stride + (uint32_t)((u ^ (q & 7)) << 4), dst + q * 1024);
+        load_group(bk, (uint32_t)r * cx.row_stride + (uint32_t)((u ^ ((q & 1) << 2)) << 4), dst + q * 1024);
       }
     }
   }
@@ -259,31 +267,29 @@ __device__ __forceinline__ void run_tile(const TileContext& cx, const TileRef& t
   asm volatile("" : "+v"(ln));
   // ---- per-lane fragment read addresses.  A 16x16x32 MFMA operand is 16 rows x 32
   // K: lane l holds row l & 15 and the 8 K values (one 16-byte chunk) number
-  // l >> 4 of the four.  Row r = w*W + f*16 + (l & 15) of the slab has swizzle
-  // (l & 7) ^ ((l >> 3) & 1) ^ ((f & 3) << 1); K step kk (0 or 1) wants chunk
-  // 4*kk + (l >> 4).  Hence position = t ^ (v << 1) with the per-lane constant
-  // t = (l >> 4) ^ (l & 7) ^ ((l >> 3) & 1) and v = 2*kk ^ (f & 3): four variants
-  // per operand, the fragment row is an immediate offset.  The addresses point
-  // into the slots of the slab pair being read (slots 0 and 1 at first) and
+  // l >> 4 of the four, so K step kk (0 or 1) wants chunk 4*kk + (l >> 4) of row
+  // w*W + f*16 + (l & 15), whose swizzle depends on l & 15 only: one address per
+  // operand and K step, the fragment row f is an immediate offset.  The addresses
+  // point into the slots of the slab pair being read (slots 0 and 1 at first) and
   // move around the ring by a uniform amount once per slab pair.
-  const int t = (ln >> 4) ^ (ln & 7) ^ ((ln >> 3) & 1);
-  uint32_t a_fr[4], b_fr[4];
+  uint32_t a_fr[2], b_fr[2];
 #pragma unroll
-  for (int v = 0; v < 4; ++v) {
-    a_fr[v] = lds0 + (uint32_t)((wm * WM + (ln & 15)) * kRowBytes + ((t ^ (v << 1)) << 4));
-    b_fr[v] = lds0 + kSlot + (uint32_t)((wn * WN + (ln & 15)) * kRowBytes + ((t ^ (v << 1)) << 4));
+  for (int kk = 0; kk < 2; ++kk) {
+    const int pos = (4 * kk + (ln >> 4)) ^ row_swizzle(ln & 15);
+    a_fr[kk] = lds0 + (uint32_t)((wm * WM + (ln & 15)) * kRowBytes + (pos << 4));
+    b_fr[kk] = lds0 + kSlot + (uint32_t)((wn * WN + (ln & 15)) * kRowBytes + (pos << 4));
   }
   uint32_t a_at = 0, b_at = kSlot;       // ring offsets of the slab pair being read
 
   // ---- per-lane global offsets of the tile loads.  Load group q = wave*G + j holds
   // rows q*8 .. q*8+7; lane l carries row q*8 + (l >> 3) and the chunk whose swizzled
-  // position is (l & 7): chunk = (l & 7) ^ (l >> 3) ^ (q & 7).
-  const int u = (ln & 7) ^ (ln >> 3);
+  // position is (l & 7): chunk = (l & 7) ^ row_swizzle(q*8 + (l >> 3)).
+  const int u = (ln & 7) ^ row_swizzle(ln >> 3);
   uint32_t a_off[GA];
 #pragma unroll
   for (int j = 0; j < GA; ++j) {
     const int q = wave * GA + j;
-    a_off[j] = (uint32_t)(q * 8 + (ln >> 3)) * row_stride + (uint32_t)((u ^ (q & 7)) << 4);
+    a_off[j] = (uint32_t)(q * 8 + (ln >> 3)) * row_stride + (uint32_t)((u ^ ((q & 1) << 2)) << 4);
   }
   // rows of B past the last column are clamped: they feed outputs that are never stored
   const int b_last = s.N - 1 - tile.col0;
@@ -293,7 +299,7 @@ __device__ __forceinline__ void run_tile(const TileContext& cx, const TileRef& t
     const int q = wave * GB + j;
     int r = q * 8 + (ln >> 3);
     r = r < b_last ? r : b_last;
-    b_off[j] = (uint32_t)r * row_stride + (uint32_t)((u ^ (q & 7)) << 4);
+    b_off[j] = (uint32_t)r * row_stride + (uint32_t)((u ^ ((q & 1) << 2)) << 4);
   }
 
   f32x4 acc[FN][FM];
@@ -307,10 +313,10 @@ __device__ __forceinline__ void run_tile(const TileContext& cx, const TileRef& t
   auto read_frags = [&](bf16x8 (&af)[FM], bf16x8 (&bf)[FN], int kk) {
 #pragma unroll
     for (int mi = 0; mi < FM; ++mi)
-      af[mi] = lds_read_frag(a_fr[(2 * kk) ^ (mi & 3)] + mi * (16 * kRowBytes));
+      af[mi] = lds_read_frag(a_fr[kk] + mi * (16 * kRowBytes));
 #pragma unroll
     for (int ni = 0; ni < FN; ++ni)
-      bf[ni] = lds_read_frag(b_fr[(2 * kk) ^ (ni & 3)] + ni * (16 * kRowBytes));
+      bf[ni] = lds_read_frag(b_fr[kk] + ni * (16 * kRowBytes));
   };
 
   // Prologue: four slabs in flight, then the first fragments.  The wait is for
@@ -344,6 +350,9 @@ __device__ __forceinline__ void run_tile(const TileContext& cx, const TileRef& t
   // constant trip counts, so they unroll fully and every array index is a
   // compile-time constant; the instruction order is the program order.
   constexpr int kMfma = FM * FN, kReads = FM + FN;
+  // the fragment reads of the next K step go under the first three quarters of the
+  // MFMAs, so that the last of them has returned when that step starts
+  constexpr int kReadSpan = kMfma * 3 / 4;
   auto first_step = [&](const uint8_t* ak, uint32_t la) {
 #pragma unroll
     for (int ni = 0; ni < FN; ++ni) {
@@ -353,12 +362,12 @@ __device__ __forceinline__ void run_tile(const TileContext& cx, const TileRef& t
         acc[ni][mi] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(bf0[ni], af0[mi], acc[ni][mi], 0, 0, 0);
 #pragma unroll
         for (int r = 0; r < FM; ++r)
-          if (r * kMfma / kReads == slot)
-            af1[r] = lds_read_frag(a_fr[2 ^ (r & 3)] + r * (16 * kRowBytes));
+          if (r * kReadSpan / kReads == slot)
+            af1[r] = lds_read_frag(a_fr[1] + r * (16 * kRowBytes));
 #pragma unroll
         for (int r = 0; r < FN; ++r)
-          if ((FM + r) * kMfma / kReads == slot)
-            bf1[r] = lds_read_frag(b_fr[2 ^ (r & 3)] + r * (16 * kRowBytes));
+          if ((FM + r) * kReadSpan / kReads == slot)
+            bf1[r] = lds_read_frag(b_fr[1] + r * (16 * kRowBytes));
 #pragma unroll
         for (int g = 0; g < GA; ++g)
           if (g * kMfma / GA == slot) load_group(ak, a_off[g], la + g * 1024);
@@ -374,15 +383,12 @@ __device__ __forceinline__ void run_tile(const TileContext& cx, const TileRef& t
     const uint32_t a_to = a_at + 2 * kSlot < kRingSlots * kSlot ? a_at + 2 * kSlot : a_at + 2 * kSlot - kRingSlots * kSlot;
     const uint32_t b_to = b_at + 2 * kSlot < kRingSlots * kSlot ? b_at + 2 * kSlot : b_at + 2 * kSlot - kRingSlots * kSlot;
 #pragma unroll
-    for (int v = 0; v < 4; ++v) {
-      a_fr[v] += a_to - a_at;
-      b_fr[v] += b_to - b_at;
+    for (int kk = 0; kk < 2; ++kk) {
+      a_fr[kk] += a_to - a_at;
+      b_fr[kk] += b_to - b_at;
     }
     a_at = a_to;
     b_at = b_to;
-    // the fragment reads of the next slab pair go under the first three quarters
-    // of the MFMAs, so that the last of them has returned when the next K step starts
-    constexpr int kReadSpan = kMfma * 3 / 4;
 #pragma unroll
     for (int ni = 0; ni < FN; ++ni) {
 #pragma unroll
@@ -395,11 +401,11 @@ __device__ __forceinline__ void run_tile(const TileContext& cx, const TileRef& t
 #pragma unroll
         for (int r = 0; r < FM; ++r)
           if (r * kReadSpan / kReads == slot)
-            af0[r] = lds_read_frag(a_fr[r & 3] + r * (16 * kRowBytes));
+            af0[r] = lds_read_frag(a_fr[0] + r * (16 * kRowBytes));
 #pragma unroll
         for (int r = 0; r < FN; ++r)
           if ((FM + r) * kReadSpan / kReads == slot)
-            bf0[r] = lds_read_frag(b_fr[r & 3] + r * (16 * kRowBytes));
+            bf0[r] = lds_read_frag(b_fr[0] + r * (16 * kRowBytes));
         __builtin_amdgcn_sched_barrier(0);
       }
     }
