@@ -10,11 +10,13 @@
 // all of the chunk's bytes have been written and released.
 //
 // The grid is small on purpose: the consumer GEMM owns the compute units.  It is
-// also paced: a copy that streams faster than about 0.25 TB/s slows the GEMM next
-// to it more than proportionally (measured: +20 % GEMM time at 0.5 TB/s, nothing
-// at 0.2 TB/s), so only the first chunks - the ones the consumer is about to ask
-// for - are copied by all workgroups; after them all but a few workgroups leave
-// and the rest of the gather trickles in just ahead of the consumer.
+// also paced.  The copy's traffic lengthens the GEMM's L2 misses (a GEMM next to a
+// copy of all eight chunks at 0.75 TB/s takes 12 % longer; a loop of nothing but
+// MFMAs next to the same copy only 2 %, so it is the memory path, not power), and
+// more so the faster the copy runs.  So only the first chunks - the ones the
+// consumer is about to ask for - are copied by all workgroups; after them all but
+// a few workgroups leave and the rest of the gather arrives just ahead of the
+// consumer.
 #include "smr_device.hpp"
 
 namespace smr {

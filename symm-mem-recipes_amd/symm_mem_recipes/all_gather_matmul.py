@@ -46,13 +46,20 @@ def all_gather_with_progress(output: torch.Tensor, inp: torch.Tensor, progress: 
     assert output.is_contiguous() and output.dtype == inp.dtype
 
     counters = torch.zeros(world_size * splits_per_rank, dtype=torch.int32, device=inp.device)
-    lib = _lib.load()
-    rc = lib.smr_all_gather_with_progress(
-        symm_mem.buffer_ptrs_dev, output.data_ptr(), progress.data_ptr(), counters.data_ptr(),
-        rank, world_size, inp.numel() * inp.element_size(), int(splits_per_rank),
-        int(num_workgroups), torch.cuda.current_stream(inp.device).cuda_stream)
-    _lib.check(rc, "all_gather_with_progress")
+    _launch_producer(symm_mem, output, inp, progress, counters, splits_per_rank, num_workgroups,
+                     torch.cuda.current_stream(inp.device).cuda_stream)
     symm_mem.barrier()
+
+
+def _launch_producer(symm_mem, output, inp, progress, counters, splits_per_rank, num_workgroups,
+                     stream_handle) -> None:
+    """The producer kernel on the given stream; ``counters`` (one zeroed int32 per
+    chunk) are its arrival counters."""
+    rc = _lib.load().smr_all_gather_with_progress(
+        symm_mem.buffer_ptrs_dev, output.data_ptr(), progress.data_ptr(), counters.data_ptr(),
+        symm_mem.rank, symm_mem.world_size, inp.numel() * inp.element_size(), int(splits_per_rank),
+        int(num_workgroups), stream_handle)
+    _lib.check(rc, "all_gather_with_progress")
 
 
 def all_gather_matmul_tma_persistent(a_shard: torch.Tensor, b: torch.Tensor, a_out: torch.Tensor,
@@ -96,12 +103,16 @@ def all_gather_matmul_tma_persistent(a_shard: torch.Tensor, b: torch.Tensor, a_o
     if mm_only:
         progress_ptr = 0
     else:
-        progress = torch.zeros(world_size * splits_per_rank, dtype=torch.int32, device=device)
+        # flags and the producer's arrival counters, zeroed by one fill ahead of both kernels
+        chunks = world_size * splits_per_rank
+        flags = torch.zeros(2 * chunks, dtype=torch.int32, device=device)
+        progress, counters = flags[:chunks], flags[chunks:]
         progress_ptr = progress.data_ptr()
         symm_mem.barrier(0)
         backend = _get_backend_stream()
         backend.wait_stream(current)
-        progress.record_stream(backend)
+        flags.record_stream(backend)
+        assert a_out.dtype == a_shard.dtype and a_out.is_contiguous()
         # the producer takes the compute units the GEMM's grid leaves free
         grid = lib.smr_ag_matmul_grid(M, N, K, world_size, COMM_BLOCK_SIZE_M, 1)
         if grid < 0:
@@ -117,8 +128,8 @@ def all_gather_matmul_tma_persistent(a_shard: torch.Tensor, b: torch.Tensor, a_o
                            current.cuda_stream)
     _lib.check(rc, "all_gather_matmul")
     if not mm_only:
-        with torch.cuda.stream(backend):
-            all_gather_with_progress(a_out, a_shard, progress, splits_per_rank, producer_wgs)
+        _launch_producer(symm_mem, a_out, a_shard, progress, counters, splits_per_rank, producer_wgs,
+                         backend.cuda_stream)
         current.wait_stream(backend)
     return c_out
 
