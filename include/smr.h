@@ -36,6 +36,8 @@ extern "C" {
 
 #define SMR_DTYPE_BF16 0
 #define SMR_DTYPE_FP32 1
+#define SMR_DTYPE_BF16_STEPWISE 2 /* bf16 buffers, accumulator rounded to bf16 after every add:
+                                   the reference's add.bf16x2 chain, triton_one_shot_all_reduce.py:36-49,84-89 */
 
 #define SMR_MAX_WORLD_SIZE 8
 #define SMR_STATUS_WORDS 4

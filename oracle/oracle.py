@@ -124,8 +124,13 @@ def reduce_ref_bf16_acc(bufs: Sequence[np.ndarray]) -> np.ndarray:
     n = bufs[0].shape[0]
     acc = np.zeros(n, dtype=np.uint16)
     for b in bufs:
-        s = bf16_bits_to_f32(acc).astype(np.float64) + bf16_bits_to_f32(b).astype(np.float64)
+        with np.errstate(invalid="ignore"):
+            s = bf16_bits_to_f32(acc).astype(np.float64) + bf16_bits_to_f32(b).astype(np.float64)
         acc = _f64_to_bf16_bits(s)
+        # add.bf16x2 returns the canonical NaN 0x7FFF whatever the operands' payloads
+        # (PTX ISA 8.x, "Half Precision Floating-Point Instructions: add"; the CUDA
+        # toolkit is a third-party dependency that is not part of the reference tree)
+        acc = np.where(np.isnan(s), np.uint16(0x7FFF), acc).astype(np.uint16)
     return acc
 
 

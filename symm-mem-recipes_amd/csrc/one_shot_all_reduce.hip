@@ -59,10 +59,40 @@ __device__ __forceinline__ void store_stream(GlobalVec* p, const Vec16& v) {
   __builtin_nontemporal_store(t, p);
 }
 
-template <bool BF16, int WS>
+// One correctly rounded bf16 add, canonical NaN: what add.bf16x2 computes per half
+// (triton_one_shot_all_reduce.py:44-47).  The fp32 sum of two bf16 values is exact
+// when their exponents differ by at most 16; beyond that the smaller one is less
+// than 2^-9 of a bf16 ulp of the larger and no rounding of the fp32 sum can carry
+// the result to another bf16, so rounding the fp32 sum once is the bf16 add.
+__device__ __forceinline__ float add_bf16_step(float acc, float x) {
+  const float s = acc + x;
+  const uint32_t u = __float_as_uint(s);
+  const uint32_t r = (u + 0x7FFFu + ((u >> 16) & 1u)) >> 16;
+  const uint32_t bits = ((u & 0x7FFFFFFFu) > 0x7F800000u) ? 0x7FFFu : r;
+  return __uint_as_float(bits << 16);
+}
+
+// KIND follows the dtype codes: 0 bf16 with an fp32 accumulator, 1 fp32, 2 bf16 with
+// the accumulator rounded to bf16 after every add.
+template <int KIND, int WS>
 __device__ __forceinline__ Vec16 sum_in_rank_order(const Vec16 (&v)[WS]) {
   Vec16 o;
-  if constexpr (BF16) {
+  if constexpr (KIND == SMR_DTYPE_BF16_STEPWISE) {
+    float acc[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc[e] = 0.0f;
+#pragma unroll
+    for (int r = 0; r < WS; ++r) {
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        acc[2 * k] = add_bf16_step(acc[2 * k], bf16_lo(v[r].w[k]));
+        acc[2 * k + 1] = add_bf16_step(acc[2 * k + 1], bf16_hi(v[r].w[k]));
+      }
+    }
+#pragma unroll
+    for (int k = 0; k < 4; ++k)
+      o.w[k] = (__float_as_uint(acc[2 * k]) >> 16) | (__float_as_uint(acc[2 * k + 1]) & 0xFFFF0000u);
+  } else if constexpr (KIND == SMR_DTYPE_BF16) {
     float acc[8];
 #pragma unroll
     for (int e = 0; e < 8; ++e) acc[e] = 0.0f;
@@ -91,7 +121,7 @@ __device__ __forceinline__ Vec16 sum_in_rank_order(const Vec16 (&v)[WS]) {
   return o;
 }
 
-template <bool BF16, int WS, bool WRITE_ALL>
+template <int KIND, int WS, bool WRITE_ALL>
 __global__ __launch_bounds__(kReduceMaxThreads) void one_shot_all_reduce_kernel(
     const uint64_t* __restrict__ buffer_ptrs, const uint64_t* __restrict__ signal_pad_ptrs,
     Vec16* __restrict__ out, int64_t nvec, int rank, int layout, int nblocks, int do_barrier,
@@ -136,7 +166,7 @@ __global__ __launch_bounds__(kReduceMaxThreads) void one_shot_all_reduce_kernel(
     Vec16 v[WS];
 #pragma unroll
     for (int r = 0; r < WS; ++r) v[r] = load_stream(src[r] + i);
-    Vec16 o = sum_in_rank_order<BF16, WS>(v);
+    Vec16 o = sum_in_rank_order<KIND, WS>(v);
     if constexpr (WRITE_ALL) {
 #pragma unroll
       for (int r = 0; r < WS; ++r) store_stream(src[r] + i, o);
@@ -146,27 +176,27 @@ __global__ __launch_bounds__(kReduceMaxThreads) void one_shot_all_reduce_kernel(
   }
 }
 
-template <bool BF16, int WS>
+template <int KIND, int WS>
 static int launch_ws(bool write_all, dim3 grid, int threads, hipStream_t s, const uint64_t* bp, const uint64_t* sp,
                      Vec16* out, int64_t nvec, int rank, int layout, int nblocks, int do_barrier,
                      uint32_t* status) {
   const uint64_t lim = spin_limit_ticks();
   if (write_all)
-    hipLaunchKernelGGL((one_shot_all_reduce_kernel<BF16, WS, true>), grid, dim3(threads), 0, s,
+    hipLaunchKernelGGL((one_shot_all_reduce_kernel<KIND, WS, true>), grid, dim3(threads), 0, s,
                        bp, sp, out, nvec, rank, layout, nblocks, do_barrier, lim, status);
   else
-    hipLaunchKernelGGL((one_shot_all_reduce_kernel<BF16, WS, false>), grid, dim3(threads), 0, s,
+    hipLaunchKernelGGL((one_shot_all_reduce_kernel<KIND, WS, false>), grid, dim3(threads), 0, s,
                        bp, sp, out, nvec, rank, layout, nblocks, do_barrier, lim, status);
   return check_hip(hipGetLastError(), "smr_one_shot_all_reduce launch");
 }
 
-template <bool BF16>
+template <int KIND>
 static int launch_dtype(int ws, bool write_all, dim3 grid, int threads, hipStream_t s, const uint64_t* bp,
                         const uint64_t* sp, Vec16* out, int64_t nvec, int rank, int layout,
                         int nblocks, int do_barrier, uint32_t* status) {
 #define SMR_WS_CASE(W)                                                                          \
   case W:                                                                                       \
-    return launch_ws<BF16, W>(write_all, grid, threads, s, bp, sp, out, nvec, rank, layout, nblocks,     \
+    return launch_ws<KIND, W>(write_all, grid, threads, s, bp, sp, out, nvec, rank, layout, nblocks,     \
                               do_barrier, status);
   switch (ws) {
     SMR_WS_CASE(1) SMR_WS_CASE(2) SMR_WS_CASE(3) SMR_WS_CASE(4)
@@ -192,7 +222,7 @@ int smr_set_reduce_launch(int threads, int max_blocks) {
 }
 
 int smr_reduce_num_blocks(int64_t numel, int dtype) {
-  const int per_vec = dtype == SMR_DTYPE_BF16 ? 8 : 4;
+  const int per_vec = dtype == SMR_DTYPE_FP32 ? 4 : 8;
   if (numel <= 0) return 0;
   const int64_t nvec = numel / per_vec;
   const int threads = smr::reduce_threads_for(nvec);
@@ -206,13 +236,13 @@ int smr_one_shot_all_reduce(const uint64_t* buffer_ptrs_dev, const uint64_t* sig
                             void* out, int64_t numel, int dtype, int rank, int world_size,
                             int write_all, int barrier_mode, uint32_t* status, void* stream) {
   using namespace smr;
-  if (dtype != SMR_DTYPE_BF16 && dtype != SMR_DTYPE_FP32)
-    return fail(SMR_E_INVALID, "smr_one_shot_all_reduce: dtype must be bf16 (0) or fp32 (1)");
+  if (dtype != SMR_DTYPE_BF16 && dtype != SMR_DTYPE_FP32 && dtype != SMR_DTYPE_BF16_STEPWISE)
+    return fail(SMR_E_INVALID, "smr_one_shot_all_reduce: dtype must be bf16 (0), fp32 (1) or stepwise bf16 (2)");
   if (world_size < 1 || world_size > SMR_MAX_WORLD_SIZE)
     return fail(SMR_E_INVALID, "smr_one_shot_all_reduce: world_size must be 1..8");
   if (rank < -1 || rank >= world_size)
     return fail(SMR_E_INVALID, "smr_one_shot_all_reduce: rank out of range");
-  const int per_vec = dtype == SMR_DTYPE_BF16 ? 8 : 4;
+  const int per_vec = dtype == SMR_DTYPE_FP32 ? 4 : 8;
   if (numel < 0 || numel % per_vec != 0)
     return fail(SMR_E_INVALID, "smr_one_shot_all_reduce: The number of elements must be 128-bit aligned.");
   if (buffer_ptrs_dev == nullptr)
@@ -246,9 +276,13 @@ int smr_one_shot_all_reduce(const uint64_t* buffer_ptrs_dev, const uint64_t* sig
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
   Vec16* o = reinterpret_cast<Vec16*>(out);
   if (dtype == SMR_DTYPE_BF16)
-    return launch_dtype<true>(world_size, write_all != 0, dim3(grid), threads, s, buffer_ptrs_dev,
-                              signal_pad_ptrs_dev, o, nvec, rank, layout, nblocks, do_barrier, status);
-  return launch_dtype<false>(world_size, write_all != 0, dim3(grid), threads, s, buffer_ptrs_dev,
+    return launch_dtype<SMR_DTYPE_BF16>(world_size, write_all != 0, dim3(grid), threads, s, buffer_ptrs_dev,
+                                        signal_pad_ptrs_dev, o, nvec, rank, layout, nblocks, do_barrier, status);
+  if (dtype == SMR_DTYPE_BF16_STEPWISE)
+    return launch_dtype<SMR_DTYPE_BF16_STEPWISE>(world_size, write_all != 0, dim3(grid), threads, s,
+                                                 buffer_ptrs_dev, signal_pad_ptrs_dev, o, nvec, rank, layout,
+                                                 nblocks, do_barrier, status);
+  return launch_dtype<SMR_DTYPE_FP32>(world_size, write_all != 0, dim3(grid), threads, s, buffer_ptrs_dev,
                              signal_pad_ptrs_dev, o, nvec, rank, layout, nblocks, do_barrier, status);
 }
 

@@ -14,6 +14,7 @@ LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), LIB_NAME)
 
 DTYPE_BF16 = 0
 DTYPE_FP32 = 1
+DTYPE_BF16_STEPWISE = 2
 BARRIER_NONE = 0
 BARRIER_PROXY = 1
 STATUS_WORDS = 4

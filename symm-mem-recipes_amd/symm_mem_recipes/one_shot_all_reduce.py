@@ -23,7 +23,7 @@ def num_blocks(numel: int, dtype: torch.dtype = torch.bfloat16) -> int:
 
 
 def one_shot_all_reduce(tensor: torch.Tensor, *, barrier: bool = True, write_all: bool = False,
-                        all_ranks: bool = False) -> torch.Tensor:
+                        all_ranks: bool = False, accumulate: str = "fp32") -> torch.Tensor:
     """Sum the symmetric buffers of all ranks element-wise (fp32 accumulator,
     rank order 0..world_size-1) and return the calling rank's result.
 
@@ -34,7 +34,13 @@ def one_shot_all_reduce(tensor: torch.Tensor, *, barrier: bool = True, write_all
                    return the calling rank's buffer (``tensor`` itself).
     ``all_ranks``  run every emulated rank in one launch, each behind the real
                    barrier; returns ``[world_size, *tensor.shape]``.
+    ``accumulate`` "fp32" (default) keeps an fp32 accumulator and rounds once;
+                   "bf16" rounds the accumulator to bf16 after every add, which is
+                   bit for bit the reference's add.bf16x2 chain
+                   (triton_one_shot_all_reduce.py:36-49, 84-89); bf16 tensors only.
     """
+    assert accumulate in ("fp32", "bf16"), "accumulate must be 'fp32' or 'bf16'"
+    assert accumulate == "fp32" or tensor.dtype == torch.bfloat16, "accumulate='bf16' needs a bfloat16 tensor"
     assert tensor.dtype in _DTYPE_CODE, "Only bfloat16 and float32 are supported for now."
     assert (
         tensor.numel() % NUMEL_PER_THREAD[tensor.dtype] == 0
@@ -60,7 +66,7 @@ def one_shot_all_reduce(tensor: torch.Tensor, *, barrier: bool = True, write_all
         symm_mem.signal_pad_ptrs_dev,
         out_ptr,
         tensor.numel(),
-        _DTYPE_CODE[tensor.dtype],
+        _lib.DTYPE_BF16_STEPWISE if accumulate == "bf16" else _DTYPE_CODE[tensor.dtype],
         -1 if all_ranks else symm_mem.rank,
         symm_mem.world_size,
         1 if write_all else 0,

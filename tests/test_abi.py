@@ -54,7 +54,7 @@ def test_reduce_argument_errors_before_launch(lib):
     p = 0x1000
     assert bad(p, p, p, 12, 0, 0, 8, 0, 0, None, None) == -1       # numel % 8
     assert b"128-bit aligned" in lib.smr_last_error_string()
-    assert bad(p, p, p, 16, 2, 0, 8, 0, 0, None, None) == -1       # dtype
+    assert bad(p, p, p, 16, 3, 0, 8, 0, 0, None, None) == -1       # dtype
     assert bad(p, p, p, 16, 0, 8, 8, 0, 0, None, None) == -1       # rank
     assert bad(p, p, p, 16, 0, 0, 9, 0, 0, None, None) == -1       # world size
     assert bad(None, p, p, 16, 0, 0, 8, 0, 0, None, None) == -1    # null table

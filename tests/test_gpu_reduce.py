@@ -141,6 +141,51 @@ def test_special_values(cuda):
     assert np.all(out[:8] == 0x0000)
 
 
+@pytest.mark.parametrize("numel", [8, 4096, 1 << 20])
+def test_stepwise_bf16_matches_reference_chain(cuda, numel):
+    """accumulate="bf16": the accumulator is rounded to bf16 after every add, as the
+    reference's add.bf16x2 chain does (triton_one_shot_all_reduce.py:36-49, 84-89).
+    Bar: bit-exact against the oracle's restatement of that chain."""
+    from symm_mem_recipes import one_shot_all_reduce
+    t, h = _alloc(numel, torch.bfloat16, cuda)
+    bufs = _fill(h, numel, torch.bfloat16, seed0=40)
+    out = _bits(one_shot_all_reduce(t, accumulate="bf16"))
+    h.check_status()
+    want = O.reduce_ref_bf16_acc(bufs)
+    assert np.array_equal(out, want)
+    if numel >= 4096:
+        # the two accumulation modes are different functions of the same inputs
+        assert not np.array_equal(want, O.reduce_ref(bufs, "bf16"))
+    # write-back to all peers and all ranks in one launch share the arithmetic
+    allr = _bits(one_shot_all_reduce(t, accumulate="bf16", all_ranks=True))
+    h.check_status()
+    assert all(np.array_equal(allr[r], want) for r in range(WS))
+
+
+def test_stepwise_bf16_special_values(cuda):
+    """Signed zeros, subnormals, overflow to infinity, NaN (canonical 0x7FFF), ties and
+    sums whose fp32 value lies next to a bf16 rounding boundary."""
+    from symm_mem_recipes import one_shot_all_reduce
+    numel = 4096
+    t, h = _alloc(numel, torch.bfloat16, cuda)
+    rng = np.random.default_rng(11)
+    specials = np.array([0x0000, 0x8000, 0x0001, 0x8001, 0x007F, 0x0080, 0x807F, 0x7F7F, 0xFF7F, 0x7F80,
+                         0xFF80, 0x7FC0, 0xFFC1, 0x3F80, 0xBF80, 0x3B80, 0x4000, 0x3F81, 0x3780, 0x4B80,
+                         0x3F7F, 0xBF7F, 0x0100, 0x8100], dtype=np.uint16)
+    bufs = [rng.choice(specials, size=numel).astype(np.uint16) for _ in range(WS)]
+    # random bit patterns too: every exponent distance between the operands occurs
+    for r in range(WS):
+        bufs[r][numel // 2:] = rng.integers(0, 1 << 16, numel // 2).astype(np.uint16)
+        bufs[r][:8] = 0x8000                  # -0 + ... + -0 with a +0 start is +0
+        h.get_buffer(r, (numel,), torch.int16).copy_(torch.from_numpy(bufs[r].view(np.int16)))
+    out = _bits(one_shot_all_reduce(t, accumulate="bf16"))
+    h.check_status()
+    want = O.reduce_ref_bf16_acc(bufs)
+    assert np.array_equal(out, want)
+    assert np.all(out[:8] == 0x0000)
+    assert np.any(want == 0x7FFF)
+
+
 def test_validation_asserts(cuda):
     """Contract violations are AssertionErrors, as in the reference
     (triton_one_shot_all_reduce.py:102-105)."""
@@ -200,6 +245,7 @@ def test_golden_vectors(cuda):
     for r in range(WS):
         h.get_buffer(r, (256,), torch.int16).copy_(torch.from_numpy(g["bf16_in"][r].view(np.int16)))
     assert np.array_equal(_bits(one_shot_all_reduce(t)), g["bf16_out"])
+    assert np.array_equal(_bits(one_shot_all_reduce(t, accumulate="bf16")), g["bf16_out_bf16_acc"])
     t, h = _alloc(256, torch.float32, cuda)
     for r in range(WS):
         h.get_buffer(r, (256,), torch.float32).copy_(torch.from_numpy(g["fp32_in"][r]))

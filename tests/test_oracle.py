@@ -170,6 +170,45 @@ def test_reduce_bf16_acc_chain_bruteforce():
     assert np.array_equal(got, _t_bits(t))
 
 
+def test_bf16_acc_chain_random_bit_patterns_and_nan():
+    """Every exponent distance, subnormals and overflow against exact rational
+    arithmetic; a NaN anywhere in the chain gives the canonical 0x7FFF."""
+    rng = np.random.default_rng(5)
+    bufs = [rng.integers(0, 1 << 16, 512).astype(np.uint16) for _ in range(4)]
+    got = O.reduce_ref_bf16_acc(bufs)
+    big = Fraction(2) ** 128 - Fraction(2) ** 119          # first value that rounds to infinity
+    for j in range(512):
+        vals = [int(b[j]) for b in bufs]
+        fl = [float(O.bf16_bits_to_f32(np.array([v], np.uint16))[0]) for v in vals]
+        if any(np.isnan(f) for f in fl):
+            assert got[j] == 0x7FFF
+            continue
+        acc = 0.0
+        bad = False
+        fr = Fraction(0)
+        for f in fl:
+            if np.isinf(f) or np.isinf(acc):
+                bad = True
+                break
+            fr = fr + Fraction(f)
+            if abs(fr) >= big:
+                bad = True
+                break
+            fr = _rbf16(fr)
+            acc = float(fr)
+        if bad:
+            continue                                       # infinities: covered by the torch cross-check below
+        assert _frac_of_bf16(int(got[j])) == fr, j
+    t = torch.zeros(512, dtype=torch.bfloat16)
+    for b in bufs:
+        t = t + _bits_t(b)
+    tb = _t_bits(t)
+    nan = np.isnan(O.bf16_bits_to_f32(tb))
+    assert np.array_equal(np.isnan(O.bf16_bits_to_f32(got)), nan)
+    assert np.array_equal(got[~nan], tb[~nan])
+    assert np.all(got[nan] == 0x7FFF)
+
+
 def test_bf16_acc_double_rounding_case():
     """A sum whose fp32 rounding lands on a bf16 tie: single rounding must win."""
     a = np.array([0x3F80], dtype=np.uint16)            # 1.0
