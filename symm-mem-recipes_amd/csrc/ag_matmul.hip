@@ -49,6 +49,7 @@ struct GemmSchedule {
   // local comm block in halves every workgroup starts on rows that need no flag,
   // and the producer gets that half pass as a head start.
   int head, tail;
+  int steps;                     // trips of the busiest workgroup (passes over all phases)
 };
 
 struct TileRef {
@@ -61,7 +62,7 @@ struct TileRef {
 
 __host__ __device__ inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
 
-// Tile visited by workgroup `wg` in its `step`-th trip; false when it has no more work.
+// Tile visited by workgroup `wg` in trip `step` of the grid; false when it has none in that trip.
 // Three phases: `head` ring positions in half tiles, the middle in full tiles, `tail`
 // in half tiles.  A phase is walked in passes of `grid` tiles; within a pass XCD x
 // (workgroups with id % 8 == x) takes a contiguous run of the tile order.  The tile
@@ -104,6 +105,15 @@ __host__ __device__ inline bool tile_for(const GemmSchedule& s, int wg, int step
     step -= passes;
     ring0 += positions;
   }
+  return false;
+}
+
+// First tile of workgroup `wg` at or after trip `step` (a workgroup can sit out the
+// ragged last pass of a phase and still have work in the next phase); advances `step`
+// to that trip.  False when the workgroup is done.
+__host__ __device__ inline bool next_tile(const GemmSchedule& s, int wg, int& step, TileRef& t) {
+  for (; step < s.steps; ++step)
+    if (tile_for(s, wg, step, t)) return true;
   return false;
 }
 
@@ -499,7 +509,8 @@ __global__ __launch_bounds__(kGemmThreads, 1) void ag_matmul_kernel(
   };
 
   TileRef tile;
-  bool have = tile_for(s, blockIdx.x, 0, tile);
+  int step = 0;
+  bool have = next_tile(s, blockIdx.x, step, tile);
   const uint8_t* a_base = nullptr;
   const uint8_t* b_base = nullptr;
   if (have) {
@@ -507,10 +518,10 @@ __global__ __launch_bounds__(kGemmThreads, 1) void ag_matmul_kernel(
     b_base = b_nk + (int64_t)tile.col0 * cx.row_stride;
   }
   bool preloaded = false;
-  for (int step = 0; have; ++step) {
+  for (int trip = 0; have; ++trip) {
     cx.tr = nullptr;
-    if (trace != nullptr && step < kTraceSteps && blockIdx.x < 256 && threadIdx.x == 0) {
-      cx.tr = trace + kTraceProducerWords + ((size_t)blockIdx.x * kTraceSteps + step) * 4;
+    if (trace != nullptr && trip < kTraceSteps && blockIdx.x < 256 && threadIdx.x == 0) {
+      cx.tr = trace + kTraceProducerWords + ((size_t)blockIdx.x * kTraceSteps + trip) * 4;
       cx.tr[0] = cx.tr[1] = wall_clock64();
     }
     TileRef next;
@@ -520,7 +531,8 @@ __global__ __launch_bounds__(kGemmThreads, 1) void ag_matmul_kernel(
     // Between this tile's K loop and its stores: pick the next tile, wait for its
     // flag if it has one, and start its first loads.
     auto between = [&]() {
-      have_next = tile_for(s, blockIdx.x, step + 1, next);
+      ++step;
+      have_next = next_tile(s, blockIdx.x, step, next);
       if (!have_next) return;
       a_next = a_rows_of(next);
       b_next = b_nk + (int64_t)next.col0 * cx.row_stride;
@@ -599,6 +611,14 @@ static int cu_count() {
 // find no room while the consumers spin on its flags.
 constexpr int kReservedCus = 8;
 
+static int total_steps(const GemmSchedule& s) {
+  const int cb_tiles_m = s.comm_block_m / s.BM;
+  const int n_comm = s.M / s.comm_block_m;
+  const int full = cb_tiles_m * ceil_div(s.N, s.BN), half = cb_tiles_m * ceil_div(s.N, s.BN / 2);
+  return ceil_div(s.head * half, s.grid) + ceil_div((n_comm - s.head - s.tail) * full, s.grid) +
+         ceil_div(s.tail * half, s.grid);
+}
+
 // smr_set_ag_matmul_halves: ring positions cut into half tiles at either end of a
 // gated launch, or -1 to let make_schedule choose.
 static int g_force_head = -1, g_force_tail = -1;
@@ -632,15 +652,8 @@ static GemmSchedule make_schedule(int M, int N, int K, int rank, int world_size,
       s.tail = g_force_tail;
     }
   }
+  s.steps = total_steps(s);
   return s;
-}
-
-static int total_steps(const GemmSchedule& s) {
-  const int cb_tiles_m = s.comm_block_m / s.BM;
-  const int n_comm = s.M / s.comm_block_m;
-  const int full = cb_tiles_m * ceil_div(s.N, s.BN), half = cb_tiles_m * ceil_div(s.N, s.BN / 2);
-  return ceil_div(s.head * half, s.grid) + ceil_div((n_comm - s.head - s.tail) * full, s.grid) +
-         ceil_div(s.tail * half, s.grid);
 }
 
 }  // namespace smr
@@ -700,11 +713,10 @@ int smr_ag_matmul_schedule(int M, int N, int K, int rank, int world_size, int co
   // host-only: the schedule of a 256-CU part, the one the kernels are tuned for
   const GemmSchedule s = make_schedule(M, N, K, rank, world_size, comm_block_m, 256, gated != 0);
   int count = 0;
-  const int steps = total_steps(s);
   for (int wg = 0; wg < s.grid; ++wg) {
-    for (int step = 0; step < steps; ++step) {
-      TileRef t;
-      if (!tile_for(s, wg, step, t)) continue;
+    TileRef t;
+    // the same walk as the kernel's
+    for (int step = 0; next_tile(s, wg, step, t); ++step) {
       if (out_records != nullptr && count < max_tiles) {
         int32_t* rec = out_records + (size_t)count * 8;
         rec[0] = wg;

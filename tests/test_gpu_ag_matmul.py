@@ -92,6 +92,40 @@ def test_fused_parity_small(cuda, M, N, K, ws, rank):
     assert torch.allclose(c0.float(), c_out.float(), rtol=2e-2, atol=1e-3)
 
 
+@pytest.mark.parametrize("M,N,K,ws,rank,splits", [
+    (2048, 256, 256, 8, 3, 2),       # comm blocks of 128 rows: 128x128 tiles
+    (4096, 512, 128, 8, 6, 2),       # comm blocks of 256 rows: 256x256 tiles, 16 flags
+    (4096, 384, 192, 4, 1, 4),       # world size 4, four flags per rank
+])
+def test_fused_parity_splits_per_rank(cuda, M, N, K, ws, rank, splits):
+    """Finer flags (triton_all_gather_matmul.py:24,41-49): every rank's shard arrives in
+    `splits` chunks with a flag each, and a tile waits for the chunk its rows are in."""
+    from symm_mem_recipes import all_gather_matmul_tma_persistent
+    a_shard, h, shards, b, b_bits, a_out, c_out = _setup(M, N, K, ws, rank, cuda)
+    a_out.zero_()
+    all_gather_matmul_tma_persistent(a_shard, b, a_out, c_out, None, splits_per_rank=splits)
+    h.check_status()
+    _check(_t_bits(c_out), O.ag_matmul_ref(shards, b_bits))
+    assert np.array_equal(_t_bits(a_out), np.concatenate(shards))
+
+
+@pytest.mark.parametrize("head,tail", [(0, 0), (1, 0), (1, 1), (2, 0), (0, 2), (3, 3)])
+def test_fused_parity_half_tile_phases(cuda, lib, head, tail):
+    """Every split of the gated schedule into half-width and full-width phases computes
+    the same product (the library picks one by cost; this forces the others)."""
+    from symm_mem_recipes import all_gather_matmul_tma_persistent
+    M, N, K, ws, rank = 4096, 640, 192, 8, 5
+    a_shard, h, shards, b, b_bits, a_out, c_out = _setup(M, N, K, ws, rank, cuda)
+    try:
+        assert lib.smr_set_ag_matmul_halves(head, tail) == 0
+        c_out.zero_()
+        all_gather_matmul_tma_persistent(a_shard, b, a_out, c_out, None)
+        h.check_status()
+    finally:
+        lib.smr_set_ag_matmul_halves(-1, -1)
+    _check(_t_bits(c_out), O.ag_matmul_ref(shards, b_bits))
+
+
 def test_mm_only_is_ungated(cuda, monkeypatch):
     """mm_only multiplies what the buffers already hold, as rank 0, with no flags
     (triton_all_gather_matmul.py:222-224,246-247)."""
