@@ -113,15 +113,15 @@ def bench_reduce(size_mib, steps, warmup, dev):
                 us_write_all=us_write_all, write_all_bytes=2 * WS * nbytes)
 
 
-def bench_reduce_rotating(size_mib, dev, dtype_name="bf16"):
-    """Smaller messages fit the 256 MB last-level cache; rotate over enough buffer
-    sets (> 1 GiB in total) that every call reads from HBM."""
+def bench_reduce_rotating(size_kib, dev, dtype_name="bf16", write_all=False, accumulate="fp32"):
+    """Messages below 64 MiB fit the 256 MB last-level cache; rotate over enough buffer
+    sets (1 GiB in total, at most 64 sets) that every call reads from HBM."""
     import torch
     from symm_mem_recipes import EmulatedSymmetricMemory as SM, one_shot_all_reduce
     dtype = torch.bfloat16 if dtype_name == "bf16" else torch.float32
-    nbytes = size_mib << 20
+    nbytes = size_kib << 10
     numel = nbytes // (2 if dtype == torch.bfloat16 else 4)
-    nsets = max(2, -(-(1 << 30) // (WS * nbytes)))
+    nsets = min(64, max(2, -(-(1 << 30) // (WS * nbytes))))
     sets = []
     for _ in range(nsets):
         t = SM.empty_strided_p2p((numel,), (1,), dtype, dev, world_size=WS, rank=0)
@@ -132,12 +132,38 @@ def bench_reduce_rotating(size_mib, dev, dtype_name="bf16"):
     idx = [0]
 
     def call():
-        one_shot_all_reduce(sets[idx[0] % nsets], barrier=False)
+        one_shot_all_reduce(sets[idx[0] % nsets], barrier=False, write_all=write_all, accumulate=accumulate)
         idx[0] += 1
-    us = _time_batched(call, 10 * nsets, nsets)
+    us = _time_batched(call, max(10 * nsets, 200), nsets)
+    alg = (2 * WS if write_all else WS + 1) * nbytes
+    res = dict(size_kib=size_kib, dtype=dtype_name, mode="write_all" if write_all else "single_output",
+               accumulate=accumulate, us=us, gbs=alg / us / 1e3, frac=alg / us / 1e3 / HBM_PEAK_GBS,
+               buffer_sets=nsets)
+    if nbytes <= (4 << 20) and not write_all:
+        # Below a few MiB the eager figure is the host's launch rate, not the kernel:
+        # replay one pass over the buffer sets from a HIP graph (kernel nodes only) and
+        # check every replay against the eager result.
+        ref = one_shot_all_reduce(sets[0], barrier=False, accumulate=accumulate).clone()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            outs = [one_shot_all_reduce(t, barrier=False, accumulate=accumulate) for t in sets]
+        reps = max(4, 400 // nsets)
+        for _ in range(2):
+            graph.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(outs[0], ref), "graph replay differs from the eager result"
+        a = torch.cuda.Event(enable_timing=True)
+        b = torch.cuda.Event(enable_timing=True)
+        a.record()
+        for _ in range(reps):
+            graph.replay()
+        b.record()
+        torch.cuda.synchronize()
+        assert torch.equal(outs[0], ref), "graph replay differs from the eager result"
+        res["us_graph_replay"] = a.elapsed_time(b) * 1e3 / (reps * nsets)
+        del graph, outs
     SM.release()
-    return dict(size_mib=size_mib, dtype=dtype_name, us=us, gbs=(WS + 1) * nbytes / us / 1e3,
-                frac=(WS + 1) * nbytes / us / 1e3 / HBM_PEAK_GBS, buffer_sets=nsets)
+    return res
 
 
 def bench_ag_matmul(dev):
@@ -268,9 +294,26 @@ def cpu_baseline(budget_s=10.0):
         if el >= budget_s:
             break
     nbytes = (WS + 1) * n * 2
-    return {"value": nbytes * reps / el / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
-            "sample": f"{reps} repetitions of the 8 x 1,048,576 bf16 reduce (numpy oracle, one thread) in {el:.1f} s",
-            "host_cpus": os.cpu_count()}
+    out = {"value": nbytes * reps / el / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
+           "sample": f"{reps} repetitions of the 8 x 1,048,576 bf16 reduce (numpy oracle, one thread) in {el:.1f} s",
+           "host_cpus": os.cpu_count()}
+    # the other two paths, once each on a bounded slice (numpy's BLAS uses the host's threads)
+    M, N, K = 256, 3584, 8192
+    shard = O.seeded_normal_bf16_bits(M * K, seed=0, std=0.02).reshape(M, K)
+    b_nk = O.seeded_normal_bf16_bits(N * K, seed=100, std=0.02).reshape(N, K)
+    t0 = time.perf_counter()
+    O.ag_matmul_ref([shard], b_nk)
+    el = time.perf_counter() - t0
+    out["ag_matmul"] = {"value": 2.0 * M * N * K / el / 1e12, "unit": "TFLOP/s",
+                        "sample": f"{M} of the 16384 rows of the M=16384 N=3584 K=8192 product, once, {el:.2f} s"}
+    x = O.seeded_normal_bf16_bits(8 * 8192, seed=0).reshape(8, 8192)
+    w = O.seeded_normal_bf16_bits(8192 * 8192, seed=1, std=0.02).reshape(8192, 8192)
+    t0 = time.perf_counter()
+    O.gemv_allreduce_ref(x, w, WS)
+    el = time.perf_counter() - t0
+    out["gemv_allreduce"] = {"value": (8192 * 8192 * 2 + 2 * 8 * 8192 * 2) / el / 1e9, "unit": "GB/s",
+                             "sample": f"batch 8, K = N = 8192, 8 K-shards, once, {el:.2f} s"}
+    return out
 
 
 def main():
@@ -325,8 +368,13 @@ def main():
     }
     extra["calibration_copy"] = calibration_copy(dev)
     if not args.no_extra:
-        extra["reduce_rotating"] = [bench_reduce_rotating(s, dev, d)
-                                    for d in ("bf16", "fp32") for s in (8, 16)]
+        # per-buffer sizes of the size sweep; 2 and 8 MiB are the points the targets name
+        sweep = (16, 64, 256, 1024, 2048, 4096, 8192, 16384, 32768)
+        extra["reduce_rotating"] = (
+            [bench_reduce_rotating(k, dev, "bf16") for k in sweep] +
+            [bench_reduce_rotating(k, dev, "fp32") for k in (1024, 8192, 16384)] +
+            [bench_reduce_rotating(k, dev, "bf16", write_all=True) for k in (1024, 8192, 16384)] +
+            [bench_reduce_rotating(k, dev, "bf16", accumulate="bf16") for k in (8192,)])
         extra["all_gather_matmul"] = bench_ag_matmul(dev)
         extra["gemv_allreduce"] = bench_gemv(dev)
         extra["barrier"] = bench_barrier(dev)
