@@ -106,11 +106,16 @@ def bench_reduce(size_mib, steps, warmup, dev):
     # the same call behind the blockwise barrier, and the write-back-to-all variant
     us_barrier = _time_events(lambda: one_shot_all_reduce(t, barrier=True), 20, 3)
     us_write_all = _time_events(lambda: one_shot_all_reduce(t, barrier=False, write_all=True), 20, 3)
+    # two-shot: every emulated rank reduces its eighth and writes it to all peers, two handshakes
+    for r in range(WS):
+        g.manual_seed(r)
+        h.get_buffer(r, (numel,), torch.bfloat16).normal_(generator=g)
+    us_two_shot = _time_events(lambda: one_shot_all_reduce(t, all_ranks=True, write_all=True), 12, 3)
     h.check_status()
     SM.release()
     del out
     return dict(wall_s=wall, dev_us=dev_us, alg_bytes=alg_bytes, us_barrier=us_barrier,
-                us_write_all=us_write_all, write_all_bytes=2 * WS * nbytes)
+                us_write_all=us_write_all, write_all_bytes=2 * WS * nbytes, us_two_shot=us_two_shot)
 
 
 def bench_reduce_rotating(size_kib, dev, dtype_name="bf16", write_all=False, accumulate="fp32"):
@@ -365,6 +370,8 @@ def main():
         "reduce_behind_barrier_us": r["us_barrier"],
         "reduce_write_all_us": r["us_write_all"],
         "reduce_write_all_gbs": r["write_all_bytes"] / r["us_write_all"] / 1e3,
+        "reduce_two_shot_us": r["us_two_shot"],
+        "reduce_two_shot_gbs": r["write_all_bytes"] / r["us_two_shot"] / 1e3,
     }
     extra["calibration_copy"] = calibration_copy(dev)
     if not args.no_extra:

@@ -56,6 +56,9 @@ extern "C" {
 #define SMR_BARRIER_NONE   0  /* no handshake: peers' data are already stream-ordered */
 #define SMR_BARRIER_PROXY  1  /* the rank's blocks run the real handshake; one proxy
                                  workgroup per block plays the other ranks' halves */
+#define SMR_BARRIER_BOTH   2  /* as PROXY, and a second handshake after the last store: the
+                                 reference has none behind triton_one_shot_all_reduce.py:93, so
+                                 a peer may overwrite its buffer while others still read it */
 
 int smr_version(void);
 const char* smr_last_error_string(void);
@@ -82,8 +85,13 @@ int64_t smr_get_spin_timeout_us(void);
  *   rank       0..ws-1: that rank's share.  -1: all emulated ranks in one launch
  *              (out is then [ws, numel], and the ranks run the real barrier
  *              against each other when barrier_mode != NONE)
+ *   dtype      SMR_DTYPE_BF16 / _FP32: fp32 accumulator as above; _BF16_STEPWISE: the
+ *              accumulator is rounded to bf16 after every add, as :36-49 does
  *   write_all  0: result goes to `out`.  1: result is written back into all ws
- *              peer buffers in place (`out` may be NULL); rank must be >= 0
+ *              peer buffers in place (`out` may be NULL).  With rank = -1 this is the
+ *              two-shot form: rank r reduces slots [numel/16*r/ws, numel/16*(r+1)/ws)
+ *              only and writes them to every peer, between two handshakes
+ *              (barrier_mode must be SMR_BARRIER_BOTH); no reference counterpart
  *   signal_pad_ptrs_dev may be NULL when barrier_mode == SMR_BARRIER_NONE;
  *              each pad must hold smr_reduce_num_blocks(...) * ws uint32 slots. */
 int smr_one_shot_all_reduce(const uint64_t* buffer_ptrs_dev, const uint64_t* signal_pad_ptrs_dev,

@@ -128,6 +128,7 @@ __global__ __launch_bounds__(kReduceMaxThreads) void one_shot_all_reduce_kernel(
     uint64_t limit_ticks, uint32_t* status) {
   int block = blockIdx.x;
   const int nthreads = blockDim.x;
+  int64_t lo = 0, hi = nvec;             // slots this rank reduces
   if (layout == kProxy) {
     const int per_proxy = nthreads >> 3;
     const int nproxy = (nblocks + per_proxy - 1) / per_proxy;
@@ -138,10 +139,16 @@ __global__ __launch_bounds__(kReduceMaxThreads) void one_shot_all_reduce_kernel(
       if (b < nblocks && j < WS && j != rank) {
         uint32_t* to_rank = reinterpret_cast<uint32_t*>(signal_pad_ptrs[rank]) + (size_t)b * WS + j;
         uint32_t* from_rank = reinterpret_cast<uint32_t*>(signal_pad_ptrs[j]) + (size_t)b * WS + rank;
-        if (!send_signal(to_rank, limit_ticks)) {
-          report(status, SMR_ST_SEND_TIMEOUT, j, b, rank);
-        } else if (!wait_signal_reset(from_rank, limit_ticks)) {
-          report(status, SMR_ST_WAIT_TIMEOUT, j, b, rank);
+        // one round per handshake of the rank's block (leading, and trailing if asked for)
+        for (int round = 0; round < do_barrier; ++round) {
+          if (!send_signal(to_rank, limit_ticks)) {
+            report(status, SMR_ST_SEND_TIMEOUT, j, b, rank);
+            break;
+          }
+          if (!wait_signal_reset(from_rank, limit_ticks)) {
+            report(status, SMR_ST_WAIT_TIMEOUT, j, b, rank);
+            break;
+          }
         }
       }
       return;
@@ -150,7 +157,13 @@ __global__ __launch_bounds__(kReduceMaxThreads) void one_shot_all_reduce_kernel(
   } else if (layout == kAllRanks) {
     block = blockIdx.x / WS;
     rank = blockIdx.x % WS;
-    out += (size_t)rank * nvec;
+    if constexpr (WRITE_ALL) {
+      // two-shot: the rank reduces its own slice only and hands it to every peer
+      lo = nvec * rank / WS;
+      hi = nvec * (rank + 1) / WS;
+    } else {
+      out += (size_t)rank * nvec;
+    }
   }
 
   // the peers' buffers were written by earlier kernels: nothing of this kernel to publish
@@ -162,7 +175,7 @@ __global__ __launch_bounds__(kReduceMaxThreads) void one_shot_all_reduce_kernel(
   GlobalVec* dst = (GlobalVec*)(uintptr_t)out;
 
   const int64_t stride = (int64_t)nblocks * nthreads;
-  for (int64_t i = (int64_t)block * nthreads + threadIdx.x; i < nvec; i += stride) {
+  for (int64_t i = lo + (int64_t)block * nthreads + threadIdx.x; i < hi; i += stride) {
     Vec16 v[WS];
 #pragma unroll
     for (int r = 0; r < WS; ++r) v[r] = load_stream(src[r] + i);
@@ -174,6 +187,9 @@ __global__ __launch_bounds__(kReduceMaxThreads) void one_shot_all_reduce_kernel(
       store_stream(dst + i, o);
     }
   }
+  // Trailing handshake: nobody's buffer is overwritten (or, with write-back, read)
+  // before every rank is through; it publishes this workgroup's stores.
+  if (do_barrier == 2) blockwise_barrier(signal_pad_ptrs, block, rank, WS, limit_ticks, status, true, true);
 }
 
 template <int KIND, int WS>
@@ -247,12 +263,12 @@ int smr_one_shot_all_reduce(const uint64_t* buffer_ptrs_dev, const uint64_t* sig
     return fail(SMR_E_INVALID, "smr_one_shot_all_reduce: The number of elements must be 128-bit aligned.");
   if (buffer_ptrs_dev == nullptr)
     return fail(SMR_E_INVALID, "smr_one_shot_all_reduce: buffer_ptrs_dev is NULL");
-  if (barrier_mode != SMR_BARRIER_NONE && barrier_mode != SMR_BARRIER_PROXY)
+  if (barrier_mode != SMR_BARRIER_NONE && barrier_mode != SMR_BARRIER_PROXY && barrier_mode != SMR_BARRIER_BOTH)
     return fail(SMR_E_INVALID, "smr_one_shot_all_reduce: unknown barrier_mode");
   if (barrier_mode != SMR_BARRIER_NONE && signal_pad_ptrs_dev == nullptr)
     return fail(SMR_E_INVALID, "smr_one_shot_all_reduce: signal pads required for the barrier");
-  if (write_all && rank < 0)
-    return fail(SMR_E_INVALID, "smr_one_shot_all_reduce: write_all needs a single rank");
+  if (write_all && rank < 0 && barrier_mode != SMR_BARRIER_BOTH)
+    return fail(SMR_E_INVALID, "smr_one_shot_all_reduce: the two-shot form (all ranks, write-back) needs SMR_BARRIER_BOTH");
   if (!write_all && out == nullptr)
     return fail(SMR_E_INVALID, "smr_one_shot_all_reduce: out is NULL");
   if (out != nullptr && (reinterpret_cast<uintptr_t>(out) & 15u))
@@ -262,7 +278,7 @@ int smr_one_shot_all_reduce(const uint64_t* buffer_ptrs_dev, const uint64_t* sig
   const int64_t nvec = numel / per_vec;
   const int nblocks = smr_reduce_num_blocks(numel, dtype);
   const int threads = reduce_threads_for(nvec);
-  const int do_barrier = barrier_mode != SMR_BARRIER_NONE;
+  const int do_barrier = barrier_mode == SMR_BARRIER_BOTH ? 2 : (barrier_mode != SMR_BARRIER_NONE ? 1 : 0);
   int layout = kPlain;
   unsigned grid = (unsigned)nblocks;
   if (rank < 0) {

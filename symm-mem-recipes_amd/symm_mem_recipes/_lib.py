@@ -17,6 +17,7 @@ DTYPE_FP32 = 1
 DTYPE_BF16_STEPWISE = 2
 BARRIER_NONE = 0
 BARRIER_PROXY = 1
+BARRIER_BOTH = 2
 STATUS_WORDS = 4
 MAX_WORLD_SIZE = 8
 

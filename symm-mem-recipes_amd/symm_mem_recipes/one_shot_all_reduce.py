@@ -23,7 +23,8 @@ def num_blocks(numel: int, dtype: torch.dtype = torch.bfloat16) -> int:
 
 
 def one_shot_all_reduce(tensor: torch.Tensor, *, barrier: bool = True, write_all: bool = False,
-                        all_ranks: bool = False, accumulate: str = "fp32") -> torch.Tensor:
+                        all_ranks: bool = False, accumulate: str = "fp32",
+                        trailing_barrier: bool = False) -> torch.Tensor:
     """Sum the symmetric buffers of all ranks element-wise (fp32 accumulator,
     rank order 0..world_size-1) and return the calling rank's result.
 
@@ -34,6 +35,13 @@ def one_shot_all_reduce(tensor: torch.Tensor, *, barrier: bool = True, write_all
                    return the calling rank's buffer (``tensor`` itself).
     ``all_ranks``  run every emulated rank in one launch, each behind the real
                    barrier; returns ``[world_size, *tensor.shape]``.
+                   Together with ``write_all`` it is the two-shot all-reduce:
+                   rank r reduces the r-th slice only and writes it into every
+                   peer's buffer, between two handshakes; returns the
+                   ``[world_size, *tensor.shape]`` view of the buffers.
+    ``trailing_barrier`` a second handshake after the last store (the reference
+                   has none behind triton_one_shot_all_reduce.py:93): no peer
+                   can overwrite its buffer while another still reads it.
     ``accumulate`` "fp32" (default) keeps an fp32 accumulator and rounds once;
                    "bf16" rounds the accumulator to bf16 after every add, which is
                    bit for bit the reference's add.bf16x2 chain
@@ -48,11 +56,14 @@ def one_shot_all_reduce(tensor: torch.Tensor, *, barrier: bool = True, write_all
     assert tensor.is_contiguous(), "tensor must be contiguous"
     symm_mem = EmulatedSymmetricMemory.rendezvous(tensor)
     assert symm_mem is not None, "tensor must be allocated via SymmetricMemory"
-    assert not (write_all and all_ranks)
 
     lib = _lib.load()
     stream = torch.cuda.current_stream(tensor.device).cuda_stream
-    if write_all:
+    two_shot = write_all and all_ranks
+    if two_shot:
+        assert barrier, "the two-shot form needs its handshakes"
+        output, out_ptr = None, 0
+    elif write_all:
         output, out_ptr = tensor, 0
     elif all_ranks:
         output = torch.empty((symm_mem.world_size,) + tuple(tensor.shape), dtype=tensor.dtype,
@@ -70,9 +81,12 @@ def one_shot_all_reduce(tensor: torch.Tensor, *, barrier: bool = True, write_all
         -1 if all_ranks else symm_mem.rank,
         symm_mem.world_size,
         1 if write_all else 0,
-        _lib.BARRIER_PROXY if barrier else _lib.BARRIER_NONE,
+        (_lib.BARRIER_BOTH if (trailing_barrier or two_shot) else _lib.BARRIER_PROXY) if barrier
+        else _lib.BARRIER_NONE,
         symm_mem.status.data_ptr(),
         stream,
     )
     _lib.check(rc, "one_shot_all_reduce")
+    if two_shot:
+        return symm_mem.all_buffers(tuple(tensor.shape), tensor.dtype)
     return output

@@ -166,6 +166,18 @@ class EmulatedSymmetricMemory:
             acc *= max(n, 1)
         return self._view(int(rank), sizes, tuple(reversed(strides)), dtype, int(storage_offset))
 
+    def all_buffers(self, sizes: Sequence[int], dtype: torch.dtype) -> torch.Tensor:
+        """``[world_size, *sizes]`` view over every rank's buffer (no copy; an
+        emulation-only convenience: on real peers these are eight allocations)."""
+        sizes = tuple(int(s) for s in sizes)
+        first = self.get_buffer(0, sizes, dtype)
+        itemsize = first.element_size()
+        g = self._group
+        assert g.buffer_size % itemsize == 0
+        return g.slab.view(dtype).as_strided((self.world_size,) + sizes,
+                                            (g.buffer_size // itemsize,) + tuple(first.stride()),
+                                            g.slab.view(dtype).storage_offset())
+
     def get_signal_pad(self, rank: int, sizes: Optional[Sequence[int]] = None,
                        dtype: torch.dtype = torch.int32) -> torch.Tensor:
         g = self._group

@@ -186,6 +186,52 @@ def test_stepwise_bf16_special_values(cuda):
     assert np.any(want == 0x7FFF)
 
 
+@pytest.mark.parametrize("dtype,numel", [(torch.bfloat16, 8), (torch.bfloat16, 40), (torch.bfloat16, 1 << 20),
+                                         (torch.float32, 3 * 4096 + 4)])
+def test_two_shot_all_reduce(cuda, dtype, numel):
+    """all_ranks + write_all: rank r reduces slice r and writes it into every peer's
+    buffer, between two real handshakes.  Every buffer must end up holding the
+    rank-ordered sum of the original buffers, bit for bit (slices that are empty or
+    ragged included: 8 bf16 = one 16-byte slot for 8 ranks)."""
+    from symm_mem_recipes import one_shot_all_reduce
+    t, h = _alloc(numel, dtype, cuda)
+    bufs = _fill(h, numel, dtype, seed0=70)
+    out = one_shot_all_reduce(t, all_ranks=True, write_all=True)
+    h.check_status()
+    want = O.reduce_ref(bufs, "bf16" if dtype == torch.bfloat16 else "fp32")
+    assert out.shape[0] == WS
+    for r in range(WS):
+        assert _same(_bits(out[r]), want), r
+        assert _same(_bits(h.get_buffer(r, (numel,), dtype)), want), r
+    # pads are back to zero: the next collective can start
+    for r in range(WS):
+        assert int(h.get_signal_pad(r).abs().sum()) == 0
+
+
+@pytest.mark.parametrize("write_all", [False, True])
+def test_trailing_barrier(cuda, write_all):
+    """A second handshake behind the last store (the reference has none): same
+    result, pads self-reset after both rounds, and it can be called back to back."""
+    from symm_mem_recipes import one_shot_all_reduce
+    numel = 1 << 18
+    t, h = _alloc(numel, torch.bfloat16, cuda)
+    bufs = _fill(h, numel, torch.bfloat16, seed0=80)
+    want = O.reduce_ref(bufs, "bf16")
+    out = one_shot_all_reduce(t, write_all=write_all, trailing_barrier=True)
+    h.check_status()
+    assert _same(_bits(out), want)
+    if write_all:
+        for r in range(WS):
+            assert _same(_bits(h.get_buffer(r, (numel,), torch.bfloat16)), want)
+    else:
+        for _ in range(3):
+            out = one_shot_all_reduce(t, trailing_barrier=True)
+        h.check_status()
+        assert _same(_bits(out), want)
+    for r in range(WS):
+        assert int(h.get_signal_pad(r).abs().sum()) == 0
+
+
 def test_validation_asserts(cuda):
     """Contract violations are AssertionErrors, as in the reference
     (triton_one_shot_all_reduce.py:102-105)."""
