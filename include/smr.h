@@ -193,6 +193,14 @@ int smr_ag_matmul(const void* a_shard_dev, const void* a_out_dev, const void* b_
 int smr_ag_matmul_schedule(int M, int N, int K, int rank, int world_size, int comm_block_m,
                            int gated, int32_t* out_records, int max_tiles);
 
+/* Host-only: how a fused launch of this shape splits the GPU.  out4 = {GEMM grid (what
+ * smr_ag_matmul will launch when gated), producer workgroups, fast_chunks,
+ * slow_workgroups} - the last two are the arguments of smr_set_gather_pacing, {0, 0} when
+ * the copy should run flat out because the GEMM would otherwise wait for it.  Replaces
+ * the fixed NUM_SMS grid of triton_all_gather_matmul.py:287-294: there the copy engines
+ * cost no SMs. */
+int smr_ag_matmul_plan(int M, int N, int K, int world_size, int comm_block_m, int32_t* out4);
+
 /* Tuning knob of the gated schedule: the first `head` and the last `tail` comm blocks
  * of the ring order are computed in tiles of half the width.  Both -1 (the default)
  * lets the library choose.  No reference counterpart. */

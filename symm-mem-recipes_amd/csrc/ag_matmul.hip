@@ -619,6 +619,32 @@ static int total_steps(const GemmSchedule& s) {
          ceil_div(s.tail * half, s.grid);
 }
 
+// Coarse model of a fused launch, for splitting the compute units between the GEMM
+// and the producer.  Rates measured on MI355X with both kernels running: a GEMM
+// workgroup sustains about 6 TFLOP/s, a producer workgroup moves about 33 GB/s
+// (bytes read plus bytes written).
+struct FusedEstimate {
+  double gemm_us, copy_us, total_us;
+  int producer_wgs;
+};
+constexpr int kMaxProducerWgs = 128;
+// every chunk ends with a release, a workgroup barrier and an arrival count
+static double copy_us(double bytes, int chunks, int wgs) { return bytes / (wgs * 33.0e3) + 6.0 * chunks; }
+static FusedEstimate estimate_fused(const GemmSchedule& s, int cus, int grid) {
+  const double tile_us = 2.0 * s.BM * s.BN * s.K / 6.0e6 + 8.0;
+  const int tiles = (s.M / s.BM) * ceil_div(s.N, s.BN);
+  const int tiles_per_cb = (s.comm_block_m / s.BM) * ceil_div(s.N, s.BN);
+  FusedEstimate e;
+  e.producer_wgs = cus - grid < kMaxProducerWgs ? cus - grid : kMaxProducerWgs;
+  if (e.producer_wgs < 1) e.producer_wgs = 1;
+  const double remote_bytes = 2.0 * 2.0 * s.M * s.K * (s.world_size - 1) / s.world_size;
+  e.gemm_us = ceil_div(tiles, grid) * tile_us;
+  e.copy_us = copy_us(remote_bytes, s.M / s.comm_block_m, e.producer_wgs);
+  const double tail_us = e.copy_us + ceil_div(tiles_per_cb, grid) * tile_us;
+  e.total_us = e.gemm_us > tail_us ? e.gemm_us : tail_us;
+  return e;
+}
+
 // smr_set_ag_matmul_halves: ring positions cut into half tiles at either end of a
 // gated launch, or -1 to let make_schedule choose.
 static int g_force_head = -1, g_force_tail = -1;
@@ -637,6 +663,22 @@ static GemmSchedule make_schedule(int M, int N, int K, int rank, int world_size,
   const int passes = (total + max_grid - 1) / max_grid;
   const int need = ((total + passes - 1) / passes + 7) / 8 * 8;
   s.grid = need < max_grid ? need : max_grid;
+  if (gated) {
+    // The producer runs on the compute units this grid leaves free, and a small or
+    // skinny problem is over before a narrow producer has copied the shards.  Take
+    // the grid (a multiple of 8) for which the later of the two - the GEMM's passes,
+    // or the last chunk's arrival plus the tiles that wait for it - comes earliest;
+    // among equals the smallest grid.
+    const FusedEstimate base = estimate_fused(s, cus, s.grid);
+    double best = base.total_us;
+    for (int g = 8; g <= max_grid; g += 8) {
+      const double t = estimate_fused(s, cus, g).total_us;
+      if (t < best * 0.97) {             // only for a clear gain: the model is coarse
+        best = t;
+        s.grid = g;
+      }
+    }
+  }
   // Gated launches: cut the local comm block (and, if that is what balances the
   // passes, the last one too) into half-width tiles when it costs no extra time.
   const int n_comm = M / comm_block_m;
@@ -695,6 +737,29 @@ int smr_set_ag_matmul_halves(int head, int tail) {
   if ((head < 0) != (tail < 0)) return smr::fail(SMR_E_INVALID, "smr_set_ag_matmul_halves: both or neither negative");
   smr::g_force_head = head;
   smr::g_force_tail = tail;
+  return 0;
+}
+
+int smr_ag_matmul_plan(int M, int N, int K, int world_size, int comm_block_m, int32_t* out4) {
+  using namespace smr;
+  const char* why;
+  if (int rc = validate(M, N, K, 0, world_size, comm_block_m, &why)) return fail(rc, why);
+  if (out4 == nullptr) return fail(SMR_E_INVALID, "smr_ag_matmul_plan: out4 is NULL");
+  const int cus = cu_count();
+  const GemmSchedule s = make_schedule(M, N, K, 0, world_size, comm_block_m, cus, true);
+  FusedEstimate e = estimate_fused(s, cus, s.grid);
+  // A copy that would be done long before the GEMM is paced: all of its workgroups for
+  // the first three chunks, two thirds of (at most 24 of) them for the rest.  A copy
+  // the GEMM has to wait for runs flat out.
+  int wgs = e.producer_wgs;
+  const int narrow = wgs > 24 ? 24 : wgs;
+  const double remote_bytes = 2.0 * 2.0 * M * K * (world_size - 1) / world_size;
+  const bool paced = copy_us(remote_bytes, M / comm_block_m, narrow) < 0.9 * e.gemm_us;
+  if (paced) wgs = narrow;
+  out4[0] = s.grid;
+  out4[1] = wgs;
+  out4[2] = paced ? 3 : 0;
+  out4[3] = paced ? (2 * wgs + 2) / 3 : 0;
   return 0;
 }
 

@@ -5,9 +5,9 @@
 // On one GPU the same role is played by a deliberately small copy kernel: a few
 // workgroups walk the chunks in the reference's order (sources rank+1, ...,
 // rank+ws-1, rank), stream every chunk with 128-bit non-temporal loads and
-// stores, and the last workgroup to finish a chunk release-stores its flag.
+// write-through stores, and the last workgroup to finish a chunk raises its flag.
 // "Last" is decided by a per-chunk arrival counter, so the flag is raised once
-// all of the chunk's bytes have been written and released.
+// all of the chunk's bytes have been written and acknowledged.
 //
 // The grid is small on purpose: the consumer GEMM owns the compute units.  It is
 // also paced.  The copy's traffic lengthens the GEMM's L2 misses (a GEMM next to a
@@ -34,6 +34,11 @@ static int g_gather_slow_workgroups = 16;
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef __attribute__((address_space(1))) u32x4 GlobalVec;
 
+// 128-bit store at agent scope: written through the XCD's L2.
+__device__ __forceinline__ void store_through(GlobalVec* p, u32x4 v) {
+  asm volatile("global_store_dwordx4 %0, %1, off sc1" : : "v"(p), "v"(v) : "memory");
+}
+
 __global__ __launch_bounds__(kGatherThreads) void all_gather_kernel(
     const uint64_t* __restrict__ buffer_ptrs, uint8_t* __restrict__ a_out,
     uint32_t* __restrict__ progress, uint32_t* __restrict__ counters, int rank, int world_size,
@@ -59,22 +64,24 @@ __global__ __launch_bounds__(kGatherThreads) void all_gather_kernel(
 #pragma unroll
         for (int u = 0; u < 8; ++u) v[u] = __builtin_nontemporal_load(src + i + u * stride);
 #pragma unroll
-        for (int u = 0; u < 8; ++u) __builtin_nontemporal_store(v[u], dst + i + u * stride);
+        for (int u = 0; u < 8; ++u) store_through(dst + i + u * stride, v[u]);
       }
       for (; i < chunk_vecs; i += stride) {
         u32x4 v = __builtin_nontemporal_load(src + i);
-        __builtin_nontemporal_store(v, dst + i);
+        store_through(dst + i, v);
       }
-      // publish: every wave releases its stores, the workgroup meets, one thread
-      // counts the arrival; the last arrival raises the flag.
-      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+      // publish: the stores went through to where every XCD sees them, so a thread
+      // only has to wait for their acknowledgement - no cache-wide write-back, which
+      // two thousand waves per chunk would queue up for.  Then the workgroup meets,
+      // one thread counts the arrival, and the last arrival raises the flag.
+      wait_stores_acknowledged();
       __syncthreads();
       if (threadIdx.x == 0) {
         const uint32_t prev =
-            __hip_atomic_fetch_add(&counters[idx], 1u, __ATOMIC_ACQ_REL, kScope);
+            __hip_atomic_fetch_add(&counters[idx], 1u, __ATOMIC_RELAXED, kScope);
         if (prev + 1u == (uint32_t)nwg) {
           __hip_atomic_store(&counters[idx], 0u, __ATOMIC_RELAXED, kScope);
-          __hip_atomic_store(&progress[idx], 1u, __ATOMIC_RELEASE, kScope);
+          __hip_atomic_store(&progress[idx], 1u, __ATOMIC_RELAXED, kScope);
           if (trace != nullptr && idx < kTraceProducerWords - 1) trace[idx] = wall_clock64();
         }
       }

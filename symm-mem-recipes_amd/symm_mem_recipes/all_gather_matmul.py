@@ -10,6 +10,7 @@ comparator ``all_gather_matmul`` (:322-326).
 """
 from __future__ import annotations
 
+import ctypes
 import os
 from typing import Optional
 
@@ -18,9 +19,10 @@ import torch
 from . import _lib
 from .symm_mem import EmulatedSymmetricMemory, _get_backend_stream
 
-#: Upper bound on the producer's workgroups (it never gets more than the compute
-#: units the GEMM's grid leaves free).
-MAX_PRODUCER_WORKGROUPS = 24
+#: Producer width and pacing of a fused launch.  None = the library's plan for the
+#: shape (smr_ag_matmul_plan); a number / a (fast_chunks, slow_workgroups) pair overrides.
+MAX_PRODUCER_WORKGROUPS = None
+PRODUCER_PACING = None
 
 
 def all_gather_with_progress(output: torch.Tensor, inp: torch.Tensor, progress: torch.Tensor,
@@ -113,12 +115,11 @@ def all_gather_matmul_tma_persistent(a_shard: torch.Tensor, b: torch.Tensor, a_o
         backend.wait_stream(current)
         flags.record_stream(backend)
         assert a_out.dtype == a_shard.dtype and a_out.is_contiguous()
-        # the producer takes the compute units the GEMM's grid leaves free
-        grid = lib.smr_ag_matmul_grid(M, N, K, world_size, COMM_BLOCK_SIZE_M, 1)
-        if grid < 0:
-            _lib.check(grid, "all_gather_matmul")
-        cus = torch.cuda.get_device_properties(device).multi_processor_count
-        producer_wgs = max(8, min(MAX_PRODUCER_WORKGROUPS, cus - grid))
+        # the producer takes (some of) the compute units the GEMM's grid leaves free
+        plan = (ctypes.c_int32 * 4)()
+        _lib.check(lib.smr_ag_matmul_plan(M, N, K, world_size, COMM_BLOCK_SIZE_M, plan), "all_gather_matmul")
+        producer_wgs = plan[1] if MAX_PRODUCER_WORKGROUPS is None else min(MAX_PRODUCER_WORKGROUPS, plan[1])
+        pacing = (plan[2], plan[3]) if PRODUCER_PACING is None else PRODUCER_PACING
 
     # The GEMM goes first: its first tiles are local rows and need no flag, so the
     # producer's launch latency is hidden behind them instead of delaying the GEMM.
@@ -128,6 +129,7 @@ def all_gather_matmul_tma_persistent(a_shard: torch.Tensor, b: torch.Tensor, a_o
                            current.cuda_stream)
     _lib.check(rc, "all_gather_matmul")
     if not mm_only:
+        _lib.check(lib.smr_set_gather_pacing(int(pacing[0]), int(pacing[1])), "all_gather_matmul")
         _launch_producer(symm_mem, a_out, a_shard, progress, counters, splits_per_rank, producer_wgs,
                          backend.cuda_stream)
         current.wait_stream(backend)

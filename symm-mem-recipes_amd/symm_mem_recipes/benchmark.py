@@ -1,0 +1,108 @@
+"""Shape sweep of the all-gather matmul, one row per problem as in the tables of the
+reference's README (symm_mem_recipes/README.md:17-36) and with its harness's method
+(utils.py:56-82: warm-up, last-level-cache flush before every timed call, median of
+event-timed iterations).
+
+    python -m symm_mem_recipes.benchmark --M 16384 --N 3584 --K 8192
+    python -m symm_mem_recipes.benchmark --readme
+
+Columns (README's in brackets): library matmul only [cublas mm only], this library's
+GEMM with flags preset [triton mm only], gather then library matmul [cublas + nccl]
+and the fused flag-gated launch [triton fused].  The eight ranks are emulated in one
+GPU's memory: the "gather" is a device copy, not a link transfer.
+"""
+from __future__ import annotations
+
+import argparse
+import statistics
+
+import torch
+
+from .all_gather_matmul import all_gather_matmul, all_gather_matmul_tma_persistent
+from .symm_mem import EmulatedSymmetricMemory
+
+#: (name, N, K) of the README's three model shapes; M is swept over README_MS
+README_SHAPES = (("Llama 3 8B", 1792, 4096), ("Llama 3 70B", 3584, 8192), ("Llama 3 105B", 6656, 16384))
+README_MS = (4096, 8192, 16384)
+
+
+def _median_us(fn, flush, warmup, iters):
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    times = []
+    for _ in range(iters):
+        flush.zero_()
+        a = torch.cuda.Event(enable_timing=True)
+        b = torch.cuda.Event(enable_timing=True)
+        a.record()
+        fn()
+        b.record()
+        torch.cuda.synchronize()
+        times.append(a.elapsed_time(b) * 1e3)
+    return statistics.median(times)
+
+
+def benchmark_all_gather_matmul(M: int, N: int, K: int, world_size: int = 8, rank: int = 0,
+                                warmup: int = 20, iters: int = 25, device=None) -> dict:
+    """Median microseconds of the four variants for one problem; inputs N(0, 0.02)
+    seeded as the reference seeds its harness (42 + rank)."""
+    device = torch.device("cuda:0") if device is None else device
+    a_shard = EmulatedSymmetricMemory.empty_strided_p2p((M // world_size, K), (K, 1), torch.bfloat16,
+                                                        device, world_size=world_size, rank=rank)
+    h = EmulatedSymmetricMemory.rendezvous(a_shard)
+    g = torch.Generator(device=device)
+    for r in range(world_size):
+        g.manual_seed(42 + r)
+        h.get_buffer(r, (M // world_size, K), torch.bfloat16).normal_(0, 0.02, generator=g)
+    g.manual_seed(41)
+    b = torch.empty(N, K, dtype=torch.bfloat16, device=device).normal_(0, 0.02, generator=g)
+    a_out = torch.cat([h.get_buffer(r, (M // world_size, K), torch.bfloat16) for r in range(world_size)])
+    c = torch.empty(M, N, dtype=torch.bfloat16, device=device)
+    flush = torch.empty(1 << 28, dtype=torch.int32, device=device)          # 1 GiB
+    res = {
+        "M": M, "N": N, "K": K,
+        "library_mm_only_us": _median_us(lambda: torch.matmul(a_out, b.T, out=c), flush, warmup, iters),
+        "hip_mm_only_us": _median_us(
+            lambda: all_gather_matmul_tma_persistent(a_shard, b, a_out, c, None, mm_only=True),
+            flush, warmup, iters),
+        "library_gather_mm_us": _median_us(lambda: all_gather_matmul(a_shard, b.T), flush, warmup, iters),
+        "hip_fused_us": _median_us(lambda: all_gather_matmul_tma_persistent(a_shard, b, a_out, c, None),
+                                   flush, warmup, iters),
+    }
+    h.check_status()
+    res["tflops_fused"] = 2.0 * M * N * K / res["hip_fused_us"] / 1e6
+    res["tflops_mm_only"] = 2.0 * M * N * K / res["hip_mm_only_us"] / 1e6
+    EmulatedSymmetricMemory.release(a_shard)
+    return res
+
+
+def _row(r):
+    return (f"| {r['M']} | {r['library_mm_only_us']:.0f} | {r['hip_mm_only_us']:.0f} | "
+            f"{r['library_gather_mm_us']:.0f} | {r['hip_fused_us']:.0f} | {r['tflops_fused']:.0f} |")
+
+
+def main(argv=None):
+    ap = argparse.ArgumentParser(description=__doc__.split("\n\n")[0])
+    ap.add_argument("--M", type=int, default=16384)
+    ap.add_argument("--N", type=int, default=3584)
+    ap.add_argument("--K", type=int, default=8192)
+    ap.add_argument("--world-size", type=int, default=8)
+    ap.add_argument("--rank", type=int, default=0)
+    ap.add_argument("--readme", action="store_true", help="all nine problems of the reference's README")
+    args = ap.parse_args(argv)
+    head = ("| Problem Size (M) | library mm only (us) | hip mm only (us) | library gather + mm (us) | "
+            "hip fused (us) | fused TFLOP/s |\n|---|---|---|---|---|---|")
+    if args.readme:
+        for name, n, k in README_SHAPES:
+            print(f"#### {name} (N={n}, K={k})\n{head}", flush=True)
+            for m in README_MS:
+                print(_row(benchmark_all_gather_matmul(m, n, k, args.world_size, args.rank)), flush=True)
+            print(flush=True)
+    else:
+        print(head)
+        print(_row(benchmark_all_gather_matmul(args.M, args.N, args.K, args.world_size, args.rank)))
+
+
+if __name__ == "__main__":
+    main()
