@@ -169,7 +169,7 @@ int smr_all_gather_with_progress(const uint64_t* buffer_ptrs_dev, void* a_out_de
 
 /* Pacing of the producer: the first `fast_chunks` chunks are copied by all
  * workgroups, the remaining ones by `slow_workgroups` of them (0 = all, i.e. no
- * pacing).  Default 3 and 16.  No reference counterpart (copy engines pace
+ * pacing).  Default 0 and 0.  No reference counterpart (copy engines pace
  * themselves by link speed). */
 int smr_set_gather_pacing(int fast_chunks, int slow_workgroups);
 
@@ -195,15 +195,15 @@ int smr_ag_matmul_schedule(int M, int N, int K, int rank, int world_size, int co
 
 /* Host-only: how a fused launch of this shape splits the GPU.  out4 = {GEMM grid (what
  * smr_ag_matmul will launch when gated), producer workgroups, fast_chunks,
- * slow_workgroups} - the last two are the arguments of smr_set_gather_pacing, {0, 0} when
- * the copy should run flat out because the GEMM would otherwise wait for it.  Replaces
+ * slow_workgroups} - the last two are the arguments of smr_set_gather_pacing ({0, 0}: the
+ * copy runs flat out).  Replaces
  * the fixed NUM_SMS grid of triton_all_gather_matmul.py:287-294: there the copy engines
  * cost no SMs. */
 int smr_ag_matmul_plan(int M, int N, int K, int world_size, int comm_block_m, int32_t* out4);
 
 /* Tuning knob of the gated schedule: the first `head` and the last `tail` comm blocks
  * of the ring order are computed in tiles of half the width.  Both -1 (the default)
- * lets the library choose.  No reference counterpart. */
+ * means none.  No reference counterpart. */
 int smr_set_ag_matmul_halves(int head, int tail);
 
 /* Workgroups smr_ag_matmul launches on the current device for this shape; a

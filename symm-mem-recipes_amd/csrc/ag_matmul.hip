@@ -44,10 +44,10 @@ struct GemmSchedule {
   int BM, BN;
   int grid;                      // persistent workgroups, a multiple of 8
   // The comm blocks are visited in ring order starting at the local one.  The
-  // first `head` and the last `tail` ring positions (0 or 1 each) are cut into
-  // tiles of half the width: a pass over half tiles takes half as long, so with the
-  // local comm block in halves every workgroup starts on rows that need no flag,
-  // and the producer gets that half pass as a head start.
+  // first `head` and the last `tail` ring positions can be cut into tiles of half
+  // the width (smr_set_ag_matmul_halves; 0 and 0 by default): a pass over half
+  // tiles takes half as long, so with the local comm block in halves every
+  // workgroup starts on rows that need no flag.
   int head, tail;
   int steps;                     // trips of the busiest workgroup (passes over all phases)
 };
@@ -679,20 +679,15 @@ static GemmSchedule make_schedule(int M, int N, int K, int rank, int world_size,
       }
     }
   }
-  // Gated launches: cut the local comm block (and, if that is what balances the
-  // passes, the last one too) into half-width tiles when it costs no extra time.
+  // Half-width phases are off unless asked for (smr_set_ag_matmul_halves).  They let
+  // every workgroup of a gated launch start on local rows, but half tiles are bound
+  // by their loads, and with a producer that delivers a chunk in less than a pass it
+  // is cheaper to let the workgroups of the first remote comm block wait for it.
   const int n_comm = M / comm_block_m;
-  if (gated && s.BN == 256 && n_comm >= 3) {
-    const int base = schedule_cost(s);
-    GemmSchedule both = s, head = s;
-    both.head = both.tail = 1;
-    head.head = 1;
-    if (schedule_cost(both) <= base) s = both;
-    else if (schedule_cost(head) <= base) s = head;
-    if (g_force_head >= 0 && g_force_tail >= 0 && g_force_head + g_force_tail <= n_comm) {
-      s.head = g_force_head;
-      s.tail = g_force_tail;
-    }
+  if (gated && s.BN == 256 && g_force_head >= 0 && g_force_tail >= 0 &&
+      g_force_head + g_force_tail <= n_comm) {
+    s.head = g_force_head;
+    s.tail = g_force_tail;
   }
   s.steps = total_steps(s);
   return s;
@@ -748,18 +743,13 @@ int smr_ag_matmul_plan(int M, int N, int K, int world_size, int comm_block_m, in
   const int cus = cu_count();
   const GemmSchedule s = make_schedule(M, N, K, 0, world_size, comm_block_m, cus, true);
   FusedEstimate e = estimate_fused(s, cus, s.grid);
-  // A copy that would be done long before the GEMM is paced: all of its workgroups for
-  // the first three chunks, two thirds of (at most 24 of) them for the rest.  A copy
-  // the GEMM has to wait for runs flat out.
-  int wgs = e.producer_wgs;
-  const int narrow = wgs > 24 ? 24 : wgs;
-  const double remote_bytes = 2.0 * 2.0 * M * K * (world_size - 1) / world_size;
-  const bool paced = copy_us(remote_bytes, M / comm_block_m, narrow) < 0.9 * e.gemm_us;
-  if (paced) wgs = narrow;
+  // The copy runs flat out on what the grid leaves free: with write-through stores it
+  // no longer pays to hold it back (pacing it to two thirds of its width cost 3 % on
+  // the M=16384 N=3584 K=8192 problem, where it used to gain 2 %).
   out4[0] = s.grid;
-  out4[1] = wgs;
-  out4[2] = paced ? 3 : 0;
-  out4[3] = paced ? (2 * wgs + 2) / 3 : 0;
+  out4[1] = e.producer_wgs;
+  out4[2] = 0;
+  out4[3] = 0;
   return 0;
 }
 

@@ -9,14 +9,14 @@
 // "Last" is decided by a per-chunk arrival counter, so the flag is raised once
 // all of the chunk's bytes have been written and acknowledged.
 //
-// The grid is small on purpose: the consumer GEMM owns the compute units.  It is
-// also paced.  The copy's traffic lengthens the GEMM's L2 misses (a GEMM next to a
-// copy of all eight chunks at 0.75 TB/s takes 12 % longer; a loop of nothing but
-// MFMAs next to the same copy only 2 %, so it is the memory path, not power), and
-// more so the faster the copy runs.  So only the first chunks - the ones the
-// consumer is about to ask for - are copied by all workgroups; after them all but
-// a few workgroups leave and the rest of the gather arrives just ahead of the
-// consumer.
+// The grid is small on purpose: the consumer GEMM owns most compute units, and the
+// caller sizes the producer to what the GEMM's grid leaves free.  The stores are
+// written through the L2 (agent scope) and a chunk is published by waiting for their
+// acknowledgement: releasing cached stores instead costs a cache-wide write-back per
+// wave and chunk, which stalled the GEMM next to it (fused M=16384 N=3584 K=8192:
+// 860 us with the write-backs, 760 us without).  The producer can be paced
+// (smr_set_gather_pacing: full width for the first chunks, fewer workgroups after);
+// with write-through stores that no longer gains anything and is off by default.
 #include "smr_device.hpp"
 
 namespace smr {
@@ -28,8 +28,8 @@ constexpr int kGatherThreads = 1024;
 constexpr int kGatherDefaultWorkgroups = 8;
 // Pacing (smr_set_gather_pacing): chunks copied at full width, workgroups that stay
 // for the rest.
-static int g_gather_fast_chunks = 3;
-static int g_gather_slow_workgroups = 16;
+static int g_gather_fast_chunks = 0;
+static int g_gather_slow_workgroups = 1024;
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef __attribute__((address_space(1))) u32x4 GlobalVec;
