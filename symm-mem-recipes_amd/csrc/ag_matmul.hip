@@ -559,10 +559,14 @@ __global__ __launch_bounds__(kGemmThreads, 1) void ag_matmul_kernel(
   }
 }
 
-static int pick_tile(int M, int N, int comm_block_m, int& BM, int& BN) {
+// Tile shape: the largest the flags' granularity allows, stepped down while the
+// problem has too few tiles to occupy more than half of the compute units.
+static int pick_tile(int M, int N, int comm_block_m, int& BM, int& BN, int cus = 256) {
   if (comm_block_m % 256 == 0) {
     BM = 256;
     BN = N >= 256 ? 256 : 128;
+    if (BN == 256 && (M / 256) * ceil_div(N, 256) * 2 <= cus) BN = 128;
+    if (BN == 128 && (M / 256) * ceil_div(N, 128) * 2 <= cus) BM = 128;
   } else if (comm_block_m % 128 == 0) {
     BM = 128;
     BN = 128;
@@ -655,7 +659,7 @@ static GemmSchedule make_schedule(int M, int N, int K, int rank, int world_size,
   s.M = M; s.N = N; s.K = K;
   s.rank = rank; s.world_size = world_size; s.comm_block_m = comm_block_m;
   s.head = s.tail = 0;
-  pick_tile(M, N, comm_block_m, s.BM, s.BN);
+  pick_tile(M, N, comm_block_m, s.BM, s.BN, cus);
   const int tn = (N + s.BN - 1) / s.BN;
   const int total = (M / s.BM) * tn;
   int max_grid = ((gated ? cus - kReservedCus : cus) / 8) * 8;

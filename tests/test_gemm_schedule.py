@@ -101,7 +101,7 @@ def test_schedule_forced_half_tile_phases(lib, head, tail):
     phase and have work again in the next one."""
     try:
         assert lib.smr_set_ag_matmul_halves(head, tail) == 0
-        for (M, N, K, ws) in [(4096, 640, 192, 8), (16384, 3584, 8192, 8), (8192, 4096, 256, 8)]:
+        for (M, N, K, ws) in [(8192, 1280, 192, 8), (16384, 3584, 8192, 8), (8192, 4096, 256, 8)]:
             for rank in (0, 5):
                 s = gemm_schedule(M, N, K, rank, ws, M // ws)
                 _covers_exactly(s, M, N)

@@ -114,7 +114,7 @@ def test_fused_parity_half_tile_phases(cuda, lib, head, tail):
     """Every split of the gated schedule into half-width and full-width phases computes
     the same product (the library picks one by cost; this forces the others)."""
     from symm_mem_recipes import all_gather_matmul_tma_persistent
-    M, N, K, ws, rank = 4096, 640, 192, 8, 5
+    M, N, K, ws, rank = 8192, 1280, 192, 8, 5        # enough 256x256 tiles that the library keeps that shape
     a_shard, h, shards, b, b_bits, a_out, c_out = _setup(M, N, K, ws, rank, cuda)
     try:
         assert lib.smr_set_ag_matmul_halves(head, tail) == 0
