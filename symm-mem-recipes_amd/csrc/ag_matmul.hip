@@ -50,6 +50,7 @@ struct GemmSchedule {
   // workgroup starts on rows that need no flag.
   int head, tail;
   int steps;                     // trips of the busiest workgroup (passes over all phases)
+  int group_m;                   // row tiles per group of the tile order; divides the comm block's
 };
 
 struct TileRef {
@@ -66,7 +67,9 @@ __host__ __device__ inline int ceil_div(int a, int b) { return (a + b - 1) / b; 
 // Three phases: `head` ring positions in half tiles, the middle in full tiles, `tail`
 // in half tiles.  A phase is walked in passes of `grid` tiles; within a pass XCD x
 // (workgroups with id % 8 == x) takes a contiguous run of the tile order.  The tile
-// order inside a phase is comm block (ring order), then column tile, then row tile.
+// order inside a phase is comm block (ring order), then group of row tiles, then column
+// tile, then row tile: an XCD's run is then a patch about as wide as it is high, and
+// the workgroups that share an L2 load the fewest distinct A and B slabs.
 __host__ __device__ inline bool tile_for(const GemmSchedule& s, int wg, int step, TileRef& t) {
   const int cb_tiles_m = s.comm_block_m / s.BM;
   const int n_comm = s.M / s.comm_block_m;
@@ -91,8 +94,12 @@ __host__ __device__ inline bool tile_for(const GemmSchedule& s, int wg, int step
       const int lin = start + in_pass;
       const int pos = lin / tiles_per_cb;
       const int rem = lin - pos * tiles_per_cb;
-      const int tile_n = rem / cb_tiles_m;
-      const int tile_m = rem - tile_n * cb_tiles_m;
+      // inside a comm block: groups of group_m row tiles, column by column inside a group
+      const int per_group = s.group_m * tn;
+      const int group = rem / per_group;
+      const int in_group = rem - group * per_group;
+      const int tile_n = in_group / s.group_m;
+      const int tile_m = group * s.group_m + (in_group - tile_n * s.group_m);
       const int cb = (first_local + ring0 + pos) % n_comm;
       t.comm_block = cb;
       t.row0 = cb * s.comm_block_m + tile_m * s.BM;
@@ -692,6 +699,23 @@ static GemmSchedule make_schedule(int M, int N, int K, int rank, int world_size,
       g_force_head + g_force_tail <= n_comm) {
     s.head = g_force_head;
     s.tail = g_force_tail;
+  }
+  // Rows per group: the divisor of the comm block's row tiles for which an XCD's run of
+  // a full pass touches the fewest slabs (rows of the patch + columns of the patch).
+  {
+    const int cb_tiles_m = comm_block_m / s.BM;
+    const int per_xcd = ceil_div(total < s.grid ? total : s.grid, 8);
+    int best_cost = 1 << 30;
+    s.group_m = cb_tiles_m;
+    for (int g = 1; g <= cb_tiles_m; ++g) {
+      if (cb_tiles_m % g != 0) continue;
+      const int rows = g < per_xcd ? g : per_xcd;
+      const int cost = rows + ceil_div(per_xcd, g);
+      if (cost < best_cost || (cost == best_cost && g > s.group_m)) {
+        best_cost = cost;
+        s.group_m = g;
+      }
+    }
   }
   s.steps = total_steps(s);
   return s;
