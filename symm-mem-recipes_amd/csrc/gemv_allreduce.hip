@@ -6,8 +6,11 @@
 // The job is bound by reading W once (K*N*2 bytes).  W is row-major [K, N], so a
 // row is N contiguous bf16: TPR threads cover a row segment with one 128-bit load
 // each, and the 256/TPR thread groups of a workgroup stride over the K rows of
-// their share with 4 to 16 independent loads in flight per thread.  x (at most 8
-// rows) is staged in LDS as fp32, transposed to [k][batch].
+// their share, two rows at a time, with 4 to 16 independent loads in flight per
+// thread.  x (at most 8 rows) is staged in LDS as pairs of consecutive k,
+// transposed to [k/2][batch]; a byte permute pairs W[k][j] with W[k+1][j], and one
+// v_dot2c_f32_bf16 per column and batch row does both multiply-adds (half the
+// vector instructions of convert-and-FMA, which is what a batch of 8 was bound by).
 //
 // Workgroup id -> (sender = rank * sub + sub-shard, column block), column block
 // fastest.  Every workgroup writes its fp32 partial, waits until the stores are
@@ -34,22 +37,24 @@ static int g_gemv_sub = 0;                   // 0 = pick so that >= 256 workgrou
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef __attribute__((address_space(1))) u32x4 GlobalVec;
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 
 template <int B, int TPR>
 __global__ __launch_bounds__(kGemvThreads) void gemv_allreduce_kernel(
     const uint16_t* __restrict__ x, const uint8_t* __restrict__ w, float* __restrict__ partials,
     uint32_t* __restrict__ flags, uint16_t* __restrict__ out, int batch, int K, int N,
     int world_size, int sub, uint64_t limit_ticks, uint32_t* status) {
-  // 128-bit loads in flight per thread: fewer for larger batches, whose 8*B
-  // accumulators would otherwise leave one wave per SIMD
-  constexpr int kGemvUnroll = B >= 8 ? 4 : (B >= 4 ? 8 : 16);
+  // Row pairs in flight per thread (two 128-bit loads each): fewer for larger
+  // batches, whose 8*B accumulators would otherwise leave one wave per SIMD
+  constexpr int kGemvUnroll = B >= 8 ? 2 : (B >= 4 ? 4 : 8);
   constexpr int kCols = TPR * 8;                         // columns per workgroup
   constexpr int kKGroups = kGemvThreads / TPR;           // row groups per workgroup
   constexpr int kKGroupsPerWave = 64 / TPR;
   // x staging and the cross-wave reduction never live at the same time: one buffer
-  constexpr int kXsFloats = kGemvKChunk * B, kRedFloats = (kGemvThreads / 64) * B * kCols;
-  __shared__ __attribute__((aligned(16))) float smem[kXsFloats > kRedFloats ? kXsFloats : kRedFloats];
-  float (*xs)[B] = reinterpret_cast<float (*)[B]>(smem);
+  constexpr int kXsWords = kGemvKChunk / 2 * B, kRedFloats = (kGemvThreads / 64) * B * kCols;
+  __shared__ __attribute__((aligned(16))) float smem[kXsWords > kRedFloats ? kXsWords : kRedFloats];
+  // x as bf16 pairs of consecutive k: word [k/2][batch] = x[batch][k] | x[batch][k+1] << 16
+  uint32_t (*xp)[B] = reinterpret_cast<uint32_t (*)[B]>(smem);
   float (*red)[B][kCols] = reinterpret_cast<float (*)[B][kCols]>(smem);
 
   // Column block fastest: workgroups with neighbouring ids read neighbouring 1 KiB
@@ -80,13 +85,17 @@ __global__ __launch_bounds__(kGemvThreads) void gemv_allreduce_kernel(
 
   for (int k0 = k_begin; k0 < k_end; k0 += kGemvKChunk) {
     const int kc = (k_end - k0) < kGemvKChunk ? (k_end - k0) : kGemvKChunk;
-    // stage x[:, k0 .. k0+kc) as fp32, transposed to [k][batch]
+    // stage x[:, k0 .. k0+kc) as pairs, transposed to [k/2][batch]; zero past the end
 #pragma unroll
     for (int b = 0; b < B; ++b) {
 #pragma unroll
-      for (int i = 0; i < kGemvKChunk / kGemvThreads; ++i) {
-        const int k = tid + i * kGemvThreads;
-        if (k < kc) xs[k][b] = b < batch ? bf16_lo((uint32_t)x[(int64_t)b * K + k0 + k]) : 0.0f;
+      for (int i = 0; i < kGemvKChunk / 2 / kGemvThreads; ++i) {
+        const int kp = tid + i * kGemvThreads;
+        const int k = 2 * kp;
+        uint32_t lo = 0, hi = 0;
+        if (b < batch && k < kc) lo = x[(int64_t)b * K + k0 + k];
+        if (b < batch && k + 1 < kc) hi = x[(int64_t)b * K + k0 + k + 1];
+        xp[kp][b] = lo | (hi << 16);
       }
     }
     __syncthreads();
@@ -94,30 +103,34 @@ __global__ __launch_bounds__(kGemvThreads) void gemv_allreduce_kernel(
       const __attribute__((address_space(1))) uint8_t* wp =
           (const __attribute__((address_space(1))) uint8_t*)(uintptr_t)(w + (int64_t)k0 * row_bytes +
                                                                       (int64_t)col0 * 2);
-      for (int k = kg; k < kc; k += kKGroups * kGemvUnroll) {
-        u32x4 wv[kGemvUnroll];
+      const int pairs = (kc + 1) >> 1;
+      for (int p = kg; p < pairs; p += kKGroups * kGemvUnroll) {
+        u32x4 w0[kGemvUnroll], w1[kGemvUnroll];
 #pragma unroll
         for (int u = 0; u < kGemvUnroll; ++u) {
-          // rows past the end are re-read from the last valid row and weighted by 0
-          const int kk = k + u * kKGroups;
-          const int kr = kk < kc ? kk : kc - 1;
-          wv[u] = __builtin_nontemporal_load((const GlobalVec*)(wp + (int64_t)kr * row_bytes));
+          // rows past the end are re-read from the last valid row; their x is 0
+          const int k = 2 * (p + u * kKGroups);
+          const int r0 = k < kc ? k : kc - 1, r1 = k + 1 < kc ? k + 1 : kc - 1;
+          w0[u] = __builtin_nontemporal_load((const GlobalVec*)(wp + (int64_t)r0 * row_bytes));
+          w1[u] = __builtin_nontemporal_load((const GlobalVec*)(wp + (int64_t)r1 * row_bytes));
         }
 #pragma unroll
         for (int u = 0; u < kGemvUnroll; ++u) {
-          const int kk = k + u * kKGroups;
-          const bool live = kk < kc;
-          const int kr = live ? kk : kc - 1;
-          float wf[8];
-          wf[0] = bf16_lo(wv[u].x); wf[1] = bf16_hi(wv[u].x);
-          wf[2] = bf16_lo(wv[u].y); wf[3] = bf16_hi(wv[u].y);
-          wf[4] = bf16_lo(wv[u].z); wf[5] = bf16_hi(wv[u].z);
-          wf[6] = bf16_lo(wv[u].w); wf[7] = bf16_hi(wv[u].w);
+          const int pp = p + u * kKGroups;
+          const int pr = pp < kGemvKChunk / 2 ? pp : kGemvKChunk / 2 - 1;   // (its x words are 0 there)
+          // (W[k][j], W[k+1][j]) as one bf16 pair per column: two byte permutes per word
+          uint32_t wq[8];
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            wq[2 * q] = __builtin_amdgcn_perm(w1[u][q], w0[u][q], 0x05040100u);
+            wq[2 * q + 1] = __builtin_amdgcn_perm(w1[u][q], w0[u][q], 0x07060302u);
+          }
 #pragma unroll
           for (int b = 0; b < B; ++b) {
-            const float xb = live ? xs[kr][b] : 0.0f;
+            const bf16x2 xb = __builtin_bit_cast(bf16x2, pp < pairs ? xp[pr][b] : 0u);
 #pragma unroll
-            for (int j = 0; j < 8; ++j) acc[b][j] = __builtin_fmaf(xb, wf[j], acc[b][j]);
+            for (int j = 0; j < 8; ++j)
+              acc[b][j] = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, wq[j]), xb, acc[b][j], false);
           }
         }
       }
