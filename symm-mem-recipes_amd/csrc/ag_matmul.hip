@@ -8,21 +8,22 @@
 //     but draws more power, and the clock of a GEMM this size is power-limited);
 //   * both operands are K-contiguous, so a tile's K-slab (rows x 64 bf16 = 128 B
 //     per row) is brought straight from global memory into LDS with 128-bit
-//     direct-to-LDS loads (no staging registers), two stages deep: the loads of
-//     slab k+1 are in flight while slab k is multiplied;
+//     direct-to-LDS loads (no staging registers).  LDS is a ring of five slots that
+//     hold one slab each (2.5 slab pairs): while one pair is multiplied, up to three
+//     slabs are landing, and only half of a pair's bytes are ever due within one
+//     pair's time;
 //   * an LDS row is 8 chunks of 16 B; chunk c of row r is stored at position
 //     c ^ row_swizzle(r), which keeps the 128-bit fragment reads free of bank
 //     conflicts;
 //   * the MFMA is issued with the B fragment as its first operand, so a lane
-//     ends up with 4 consecutive output columns of one row and stores 8 bytes
-//     at a time;
+//     ends up with 4 consecutive output columns of one row; the epilogue turns 32
+//     rows at a time through LDS and stores whole rows;
 //   * tiles are walked in the ready order of the all-gather: all tiles of the
 //     local comm block first, then the comm blocks in ring order; a tile of a
 //     non-local comm block first waits for that block's progress flag.  Within
 //     one pass over the grid, XCD x (workgroups with id % 8 == x) takes a
-//     contiguous run of the tile order - 8 row tiles x 4 column tiles when the
-//     pass is full - so the workgroups that share an L2 also share A rows and
-//     B columns.
+//     contiguous run of the tile order - a patch about as wide as it is high - so
+//     the workgroups that share an L2 also share A rows and B columns.
 #include <type_traits>
 
 #include "smr_device.hpp"
@@ -32,10 +33,9 @@ namespace smr {
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef __attribute__((address_space(3))) void LdsVoid;
-typedef __attribute__((address_space(1))) void GlobalVoid;
 
 constexpr int kGemmThreads = 256;
-constexpr int kBK = 64;          // K extent of one LDS stage (128 bytes per row)
+constexpr int kBK = 64;          // K extent of one slab (128 bytes per row)
 constexpr int kRowBytes = kBK * 2;
 
 struct GemmSchedule {
@@ -122,15 +122,6 @@ __host__ __device__ inline bool next_tile(const GemmSchedule& s, int wg, int& st
   for (; step < s.steps; ++step)
     if (tile_for(s, wg, step, t)) return true;
   return false;
-}
-
-// Number of trips of the busiest workgroup, in units of half a full-tile pass.
-__host__ __device__ inline int schedule_cost(const GemmSchedule& s) {
-  const int cb_tiles_m = s.comm_block_m / s.BM;
-  const int n_comm = s.M / s.comm_block_m;
-  const int full = cb_tiles_m * ceil_div(s.N, s.BN), half = cb_tiles_m * ceil_div(s.N, s.BN / 2);
-  return ceil_div(s.head * half, s.grid) + 2 * ceil_div((n_comm - s.head - s.tail) * full, s.grid) +
-         ceil_div(s.tail * half, s.grid);
 }
 
 // Position swizzle of an LDS row: chunk c of slab row r is stored at position
