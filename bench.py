@@ -171,7 +171,7 @@ def bench_reduce_rotating(size_kib, dev, dtype_name="bf16", write_all=False, acc
     return res
 
 
-def bench_ag_matmul(dev):
+def bench_ag_matmul(dev, gated=True):
     import torch
     from symm_mem_recipes import EmulatedSymmetricMemory as SM, all_gather_matmul_tma_persistent
     M, N, K = 16384, 3584, 8192
@@ -190,7 +190,7 @@ def bench_ag_matmul(dev):
     us_ungated = _time_events(lambda: all_gather_matmul_tma_persistent(a_shard, b, a_out, c, None, mm_only=True),
                               25, 20, pre=flush.zero_)
     us_gated = _time_events(lambda: all_gather_matmul_tma_persistent(a_shard, b, a_out, c, None),
-                            25, 20, pre=flush.zero_)
+                            25, 20, pre=flush.zero_) if gated else float("nan")
     h.check_status()
     us_lib = _time_events(lambda: torch.matmul(a_out, b.T, out=c), 25, 20, pre=flush.zero_)
     SM.release()
@@ -329,6 +329,10 @@ def main():
     ap.add_argument("--size-mib", type=int, default=64)
     ap.add_argument("--no-extra", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=10.0)
+    ap.add_argument("--gemm-only", action="store_true",
+                    help="only the ungated GEMM and the library matmul of the same operands: the run to "
+                         "collect hardware counters on (a counter run serialises kernels, and a gated GEMM "
+                         "whose producer cannot run beside it only times out)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on exactly one GPU (the 8 ranks are emulated in one "
@@ -341,6 +345,10 @@ def main():
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+
+    if args.gemm_only:
+        print(json.dumps(bench_ag_matmul(dev, gated=False)))
+        return
 
     r = bench_reduce(args.size_mib, args.steps, args.warmup, dev)
     value = r["alg_bytes"] * args.steps / r["wall_s"] / 1e9
