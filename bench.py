@@ -29,6 +29,11 @@ HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
 # (profiles/one_shot_all_reduce_64MiB_bf16_traffic.md); keyed by MiB per buffer.
 MEASURED_REDUCE_TRAFFIC_BYTES = {64: 604405370}
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
+# Fabric bytes per launch of the ungated GEMM at M=16384 N=3584 K=8192 (FETCH_SIZE scaled
+# as above plus WRITE_SIZE; profiles/ag_matmul_M16384_N3584_K8192_counters.md).  A counter
+# run cannot hold the gated launch (it serialises kernels); the gated GEMM reads and writes
+# the same tiles in the same order.
+MEASURED_GEMM_TRAFFIC_BYTES = 1618400051
 WS = 8
 
 
@@ -200,7 +205,7 @@ def bench_ag_matmul(dev, gated=True):
                 gating_overhead=us_gated / us_ungated - 1.0,
                 roofline={"bound": "mfma", "achieved": flops / us_gated / 1e6, "peak": MFMA_BF16_PEAK_TFLOPS,
                           "unit": "TFLOP/s", "frac": flops / us_gated / 1e6 / MFMA_BF16_PEAK_TFLOPS,
-                          "traffic": None},
+                          "traffic": MEASURED_GEMM_TRAFFIC_BYTES},
                 torch_matmul_us=us_lib, torch_matmul_tflops=flops / us_lib / 1e6)
 
 
