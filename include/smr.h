@@ -193,6 +193,17 @@ int smr_ag_matmul(const void* a_shard_dev, const void* a_out_dev, const void* b_
 int smr_ag_matmul_schedule(int M, int N, int K, int rank, int world_size, int comm_block_m,
                            int gated, int32_t* out_records, int max_tiles);
 
+/* The same GEMM with e4m3fn (OCP FP8) operands and result, fp32 accumulation: the
+ * reference's FP8_OUTPUT switch (triton_all_gather_matmul.py:115,123,188,311).  The cast of
+ * the accumulator rounds to nearest even and saturates to +-448, NaN stays NaN (what
+ * Triton's cast compiles to on the reference's hardware, cvt.rn.satfinite).
+ * K % 128 == 0, N % 16 == 0, comm_block_m % 256 == 0; otherwise as smr_ag_matmul. */
+int smr_ag_matmul_fp8(const void* a_shard_dev, const void* a_out_dev, const void* b_nk_dev, void* c_dev,
+                      const uint32_t* progress_dev, int M, int N, int K, int rank, int world_size,
+                      int comm_block_m, uint32_t* status, void* stream);
+/* smr_ag_matmul_plan for the e4m3fn GEMM. */
+int smr_ag_matmul_plan_fp8(int M, int N, int K, int world_size, int comm_block_m, int32_t* out4);
+
 /* Host-only: how a fused launch of this shape splits the GPU.  out4 = {GEMM grid (what
  * smr_ag_matmul will launch when gated), producer workgroups, fast_chunks,
  * slow_workgroups} - the last two are the arguments of smr_set_gather_pacing ({0, 0}: the

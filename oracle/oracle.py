@@ -29,6 +29,9 @@ independent cross-check in the tests):
                            (triton_all_gather_matmul.py:125-174)
 * ``ag_matmul_ref``        cat + matmul (triton_all_gather_matmul.py:322-326),
                            NT layout and fp32 accumulate / bf16 store (:176-193)
+* ``ag_matmul_ref_fp8``    the same product with e4m3fn operands and result (the
+                           reference's FP8_OUTPUT switch, :115,123,188), with
+                           ``fp8_e4m3fn_to_f32`` / ``f32_to_fp8_e4m3fn``
 * ``gemv_allreduce_ref``   split-K GEMV + rank-ordered fp32 combine (no
                            reference code exists for it; closed form)
 * ``signal_round_ref``     checksum closed form for the producer/consumer
@@ -52,6 +55,14 @@ Pinning status (what the tests check each function against, other than itself):
   ag_matmul_ref      -> torch-CPU matmul (library), exact-rational brute force on
                         tiny shapes; the reference's own check is allclose against
                         all-gather + matmul (triton_all_gather_matmul.py:390-392)
+  fp8 conversions    -> torch CPU casts (library): decode exhaustive over all 256
+                        patterns, encode on random values, every midpoint and
+                        every representable value up to 448; beyond 448 torch
+                        gives NaN where the reference's hardware conversion
+                        saturates (PTX cvt.rn.satfinite): that branch is PARITY
+                        UNPINNED against the reference's toolchain and follows
+                        the published PTX semantics
+  ag_matmul_ref_fp8  -> torch-CPU matmul of the decoded operands + torch cast
   gemv_allreduce_ref -> PARITY UNPINNED against the reference (no reference code
                         or vectors exist for this path); pinned only against
                         the mathematics: x @ W library routine and
@@ -336,6 +347,60 @@ def ag_matmul_ref(shards_bits: Sequence[np.ndarray], b_nk_bits: np.ndarray,
     c = a @ b.T
     bits = f32_to_bf16_bits(c)
     return (bits, c) if return_f32 else bits
+
+
+# --------------------------------------------------------------------------
+# fp8 (e4m3fn) variant of the matmul: FP8_OUTPUT, triton_all_gather_matmul.py:115,123,188
+# --------------------------------------------------------------------------
+def fp8_e4m3fn_to_f32(bits: np.ndarray) -> np.ndarray:
+    """uint8 e4m3fn patterns -> float32 (OCP FP8: bias 7, no infinities, S.1111.111 = NaN)."""
+    b = np.ascontiguousarray(bits, dtype=np.uint8).astype(np.int32)
+    sign = np.where(b & 0x80, -1.0, 1.0)
+    e = (b >> 3) & 0xF
+    m = b & 0x7
+    val = np.where(e == 0, m * 2.0 ** -9, (8 + m) * 2.0 ** (e - 10.0))
+    val = np.where((e == 15) & (m == 7), np.nan, val)
+    return (sign * val).astype(np.float32)
+
+
+_FP8_POS = None
+
+
+def f32_to_fp8_e4m3fn(x: np.ndarray) -> np.ndarray:
+    """float32 -> uint8 e4m3fn, round to nearest even, saturating to +-448 (also for
+    infinities), NaN -> 0x7F: what Triton's cast to float8e4nv compiles to on the
+    reference's hardware, ``cvt.rn.satfinite.e4m3x2.f32`` (PTX ISA 8.x, "cvt"; the
+    CUDA toolkit is a third-party dependency outside the reference tree)."""
+    global _FP8_POS
+    if _FP8_POS is None:
+        _FP8_POS = fp8_e4m3fn_to_f32(np.arange(127, dtype=np.uint8)).astype(np.float64)   # 0 .. 448
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    a = np.abs(x).astype(np.float64)
+    hi = np.clip(np.searchsorted(_FP8_POS, a, side="left"), 1, 126)       # first code with value >= a
+    lo = hi - 1
+    dlo = a - _FP8_POS[lo]
+    dhi = _FP8_POS[hi] - a
+    code = np.where(dlo < dhi, lo, np.where(dhi < dlo, hi, np.where(lo % 2 == 0, lo, hi)))
+    code = np.where(a >= 448.0, 126, code)                                 # satfinite, infinities too
+    code = np.where(a == 0.0, 0, code)
+    out = (code | np.where(np.signbit(x), 0x80, 0)).astype(np.uint8)
+    return np.where(np.isnan(x), np.uint8(0x7F), out).astype(np.uint8)
+
+
+def ag_matmul_ref_fp8(shards_bits: Sequence[np.ndarray], b_nk_bits: np.ndarray, return_f32: bool = False):
+    """C = cat(shards) @ B^T with e4m3fn operands, fp32 accumulate, e4m3fn result
+    (triton_all_gather_matmul.py:123 dtype switch, :176-188).  uint8 in, uint8 out."""
+    a = fp8_e4m3fn_to_f32(np.concatenate(list(shards_bits), axis=0))
+    b = fp8_e4m3fn_to_f32(b_nk_bits)
+    c = a @ b.T
+    bits = f32_to_fp8_e4m3fn(c)
+    return (bits, c) if return_f32 else bits
+
+
+def seeded_normal_fp8_bits(n: int, seed: int, std: float = 1.0) -> np.ndarray:
+    """N(0, std) from numpy's PCG64 seeded per tensor, rounded to e4m3fn."""
+    rng = np.random.default_rng(seed)
+    return f32_to_fp8_e4m3fn((rng.standard_normal(n) * std).astype(np.float32))
 
 
 # --------------------------------------------------------------------------

@@ -482,7 +482,210 @@ __device__ __forceinline__ void run_tile(const TileContext& cx, const TileRef& t
   }
 }
 
-template <int BM, int BN>
+// ---------------------------------------------------------------------------
+// The same tile with e4m3fn operands and result (the reference's FP8_OUTPUT switch,
+// triton_all_gather_matmul.py:115,123,188).  A row of a slab is still 128 bytes, now
+// 128 K values; everything that moves bytes (the ring, the loads, the swizzle, the
+// waits) is the bf16 tile's.  The MFMA is v_mfma_f32_32x32x64_f8f6f4: an operand
+// fragment is 32 rows x 64 K, lane l holds row l & 31 and the 32 bytes number l >> 5
+// of the two, i.e. chunks 4*kk + 2*(l >> 5) and the one after it in K step kk
+// (0 or 1).  Both operands use the same lane -> K mapping, which is all the sum
+// over K needs.  The 8 lanes x 2 that an LDS read serves together are 8 consecutive
+// rows at two chunks that differ by 2: the case row_swizzle is built for.
+// 256x256 tiles only: a wave holds 4 x 4 accumulators of 16 registers.
+typedef int i32x8 __attribute__((ext_vector_type(8)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+__device__ __forceinline__ uint32_t pack_fp8x4(float a, float b, float c, float d) {
+  // saturate to the largest finite e4m3fn value, keep NaN (cvt.rn.satfinite semantics)
+  auto sat = [](float x) { return x != x ? x : __builtin_fminf(__builtin_fmaxf(x, -448.0f), 448.0f); };
+  int w = __builtin_amdgcn_cvt_pk_fp8_f32(sat(a), sat(b), 0, false);
+  w = __builtin_amdgcn_cvt_pk_fp8_f32(sat(c), sat(d), w, true);
+  return (uint32_t)w;
+}
+
+template <typename Between>
+__device__ __forceinline__ void run_tile_fp8(const TileContext& cx, const TileRef& tile,
+                                             const uint8_t* a_rows, const uint8_t* b_rows,
+                                             bool preloaded, Between&& between) {
+  constexpr int BM = 256, BN = 256;
+  using T = GemmTile<BM, BN>;
+  const uint8_t* a_base = uniform_ptr(a_rows);
+  const uint8_t* b_base = uniform_ptr(b_rows);
+  constexpr int WM = T::WM, WN = T::WN, GA = T::GA, GB = T::GB;
+  constexpr int FM = WM / 32, FN = WN / 32;          // 32x32 fragments per wave tile
+  constexpr uint32_t kSlot = T::kSlotBytes;
+  const int lane = cx.lane, wave = cx.wave;
+  const int wm = wave >> 1, wn = wave & 1;
+  const uint32_t row_stride = cx.row_stride;
+  const int nk = cx.nk;
+  const uint32_t lds0 = cx.lds0;
+  uint64_t* tr = cx.tr;
+  uint8_t* c = cx.c;
+  struct { int N; } s = {cx.N};
+
+  int ln = lane;
+  asm volatile("" : "+v"(ln));
+  // fragment read addresses: [K step][first or second chunk of the lane's 32 bytes]
+  uint32_t a_fr[2][2], b_fr[2][2];
+#pragma unroll
+  for (int kk = 0; kk < 2; ++kk)
+#pragma unroll
+    for (int q = 0; q < 2; ++q) {
+      const int pos = (4 * kk + 2 * (ln >> 5) + q) ^ row_swizzle(ln & 15);
+      a_fr[kk][q] = lds0 + (uint32_t)((wm * WM + (ln & 31)) * kRowBytes + (pos << 4));
+      b_fr[kk][q] = lds0 + kSlot + (uint32_t)((wn * WN + (ln & 31)) * kRowBytes + (pos << 4));
+    }
+  uint32_t a_at = 0, b_at = kSlot;
+
+  const int u = (ln & 7) ^ row_swizzle(ln >> 3);
+  uint32_t a_off[GA];
+#pragma unroll
+  for (int j = 0; j < GA; ++j) {
+    const int q = wave * GA + j;
+    a_off[j] = (uint32_t)(q * 8 + (ln >> 3)) * row_stride + (uint32_t)((u ^ ((q & 1) << 2)) << 4);
+  }
+  const int b_last = s.N - 1 - tile.col0;
+  uint32_t b_off[GB];
+#pragma unroll
+  for (int j = 0; j < GB; ++j) {
+    const int q = wave * GB + j;
+    int r = q * 8 + (ln >> 3);
+    r = r < b_last ? r : b_last;
+    b_off[j] = (uint32_t)r * row_stride + (uint32_t)((u ^ ((q & 1) << 2)) << 4);
+  }
+
+  f32x16 acc[FN][FM];
+#pragma unroll
+  for (int ni = 0; ni < FN; ++ni)
+#pragma unroll
+    for (int mi = 0; mi < FM; ++mi)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[ni][mi][e] = 0.0f;
+
+  // one 128-bit read = half a fragment: reads 0 .. 2*FM-1 fill A, the rest B
+  auto read_half = [&](i32x8 (&af)[FM], i32x8 (&bf)[FN], int kk, int r) {
+    const bool is_a = r < 2 * FM;
+    const int f = (is_a ? r : r - 2 * FM) >> 1, q = r & 1;
+    const u32x4 v = lds_read_b128((is_a ? a_fr[kk][q] : b_fr[kk][q]) + f * (32 * kRowBytes));
+    i32x8& dst = is_a ? af[f] : bf[f];
+    dst[4 * q + 0] = (int)v.x;
+    dst[4 * q + 1] = (int)v.y;
+    dst[4 * q + 2] = (int)v.z;
+    dst[4 * q + 3] = (int)v.w;
+  };
+
+  if (!preloaded) issue_prologue<BM, BN>(cx, a_base, b_base, b_last);
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();
+
+  i32x8 af0[FM], bf0[FN], af1[FM], bf1[FN];
+  constexpr int kMfma = FM * FN, kReads = 2 * (FM + FN);
+#pragma unroll
+  for (int r = 0; r < kReads; ++r) read_half(af0, bf0, 0, r);
+
+  // the reads of the next K step go under the first three quarters of the MFMAs
+  constexpr int kReadSpan = kMfma * 3 / 4;
+  auto mfma = [&](const i32x8& bfrag, const i32x8& afrag, f32x16& d) {
+    // scale exponents 127 = 2^0 on both operands
+    d = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(bfrag, afrag, d, 0, 0, 0, 0x7F7F7F7F, 0, 0x7F7F7F7F);
+  };
+  auto first_step = [&](const uint8_t* ak, uint32_t la) {
+#pragma unroll
+    for (int ni = 0; ni < FN; ++ni) {
+#pragma unroll
+      for (int mi = 0; mi < FM; ++mi) {
+        const int slot = ni * FM + mi;
+        mfma(bf0[ni], af0[mi], acc[ni][mi]);
+#pragma unroll
+        for (int r = 0; r < kReads; ++r)
+          if (r * kReadSpan / kReads == slot) read_half(af1, bf1, 1, r);
+#pragma unroll
+        for (int g = 0; g < GA; ++g)
+          if (g * kMfma / GA == slot) load_group(ak, a_off[g], la + g * 1024);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+  };
+  auto second_step = [&](int kt) {
+    const int kb = kt + 2 < nk ? kt + 2 : nk - 1;
+    const uint8_t* bk = b_base + (int64_t)kb * kRowBytes;
+    const uint32_t lb = lds0 + a_at + wave * (GB * 1024);
+    const uint32_t a_to = a_at + 2 * kSlot < kRingSlots * kSlot ? a_at + 2 * kSlot : a_at + 2 * kSlot - kRingSlots * kSlot;
+    const uint32_t b_to = b_at + 2 * kSlot < kRingSlots * kSlot ? b_at + 2 * kSlot : b_at + 2 * kSlot - kRingSlots * kSlot;
+#pragma unroll
+    for (int kk = 0; kk < 2; ++kk)
+#pragma unroll
+      for (int q = 0; q < 2; ++q) {
+        a_fr[kk][q] += a_to - a_at;
+        b_fr[kk][q] += b_to - b_at;
+      }
+    a_at = a_to;
+    b_at = b_to;
+#pragma unroll
+    for (int ni = 0; ni < FN; ++ni) {
+#pragma unroll
+      for (int mi = 0; mi < FM; ++mi) {
+        const int slot = ni * FM + mi;
+        mfma(bf1[ni], af1[mi], acc[ni][mi]);
+#pragma unroll
+        for (int g = 0; g < GB; ++g)
+          if (g * (kMfma / 2) / GB == slot) load_group(bk, b_off[g], lb + g * 1024);
+#pragma unroll
+        for (int r = 0; r < kReads; ++r)
+          if (r * kReadSpan / kReads == slot) read_half(af0, bf0, 0, r);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+  };
+  for (int kt = 0; kt < nk; ++kt) {
+    const int ka = kt + 2 < nk ? kt + 2 : nk - 1;
+    const uint8_t* ak = a_base + (int64_t)ka * kRowBytes;
+    const uint32_t a_dst = a_at >= kSlot ? a_at - kSlot : a_at + (kRingSlots - 1) * kSlot;
+    first_step(ak, lds0 + a_dst + wave * (GA * 1024));
+    asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+    __syncthreads();
+    second_step(kt);
+  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();
+  if (tr != nullptr) tr[2] = wall_clock64();
+  between();
+
+  // Epilogue.  D[n][m]: a lane holds row m = lane & 31 of a 32x32 fragment and, per
+  // group g of 4 registers, the 4 consecutive columns g*8 + (lane >> 5)*4 .. +3: one
+  // 32-bit word of e4m3fn.  32 rows at a time go through the wave's quarter of ring
+  // slot 4 (128 bytes per row, chunk c of row r at position c ^ ((r >> 1) & 7)) and
+  // leave as whole rows, 16 bytes per lane.
+  const uint32_t turn = lds0 + (kRingSlots - 1) * kSlot + wave * (32 * WN);
+  const int half = ln >> 5, wr_row = ln & 31;
+  const int rd_row = ln >> 3, rd_chunk = ln & 7;
+#pragma unroll
+  for (int mi = 0; mi < FM; ++mi) {
+#pragma unroll
+    for (int ni = 0; ni < FN; ++ni) {
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const f32x16& d = acc[ni][mi];
+        const uint32_t w = pack_fp8x4(d[g * 4 + 0], d[g * 4 + 1], d[g * 4 + 2], d[g * 4 + 3]);
+        const int chunk = ni * 2 + (g >> 1);
+        const uint32_t addr = turn + wr_row * WN + (((chunk ^ (wr_row >> 1)) & 7) << 4) + ((g & 1) * 2 + half) * 4;
+        *reinterpret_cast<__attribute__((address_space(3))) uint32_t*>((uintptr_t)addr) = w;
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int r = i * 8 + rd_row;
+      const u32x4 v = lds_read_b128(turn + r * WN + (((rd_chunk ^ (r >> 1)) & 7) << 4));
+      const int m = tile.row0 + wm * WM + mi * 32 + r;
+      const int n = tile.col0 + wn * WN + rd_chunk * 16;
+      if (n < s.N) *reinterpret_cast<u32x4*>(c + (int64_t)m * s.N + n) = v;
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  }
+}
+
+template <int BM, int BN, bool FP8 = false>
 __global__ __launch_bounds__(kGemmThreads, 1) void ag_matmul_kernel(
     const uint8_t* __restrict__ a_shard, const uint8_t* __restrict__ a_out,
     const uint8_t* __restrict__ b_nk, uint8_t* __restrict__ c, const uint32_t* __restrict__ progress,
@@ -492,8 +695,8 @@ __global__ __launch_bounds__(kGemmThreads, 1) void ag_matmul_kernel(
   TileContext cx;
   cx.lane = threadIdx.x & 63;
   cx.wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  cx.row_stride = (uint32_t)s.K * 2u;
-  cx.nk = s.K / kBK;
+  cx.row_stride = (uint32_t)s.K * (FP8 ? 1u : 2u);        // K values per row, 1 or 2 bytes each
+  cx.nk = (int)(cx.row_stride / kRowBytes);
   cx.lds0 = lds_offset_of(lds);
   cx.N = s.N;
   cx.c = c;
@@ -542,7 +745,9 @@ __global__ __launch_bounds__(kGemmThreads, 1) void ag_matmul_kernel(
         issue_prologue<BM, BN>(cx, a_next, b_next, b_last);
       }
     };
-    if constexpr (BN == 256) {
+    if constexpr (FP8) {
+      run_tile_fp8(cx, tile, a_base, b_base, preloaded, between);
+    } else if constexpr (BN == 256) {
       if (tile.cols != BN) run_tile<BM, BN / 2>(cx, tile, a_base, b_base, preloaded, between);
       else run_tile<BM, BN>(cx, tile, a_base, b_base, preloaded, between);
     } else {
@@ -632,14 +837,15 @@ struct FusedEstimate {
 constexpr int kMaxProducerWgs = 128;
 // every chunk ends with a release, a workgroup barrier and an arrival count
 static double copy_us(double bytes, int chunks, int wgs) { return bytes / (wgs * 33.0e3) + 6.0 * chunks; }
-static FusedEstimate estimate_fused(const GemmSchedule& s, int cus, int grid) {
-  const double tile_us = 2.0 * s.BM * s.BN * s.K / 6.0e6 + 8.0;
+static FusedEstimate estimate_fused(const GemmSchedule& s, int cus, int grid, int elem_bytes = 2) {
+  // (e4m3fn: twice the MFMA rate per workgroup, half the bytes to copy)
+  const double tile_us = 2.0 * s.BM * s.BN * s.K / (elem_bytes == 1 ? 12.0e6 : 6.0e6) + 8.0;
   const int tiles = (s.M / s.BM) * ceil_div(s.N, s.BN);
   const int tiles_per_cb = (s.comm_block_m / s.BM) * ceil_div(s.N, s.BN);
   FusedEstimate e;
   e.producer_wgs = cus - grid < kMaxProducerWgs ? cus - grid : kMaxProducerWgs;
   if (e.producer_wgs < 1) e.producer_wgs = 1;
-  const double remote_bytes = 2.0 * 2.0 * s.M * s.K * (s.world_size - 1) / s.world_size;
+  const double remote_bytes = 2.0 * elem_bytes * s.M * s.K * (s.world_size - 1) / s.world_size;
   e.gemm_us = ceil_div(tiles, grid) * tile_us;
   e.copy_us = copy_us(remote_bytes, s.M / s.comm_block_m, e.producer_wgs);
   const double tail_us = e.copy_us + ceil_div(tiles_per_cb, grid) * tile_us;
@@ -652,12 +858,13 @@ static FusedEstimate estimate_fused(const GemmSchedule& s, int cus, int grid) {
 static int g_force_head = -1, g_force_tail = -1;
 
 static GemmSchedule make_schedule(int M, int N, int K, int rank, int world_size, int comm_block_m,
-                                  int cus, bool gated) {
+                                  int cus, bool gated, int elem_bytes = 2) {
   GemmSchedule s;
   s.M = M; s.N = N; s.K = K;
   s.rank = rank; s.world_size = world_size; s.comm_block_m = comm_block_m;
   s.head = s.tail = 0;
-  pick_tile(M, N, comm_block_m, s.BM, s.BN, cus);
+  if (elem_bytes == 1) s.BM = s.BN = 256;        // the e4m3fn tile exists in one shape
+  else pick_tile(M, N, comm_block_m, s.BM, s.BN, cus);
   const int tn = (N + s.BN - 1) / s.BN;
   const int total = (M / s.BM) * tn;
   int max_grid = ((gated ? cus - kReservedCus : cus) / 8) * 8;
@@ -671,10 +878,10 @@ static GemmSchedule make_schedule(int M, int N, int K, int rank, int world_size,
     // the grid (a multiple of 8) for which the later of the two - the GEMM's passes,
     // or the last chunk's arrival plus the tiles that wait for it - comes earliest;
     // among equals the smallest grid.
-    const FusedEstimate base = estimate_fused(s, cus, s.grid);
+    const FusedEstimate base = estimate_fused(s, cus, s.grid, elem_bytes);
     double best = base.total_us;
     for (int g = 8; g <= max_grid; g += 8) {
-      const double t = estimate_fused(s, cus, g).total_us;
+      const double t = estimate_fused(s, cus, g, elem_bytes).total_us;
       if (t < best * 0.97) {             // only for a clear gain: the model is coarse
         best = t;
         s.grid = g;
@@ -686,7 +893,7 @@ static GemmSchedule make_schedule(int M, int N, int K, int rank, int world_size,
   // by their loads, and with a producer that delivers a chunk in less than a pass it
   // is cheaper to let the workgroups of the first remote comm block wait for it.
   const int n_comm = M / comm_block_m;
-  if (gated && s.BN == 256 && g_force_head >= 0 && g_force_tail >= 0 &&
+  if (gated && elem_bytes == 2 && s.BN == 256 && g_force_head >= 0 && g_force_tail >= 0 &&
       g_force_head + g_force_tail <= n_comm) {
     s.head = g_force_head;
     s.tail = g_force_tail;
@@ -745,6 +952,52 @@ int smr_ag_matmul(const void* a_shard_dev, const void* a_out_dev, const void* b_
     hipLaunchKernelGGL((ag_matmul_kernel<128, 128>), dim3(s.grid), dim3(kGemmThreads), 0, st, a0, a1, b,
                        c, progress_dev, s, lim, status, tb);
   return check_hip(hipGetLastError(), "smr_ag_matmul launch");
+}
+
+static int validate_fp8(int M, int N, int K, int rank, int world_size, int comm_block_m, const char** why) {
+  if (int rc = smr::validate(M, N, K, rank, world_size, comm_block_m, why)) return rc;
+  if (K % 128 != 0)
+    *why = "smr_ag_matmul_fp8: K must be a multiple of 128";
+  else if (N % 16 != 0)
+    *why = "smr_ag_matmul_fp8: N must be a multiple of 16";
+  else if (comm_block_m % 256 != 0)
+    *why = "smr_ag_matmul_fp8: rows per progress flag must be a multiple of 256";
+  return *why ? SMR_E_UNSUPPORTED : 0;
+}
+
+int smr_ag_matmul_fp8(const void* a_shard_dev, const void* a_out_dev, const void* b_nk_dev, void* c_dev,
+                      const uint32_t* progress_dev, int M, int N, int K, int rank, int world_size,
+                      int comm_block_m, uint32_t* status, void* stream) {
+  using namespace smr;
+  const char* why;
+  if (int rc = validate_fp8(M, N, K, rank, world_size, comm_block_m, &why)) return fail(rc, why);
+  if (a_shard_dev == nullptr || a_out_dev == nullptr || b_nk_dev == nullptr || c_dev == nullptr)
+    return fail(SMR_E_INVALID, "smr_ag_matmul_fp8: null pointer");
+  if ((reinterpret_cast<uintptr_t>(a_shard_dev) | reinterpret_cast<uintptr_t>(a_out_dev) |
+       reinterpret_cast<uintptr_t>(b_nk_dev) | reinterpret_cast<uintptr_t>(c_dev)) & 15u)
+    return fail(SMR_E_INVALID, "smr_ag_matmul_fp8: operands must be 16-byte aligned");
+  const GemmSchedule s = make_schedule(M, N, K, rank, world_size, comm_block_m, cu_count(),
+                                       progress_dev != nullptr, 1);
+  hipLaunchKernelGGL((ag_matmul_kernel<256, 256, true>), dim3(s.grid), dim3(kGemmThreads), 0,
+                     reinterpret_cast<hipStream_t>(stream), reinterpret_cast<const uint8_t*>(a_shard_dev),
+                     reinterpret_cast<const uint8_t*>(a_out_dev), reinterpret_cast<const uint8_t*>(b_nk_dev),
+                     reinterpret_cast<uint8_t*>(c_dev), progress_dev, s, spin_limit_ticks(), status,
+                     trace_buffer(kTraceProducerWords + kTraceGemmWords));
+  return check_hip(hipGetLastError(), "smr_ag_matmul_fp8 launch");
+}
+
+int smr_ag_matmul_plan_fp8(int M, int N, int K, int world_size, int comm_block_m, int32_t* out4) {
+  using namespace smr;
+  const char* why;
+  if (int rc = validate_fp8(M, N, K, 0, world_size, comm_block_m, &why)) return fail(rc, why);
+  if (out4 == nullptr) return fail(SMR_E_INVALID, "smr_ag_matmul_plan_fp8: out4 is NULL");
+  const int cus = cu_count();
+  const GemmSchedule s = make_schedule(M, N, K, 0, world_size, comm_block_m, cus, true, 1);
+  out4[0] = s.grid;
+  out4[1] = estimate_fused(s, cus, s.grid, 1).producer_wgs;
+  out4[2] = 0;
+  out4[3] = 0;
+  return 0;
 }
 
 int smr_set_ag_matmul_halves(int head, int tail) {

@@ -68,7 +68,7 @@ def all_gather_matmul_tma_persistent(a_shard: torch.Tensor, b: torch.Tensor, a_o
                                      c_out: torch.Tensor, configs: Optional[dict] = None,
                                      mm_only: bool = False, *, splits_per_rank: int = 1) -> torch.Tensor:
     """``c_out = cat(all ranks' a_shard) @ b.T`` with ``b`` of shape [N, K]
-    (K-contiguous).  ``mm_only`` skips the gather and the flags and multiplies
+    (K-contiguous), bf16 or - all four tensors - float8_e4m3fn.  ``mm_only`` skips the gather and the flags and multiplies
     what ``a_shard`` (rank 0's rows) and ``a_out`` already hold: the ungated
     comparator.  ``configs`` is accepted for compatibility; the tile shape is the
     library's choice."""
@@ -82,7 +82,11 @@ def all_gather_matmul_tma_persistent(a_shard: torch.Tensor, b: torch.Tensor, a_o
         rank = symm_mem.rank
         world_size = symm_mem.world_size
 
-    assert a_shard.dtype == torch.bfloat16 and b.dtype == torch.bfloat16, "Only bfloat16 is supported for now."
+    # bf16, or e4m3fn throughout as the reference's FP8_OUTPUT switch (:115,123,311)
+    fp8 = a_shard.dtype == torch.float8_e4m3fn
+    assert a_shard.dtype in (torch.bfloat16, torch.float8_e4m3fn), "Only bfloat16 and float8_e4m3fn are supported."
+    assert b.dtype == a_shard.dtype and a_out.dtype == a_shard.dtype and c_out.dtype == a_shard.dtype, \
+        "a_shard, b, a_out and c_out must have one dtype"
     M = a_shard.shape[0] * world_size
     N = b.shape[0]
     K = a_shard.shape[1]
@@ -117,16 +121,18 @@ def all_gather_matmul_tma_persistent(a_shard: torch.Tensor, b: torch.Tensor, a_o
         assert a_out.dtype == a_shard.dtype and a_out.is_contiguous()
         # the producer takes (some of) the compute units the GEMM's grid leaves free
         plan = (ctypes.c_int32 * 4)()
-        _lib.check(lib.smr_ag_matmul_plan(M, N, K, world_size, COMM_BLOCK_SIZE_M, plan), "all_gather_matmul")
+        planner = lib.smr_ag_matmul_plan_fp8 if fp8 else lib.smr_ag_matmul_plan
+        _lib.check(planner(M, N, K, world_size, COMM_BLOCK_SIZE_M, plan), "all_gather_matmul")
         producer_wgs = plan[1] if MAX_PRODUCER_WORKGROUPS is None else min(MAX_PRODUCER_WORKGROUPS, plan[1])
         pacing = (plan[2], plan[3]) if PRODUCER_PACING is None else PRODUCER_PACING
 
     # The GEMM goes first: its first tiles are local rows and need no flag, so the
     # producer's launch latency is hidden behind them instead of delaying the GEMM.
     # (The backend stream waits for what preceded the GEMM, not for the GEMM.)
-    rc = lib.smr_ag_matmul(a_shard.data_ptr(), a_out.data_ptr(), b.data_ptr(), c_out.data_ptr(),
-                           progress_ptr, M, N, K, rank, world_size, COMM_BLOCK_SIZE_M, status_ptr,
-                           current.cuda_stream)
+    gemm = lib.smr_ag_matmul_fp8 if fp8 else lib.smr_ag_matmul
+    rc = gemm(a_shard.data_ptr(), a_out.data_ptr(), b.data_ptr(), c_out.data_ptr(),
+              progress_ptr, M, N, K, rank, world_size, COMM_BLOCK_SIZE_M, status_ptr,
+              current.cuda_stream)
     _lib.check(rc, "all_gather_matmul")
     if not mm_only:
         _lib.check(lib.smr_set_gather_pacing(int(pacing[0]), int(pacing[1])), "all_gather_matmul")

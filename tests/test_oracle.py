@@ -380,3 +380,52 @@ def test_signal_round_ref_bruteforce():
                     s = (s + ((int(w) + rnd) & 0xFFFFFFFF)) & 0xFFFFFFFF
             want[b] = s
         assert np.array_equal(O.signal_round_ref(src, rnd), want)
+
+
+# ---------------------------------------------------------------- fp8 (e4m3fn)
+def test_fp8_decode_exhaustive_vs_torch():
+    bits = np.arange(256, dtype=np.uint8)
+    mine = O.fp8_e4m3fn_to_f32(bits)
+    ref = torch.from_numpy(bits.copy()).view(torch.float8_e4m3fn).float().numpy()
+    nan = np.isnan(ref)
+    assert np.array_equal(np.isnan(mine), nan) and set(bits[nan]) == {0x7F, 0xFF}
+    assert np.array_equal(mine[~nan].view(np.uint32), ref[~nan].view(np.uint32))
+
+
+def test_fp8_encode_vs_torch_ties_and_saturation():
+    pos = O.fp8_e4m3fn_to_f32(np.arange(127, dtype=np.uint8)).astype(np.float64)
+    mids = (pos[:-1] + pos[1:]) / 2
+    rng = np.random.default_rng(9)
+    x = np.concatenate([pos, mids, np.nextafter(mids.astype(np.float32), 0), np.nextafter(mids.astype(np.float32), 1e9),
+                        rng.standard_normal(200000) * 3, rng.uniform(-448, 448, 200000),
+                        rng.uniform(-2 ** -6, 2 ** -6, 100000)]).astype(np.float32)
+    x = np.concatenate([x, -x])
+    mine = O.f32_to_fp8_e4m3fn(x)
+    ref = torch.from_numpy(x).to(torch.float8_e4m3fn).view(torch.uint8).numpy()
+    assert np.array_equal(mine, ref)                                    # |x| <= 448: one answer
+    # exact values round-trip; ties go to the even code
+    assert np.array_equal(O.f32_to_fp8_e4m3fn(pos.astype(np.float32)), np.arange(127, dtype=np.uint8))
+    assert np.all(O.f32_to_fp8_e4m3fn(mids.astype(np.float32)) % 2 == 0)
+    # beyond the largest finite value: saturate (cvt.rn.satfinite), NaN stays NaN
+    big = np.array([449, 464, 465, 480, 1e6, np.inf, -500, -np.inf, np.nan], dtype=np.float32)
+    assert O.f32_to_fp8_e4m3fn(big).tolist() == [126, 126, 126, 126, 126, 126, 254, 254, 0x7F]
+
+
+def test_fp8_matmul_vs_torch_cpu():
+    rng = np.random.default_rng(2)
+    a = rng.integers(0, 256, (48, 128)).astype(np.uint8)
+    b = rng.integers(0, 256, (40, 128)).astype(np.uint8)
+    a[(a & 0x7F) == 0x7F] = 0x38                                         # no NaN operands
+    b[(b & 0x7F) == 0x7F] = 0x38
+    a = np.where((a & 0x78) > 0x50, a & 0xCF, a)                         # keep sums finite and below 448 often
+    got, c = O.ag_matmul_ref_fp8([a[:24], a[24:]], b, return_f32=True)
+    ta = torch.from_numpy(a.copy()).view(torch.float8_e4m3fn).float()
+    tb = torch.from_numpy(b.copy()).view(torch.float8_e4m3fn).float()
+    tc = ta @ tb.T
+    assert np.allclose(c, tc.numpy(), rtol=1e-6, atol=1e-6)
+    inr = np.abs(c) <= 448
+    want = tc.to(torch.float8_e4m3fn).view(torch.uint8).numpy()
+    # identical except where the two fp32 sums straddle a rounding boundary
+    same = got[inr] == want[inr]
+    assert same.mean() > 0.999
+    assert np.all(got[~inr] & 0x7F == 126)
