@@ -29,6 +29,7 @@ HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
 # (profiles/one_shot_all_reduce_64MiB_bf16_traffic.md); keyed by MiB per buffer.
 MEASURED_REDUCE_TRAFFIC_BYTES = {64: 604405370}
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
+MFMA_FP8_PEAK_TFLOPS = 5000.0   # MI355X dense fp8, published
 # Fabric bytes per launch of the ungated GEMM at M=16384 N=3584 K=8192 (FETCH_SIZE scaled
 # as above plus WRITE_SIZE; profiles/ag_matmul_M16384_N3584_K8192_counters.md).  A counter
 # run cannot hold the gated launch (it serialises kernels); the gated GEMM reads and writes
@@ -207,6 +208,48 @@ def bench_ag_matmul(dev, gated=True):
                           "unit": "TFLOP/s", "frac": flops / us_gated / 1e6 / MFMA_BF16_PEAK_TFLOPS,
                           "traffic": MEASURED_GEMM_TRAFFIC_BYTES},
                 torch_matmul_us=us_lib, torch_matmul_tflops=flops / us_lib / 1e6)
+
+
+def bench_ag_matmul_fp8(dev):
+    """The same problem with e4m3fn operands and result (the reference's FP8_OUTPUT switch)."""
+    import torch
+    from symm_mem_recipes import EmulatedSymmetricMemory as SM, all_gather_matmul_tma_persistent
+    M, N, K = 16384, 3584, 8192
+    f8 = torch.float8_e4m3fn
+    a_shard = SM.empty_strided_p2p((M // WS, K), (K, 1), f8, dev, world_size=WS, rank=0)
+    h = SM.rendezvous(a_shard)
+    g = torch.Generator(device=dev)
+    for r in range(WS):
+        g.manual_seed(r)
+        h.get_buffer(r, (M // WS, K), f8).copy_(
+            torch.empty(M // WS, K, device=dev).normal_(0, 0.05, generator=g).to(f8))
+    g.manual_seed(100)
+    b = torch.empty(N, K, device=dev).normal_(0, 0.05, generator=g).to(f8)
+    a_out = torch.cat([h.get_buffer(r, (M // WS, K), f8) for r in range(WS)]).contiguous()
+    c = torch.empty(M, N, dtype=torch.uint8, device=dev).view(f8)
+    flush = torch.empty(1 << 28, dtype=torch.int32, device=dev)
+    flops = 2.0 * M * N * K
+    us_ungated = _time_events(lambda: all_gather_matmul_tma_persistent(a_shard, b, a_out, c, None, mm_only=True),
+                              25, 20, pre=flush.zero_)
+    us_gated = _time_events(lambda: all_gather_matmul_tma_persistent(a_shard, b, a_out, c, None),
+                            25, 20, pre=flush.zero_)
+    h.check_status()
+    res = dict(workload="all-gather matmul M=16384 N=3584 K=8192 e4m3fn in and out, 8 shards of [2048, 8192], rank 0",
+               flops=flops, us_gated=us_gated, us_ungated=us_ungated,
+               tflops_gated=flops / us_gated / 1e6, tflops_ungated=flops / us_ungated / 1e6,
+               gating_overhead=us_gated / us_ungated - 1.0,
+               roofline={"bound": "mfma", "achieved": flops / us_gated / 1e6, "peak": MFMA_FP8_PEAK_TFLOPS,
+                         "unit": "TFLOP/s", "frac": flops / us_gated / 1e6 / MFMA_FP8_PEAK_TFLOPS,
+                         "traffic": None})
+    try:                                            # the library's fp8 GEMM of the same operands (bf16 result)
+        one = torch.ones((), device=dev)
+        us_lib = _time_events(lambda: torch._scaled_mm(a_out, b.T, scale_a=one, scale_b=one,
+                                                       out_dtype=torch.bfloat16), 25, 20, pre=flush.zero_)
+        res.update(torch_scaled_mm_us=us_lib, torch_scaled_mm_tflops=flops / us_lib / 1e6)
+    except Exception as exc:                        # not every torch build has it for this dtype
+        res["torch_scaled_mm_error"] = repr(exc)[:200]
+    SM.release()
+    return res
 
 
 def bench_gemv(dev):
@@ -396,6 +439,7 @@ def main():
             [bench_reduce_rotating(k, dev, "bf16", write_all=True) for k in (1024, 8192, 16384)] +
             [bench_reduce_rotating(k, dev, "bf16", accumulate="bf16") for k in (8192,)])
         extra["all_gather_matmul"] = bench_ag_matmul(dev)
+        extra["all_gather_matmul_fp8"] = bench_ag_matmul_fp8(dev)
         extra["gemv_allreduce"] = bench_gemv(dev)
         extra["barrier"] = bench_barrier(dev)
     line["extra"] = extra

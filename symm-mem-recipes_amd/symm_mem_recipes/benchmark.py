@@ -18,7 +18,7 @@ import statistics
 
 import torch
 
-from .all_gather_matmul import all_gather_matmul, all_gather_matmul_tma_persistent
+from .all_gather_matmul import all_gather_matmul_tma_persistent
 from .symm_mem import EmulatedSymmetricMemory
 
 #: (name, N, K) of the README's three model shapes; M is swept over README_MS
@@ -44,29 +44,43 @@ def _median_us(fn, flush, warmup, iters):
 
 
 def benchmark_all_gather_matmul(M: int, N: int, K: int, world_size: int = 8, rank: int = 0,
-                                warmup: int = 20, iters: int = 25, device=None) -> dict:
+                                warmup: int = 20, iters: int = 25, device=None,
+                                dtype: torch.dtype = torch.bfloat16) -> dict:
     """Median microseconds of the four variants for one problem; inputs N(0, 0.02)
-    seeded as the reference seeds its harness (42 + rank)."""
+    (N(0, 0.05) for float8_e4m3fn) seeded as the reference seeds its harness (42 + rank)."""
     device = torch.device("cuda:0") if device is None else device
-    a_shard = EmulatedSymmetricMemory.empty_strided_p2p((M // world_size, K), (K, 1), torch.bfloat16,
+    fp8 = dtype == torch.float8_e4m3fn
+    std = 0.05 if fp8 else 0.02
+    a_shard = EmulatedSymmetricMemory.empty_strided_p2p((M // world_size, K), (K, 1), dtype,
                                                         device, world_size=world_size, rank=rank)
     h = EmulatedSymmetricMemory.rendezvous(a_shard)
     g = torch.Generator(device=device)
     for r in range(world_size):
         g.manual_seed(42 + r)
-        h.get_buffer(r, (M // world_size, K), torch.bfloat16).normal_(0, 0.02, generator=g)
+        h.get_buffer(r, (M // world_size, K), dtype).copy_(
+            torch.empty(M // world_size, K, device=device).normal_(0, std, generator=g).to(dtype))
     g.manual_seed(41)
-    b = torch.empty(N, K, dtype=torch.bfloat16, device=device).normal_(0, 0.02, generator=g)
-    a_out = torch.cat([h.get_buffer(r, (M // world_size, K), torch.bfloat16) for r in range(world_size)])
-    c = torch.empty(M, N, dtype=torch.bfloat16, device=device)
+    b = torch.empty(N, K, device=device).normal_(0, std, generator=g).to(dtype)
+    a_out = torch.cat([h.get_buffer(r, (M // world_size, K), dtype) for r in range(world_size)])
+    c = torch.empty(M, N, dtype=torch.uint8 if fp8 else dtype, device=device).view(dtype)
     flush = torch.empty(1 << 28, dtype=torch.int32, device=device)          # 1 GiB
+    if fp8:
+        one = torch.ones((), device=device)
+
+        def library_mm(a, b_kn):                     # the library's fp8 GEMM gives a bf16 result
+            return torch._scaled_mm(a, b_kn, scale_a=one, scale_b=one, out_dtype=torch.bfloat16)
+    else:
+        def library_mm(a, b_kn):
+            return torch.matmul(a, b_kn)
     res = {
         "M": M, "N": N, "K": K,
-        "library_mm_only_us": _median_us(lambda: torch.matmul(a_out, b.T, out=c), flush, warmup, iters),
+        "library_mm_only_us": _median_us(lambda: library_mm(a_out, b.T), flush, warmup, iters),
         "hip_mm_only_us": _median_us(
             lambda: all_gather_matmul_tma_persistent(a_shard, b, a_out, c, None, mm_only=True),
             flush, warmup, iters),
-        "library_gather_mm_us": _median_us(lambda: all_gather_matmul(a_shard, b.T), flush, warmup, iters),
+        "library_gather_mm_us": _median_us(
+            lambda: library_mm(torch.cat([h.get_buffer(r, a_shard.shape, dtype) for r in range(world_size)]), b.T),
+            flush, warmup, iters),
         "hip_fused_us": _median_us(lambda: all_gather_matmul_tma_persistent(a_shard, b, a_out, c, None),
                                    flush, warmup, iters),
     }
@@ -90,18 +104,20 @@ def main(argv=None):
     ap.add_argument("--world-size", type=int, default=8)
     ap.add_argument("--rank", type=int, default=0)
     ap.add_argument("--readme", action="store_true", help="all nine problems of the reference's README")
+    ap.add_argument("--fp8", action="store_true", help="float8_e4m3fn operands and result instead of bfloat16")
     args = ap.parse_args(argv)
+    dtype = torch.float8_e4m3fn if args.fp8 else torch.bfloat16
     head = ("| Problem Size (M) | library mm only (us) | hip mm only (us) | library gather + mm (us) | "
             "hip fused (us) | fused TFLOP/s |\n|---|---|---|---|---|---|")
     if args.readme:
         for name, n, k in README_SHAPES:
             print(f"#### {name} (N={n}, K={k})\n{head}", flush=True)
             for m in README_MS:
-                print(_row(benchmark_all_gather_matmul(m, n, k, args.world_size, args.rank)), flush=True)
+                print(_row(benchmark_all_gather_matmul(m, n, k, args.world_size, args.rank, dtype=dtype)), flush=True)
             print(flush=True)
     else:
         print(head)
-        print(_row(benchmark_all_gather_matmul(args.M, args.N, args.K, args.world_size, args.rank)))
+        print(_row(benchmark_all_gather_matmul(args.M, args.N, args.K, args.world_size, args.rank, dtype=dtype)))
 
 
 if __name__ == "__main__":
