@@ -126,6 +126,27 @@ def test_fused_parity_half_tile_phases(cuda, lib, head, tail):
     _check(_t_bits(c_out), O.ag_matmul_ref(shards, b_bits))
 
 
+def test_fused_back_to_back_calls_are_identical(cuda):
+    """Twenty fused launches in a row without a host synchronisation in between, the
+    gathered operand wiped before each: flags, arrival counters and the two streams
+    must hand over cleanly from one call to the next, and the result is deterministic."""
+    from symm_mem_recipes import all_gather_matmul_tma_persistent
+    M, N, K, ws, rank = 8192, 1024, 1024, 8, 6
+    a_shard, h, shards, b, b_bits, a_out, c_out = _setup(M, N, K, ws, rank, cuda)
+    outs = []
+    for i in range(20):
+        a_out.zero_()
+        c = torch.empty_like(c_out)
+        all_gather_matmul_tma_persistent(a_shard, b, a_out, c, None)
+        outs.append(c)
+    torch.cuda.synchronize()
+    h.check_status()
+    _check(_t_bits(outs[0]), O.ag_matmul_ref(shards, b_bits))
+    assert np.array_equal(_t_bits(a_out), np.concatenate(shards))
+    for c in outs[1:]:
+        assert torch.equal(c.view(torch.int16), outs[0].view(torch.int16))
+
+
 def test_mm_only_is_ungated(cuda, monkeypatch):
     """mm_only multiplies what the buffers already hold, as rank 0, with no flags
     (triton_all_gather_matmul.py:222-224,246-247)."""
