@@ -202,15 +202,18 @@ int smr_ag_matmul_fp8(const void* a_shard_dev, const void* a_out_dev, const void
                       const uint32_t* progress_dev, int M, int N, int K, int rank, int world_size,
                       int comm_block_m, uint32_t* status, void* stream);
 /* smr_ag_matmul_plan for the e4m3fn GEMM. */
-int smr_ag_matmul_plan_fp8(int M, int N, int K, int world_size, int comm_block_m, int32_t* out4);
+int smr_ag_matmul_plan_fp8(int M, int N, int K, int world_size, int comm_block_m, int32_t* out5);
 
-/* Host-only: how a fused launch of this shape splits the GPU.  out4 = {GEMM grid (what
- * smr_ag_matmul will launch when gated), producer workgroups, fast_chunks,
- * slow_workgroups} - the last two are the arguments of smr_set_gather_pacing ({0, 0}: the
- * copy runs flat out).  Replaces
- * the fixed NUM_SMS grid of triton_all_gather_matmul.py:287-294: there the copy engines
- * cost no SMs. */
-int smr_ag_matmul_plan(int M, int N, int K, int world_size, int comm_block_m, int32_t* out4);
+/* Host-only: how a fused launch of this shape splits the GPU.  out5 = {GEMM grid,
+ * producer workgroups, fast_chunks, slow_workgroups, sequential}.  fast_chunks and
+ * slow_workgroups are the arguments of smr_set_gather_pacing ({0, 0}: the copy runs flat
+ * out).  sequential = 1: the problem is too small to hide the copy behind the GEMM; copy
+ * with the whole GPU first (producer workgroups = all compute units), then call
+ * smr_ag_matmul with progress = NULL in stream order behind it.  sequential = 0: launch
+ * smr_ag_matmul gated (it uses the grid given here) and the producer beside it.
+ * Replaces the fixed NUM_SMS grid of triton_all_gather_matmul.py:287-294: there the copy
+ * engines cost no SMs. */
+int smr_ag_matmul_plan(int M, int N, int K, int world_size, int comm_block_m, int32_t* out5);
 
 /* Tuning knob of the gated schedule: the first `head` and the last `tail` comm blocks
  * of the ring order are computed in tiles of half the width.  Both -1 (the default)

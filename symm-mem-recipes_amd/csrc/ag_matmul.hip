@@ -828,15 +828,15 @@ static int total_steps(const GemmSchedule& s) {
 
 // Coarse model of a fused launch, for splitting the compute units between the GEMM
 // and the producer.  Rates measured on MI355X with both kernels running: a GEMM
-// workgroup sustains about 6 TFLOP/s, a producer workgroup moves about 33 GB/s
-// (bytes read plus bytes written).
+// workgroup sustains about 6 TFLOP/s, a producer workgroup moves about 35 GB/s
+// (bytes read plus bytes written) and spends about 2.5 us per chunk on publishing it.
 struct FusedEstimate {
   double gemm_us, copy_us, total_us;
   int producer_wgs;
 };
 constexpr int kMaxProducerWgs = 128;
-// every chunk ends with a release, a workgroup barrier and an arrival count
-static double copy_us(double bytes, int chunks, int wgs) { return bytes / (wgs * 33.0e3) + 6.0 * chunks; }
+// every chunk ends with a wait for the stores, a workgroup barrier and an arrival count
+static double copy_us(double bytes, int chunks, int wgs) { return bytes / (wgs * 35.0e3) + 2.5 * chunks; }
 static FusedEstimate estimate_fused(const GemmSchedule& s, int cus, int grid, int elem_bytes = 2) {
   // (e4m3fn: twice the MFMA rate per workgroup, half the bytes to copy)
   const double tile_us = 2.0 * s.BM * s.BN * s.K / (elem_bytes == 1 ? 12.0e6 : 6.0e6) + 8.0;
@@ -954,6 +954,8 @@ int smr_ag_matmul(const void* a_shard_dev, const void* a_out_dev, const void* b_
   return check_hip(hipGetLastError(), "smr_ag_matmul launch");
 }
 
+static void fill_plan(int M, int N, int K, int world_size, int comm_block_m, int elem_bytes, int32_t* out5);
+
 static int validate_fp8(int M, int N, int K, int rank, int world_size, int comm_block_m, const char** why) {
   if (int rc = smr::validate(M, N, K, rank, world_size, comm_block_m, why)) return rc;
   if (K % 128 != 0)
@@ -986,17 +988,12 @@ int smr_ag_matmul_fp8(const void* a_shard_dev, const void* a_out_dev, const void
   return check_hip(hipGetLastError(), "smr_ag_matmul_fp8 launch");
 }
 
-int smr_ag_matmul_plan_fp8(int M, int N, int K, int world_size, int comm_block_m, int32_t* out4) {
+int smr_ag_matmul_plan_fp8(int M, int N, int K, int world_size, int comm_block_m, int32_t* out5) {
   using namespace smr;
   const char* why;
   if (int rc = validate_fp8(M, N, K, 0, world_size, comm_block_m, &why)) return fail(rc, why);
-  if (out4 == nullptr) return fail(SMR_E_INVALID, "smr_ag_matmul_plan_fp8: out4 is NULL");
-  const int cus = cu_count();
-  const GemmSchedule s = make_schedule(M, N, K, 0, world_size, comm_block_m, cus, true, 1);
-  out4[0] = s.grid;
-  out4[1] = estimate_fused(s, cus, s.grid, 1).producer_wgs;
-  out4[2] = 0;
-  out4[3] = 0;
+  if (out5 == nullptr) return fail(SMR_E_INVALID, "smr_ag_matmul_plan_fp8: out5 is NULL");
+  fill_plan(M, N, K, world_size, comm_block_m, 1, out5);
   return 0;
 }
 
@@ -1007,21 +1004,37 @@ int smr_set_ag_matmul_halves(int head, int tail) {
   return 0;
 }
 
-int smr_ag_matmul_plan(int M, int N, int K, int world_size, int comm_block_m, int32_t* out4) {
+// Fills the plan of a fused launch: {GEMM grid, producer workgroups, fast chunks, slow
+// workgroups, sequential}.
+static void fill_plan(int M, int N, int K, int world_size, int comm_block_m, int elem_bytes, int32_t* out5) {
+  using namespace smr;
+  const int cus = cu_count();
+  const GemmSchedule s = make_schedule(M, N, K, 0, world_size, comm_block_m, cus, true, elem_bytes);
+  const FusedEstimate e = estimate_fused(s, cus, s.grid, elem_bytes);
+  // The alternative for a problem too small to hide the copy behind: copy with the
+  // whole GPU, then multiply with the whole GPU.
+  const GemmSchedule u = make_schedule(M, N, K, 0, world_size, comm_block_m, cus, false, elem_bytes);
+  const double tile_us = 2.0 * u.BM * u.BN * K / (elem_bytes == 1 ? 12.0e6 : 6.0e6) + 8.0;
+  const int tiles = (M / u.BM) * ceil_div(N, u.BN);
+  const double remote_bytes = 2.0 * elem_bytes * M * K * (world_size - 1) / world_size;
+  const double seq_us = copy_us(remote_bytes, M / comm_block_m, cus) + ceil_div(tiles, u.grid) * tile_us + 5.0;
+  const bool sequential = seq_us < 0.9 * e.total_us;
+  // Fused, the copy runs flat out on what the grid leaves free: with write-through
+  // stores it no longer pays to hold it back (pacing it to two thirds of its width cost
+  // 3 % on the M=16384 N=3584 K=8192 problem, where it used to gain 2 %).
+  out5[0] = sequential ? u.grid : s.grid;
+  out5[1] = sequential ? cus : e.producer_wgs;
+  out5[2] = 0;
+  out5[3] = 0;
+  out5[4] = sequential ? 1 : 0;
+}
+
+int smr_ag_matmul_plan(int M, int N, int K, int world_size, int comm_block_m, int32_t* out5) {
   using namespace smr;
   const char* why;
   if (int rc = validate(M, N, K, 0, world_size, comm_block_m, &why)) return fail(rc, why);
-  if (out4 == nullptr) return fail(SMR_E_INVALID, "smr_ag_matmul_plan: out4 is NULL");
-  const int cus = cu_count();
-  const GemmSchedule s = make_schedule(M, N, K, 0, world_size, comm_block_m, cus, true);
-  FusedEstimate e = estimate_fused(s, cus, s.grid);
-  // The copy runs flat out on what the grid leaves free: with write-through stores it
-  // no longer pays to hold it back (pacing it to two thirds of its width cost 3 % on
-  // the M=16384 N=3584 K=8192 problem, where it used to gain 2 %).
-  out4[0] = s.grid;
-  out4[1] = e.producer_wgs;
-  out4[2] = 0;
-  out4[3] = 0;
+  if (out5 == nullptr) return fail(SMR_E_INVALID, "smr_ag_matmul_plan: out5 is NULL");
+  fill_plan(M, N, K, world_size, comm_block_m, 2, out5);
   return 0;
 }
 

@@ -23,6 +23,8 @@ from .symm_mem import EmulatedSymmetricMemory, _get_backend_stream
 #: shape (smr_ag_matmul_plan); a number / a (fast_chunks, slow_workgroups) pair overrides.
 MAX_PRODUCER_WORKGROUPS = None
 PRODUCER_PACING = None
+#: None = the plan decides between the fused launch and copy-then-multiply; True / False force one.
+FUSED = None
 
 
 def all_gather_with_progress(output: torch.Tensor, inp: torch.Tensor, progress: torch.Tensor,
@@ -120,11 +122,20 @@ def all_gather_matmul_tma_persistent(a_shard: torch.Tensor, b: torch.Tensor, a_o
         flags.record_stream(backend)
         assert a_out.dtype == a_shard.dtype and a_out.is_contiguous()
         # the producer takes (some of) the compute units the GEMM's grid leaves free
-        plan = (ctypes.c_int32 * 4)()
+        plan = (ctypes.c_int32 * 5)()
         planner = lib.smr_ag_matmul_plan_fp8 if fp8 else lib.smr_ag_matmul_plan
         _lib.check(planner(M, N, K, world_size, COMM_BLOCK_SIZE_M, plan), "all_gather_matmul")
         producer_wgs = plan[1] if MAX_PRODUCER_WORKGROUPS is None else min(MAX_PRODUCER_WORKGROUPS, plan[1])
         pacing = (plan[2], plan[3]) if PRODUCER_PACING is None else PRODUCER_PACING
+        sequential = bool(plan[4]) and FUSED is None or FUSED is False
+        if sequential:
+            # Too small to hide the copy behind the GEMM: the whole GPU copies, then the whole
+            # GPU multiplies, in stream order (the GEMM then needs no flags).
+            _lib.check(lib.smr_set_gather_pacing(0, 0), "all_gather_matmul")
+            wide = torch.cuda.get_device_properties(device).multi_processor_count
+            _launch_producer(symm_mem, a_out, a_shard, progress, counters, splits_per_rank, wide,
+                             current.cuda_stream)
+            progress_ptr = 0
 
     # The GEMM goes first: its first tiles are local rows and need no flag, so the
     # producer's launch latency is hidden behind them instead of delaying the GEMM.
@@ -134,7 +145,7 @@ def all_gather_matmul_tma_persistent(a_shard: torch.Tensor, b: torch.Tensor, a_o
               progress_ptr, M, N, K, rank, world_size, COMM_BLOCK_SIZE_M, status_ptr,
               current.cuda_stream)
     _lib.check(rc, "all_gather_matmul")
-    if not mm_only:
+    if not mm_only and not sequential:
         _lib.check(lib.smr_set_gather_pacing(int(pacing[0]), int(pacing[1])), "all_gather_matmul")
         _launch_producer(symm_mem, a_out, a_shard, progress, counters, splits_per_rank, producer_wgs,
                          backend.cuda_stream)

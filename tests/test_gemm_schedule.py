@@ -129,23 +129,29 @@ def test_grid_leaves_room_for_the_producer(lib):
 
 def test_fused_plan_splits_the_gpu(lib):
     """smr_ag_matmul_plan: GEMM grid + producer fit the GPU (256 compute units assumed
-    without one), the grid is the one the gated GEMM launches, and a skinny problem -
-    little GEMM work per copied byte - gives the producer more of the GPU."""
+    without one); a fused plan's grid is the one the gated GEMM launches; a problem too
+    small to hide the copy behind is planned as copy-then-multiply on the whole GPU."""
     import ctypes
     plans = {}
-    for (M, N, K) in [(16384, 3584, 8192), (16384, 1792, 4096), (4096, 1792, 4096), (16384, 6656, 16384),
+    for (M, N, K) in [(16384, 3584, 8192), (16384, 6656, 16384), (8192, 3584, 8192), (4096, 1792, 4096),
                       (1024, 256, 256)]:
-        out = (ctypes.c_int32 * 4)()
+        out = (ctypes.c_int32 * 5)()
         assert lib.smr_ag_matmul_plan(M, N, K, 8, M // 8, out) == 0
-        grid, wgs, fast, slow = list(out)
-        assert grid == lib.smr_ag_matmul_grid(M, N, K, 8, M // 8, 1)
-        assert grid % 8 == 0 and 8 <= grid <= 248
-        assert 1 <= wgs <= 128 and grid + wgs <= 256
+        grid, wgs, fast, slow, sequential = list(out)
+        assert grid % 8 == 0 and 8 <= grid <= 256
         assert (fast, slow) == (0, 0)
-        plans[(M, N, K)] = (grid, wgs)
-    assert plans[(16384, 3584, 8192)] == (224, 32)
-    assert plans[(16384, 1792, 4096)][1] > plans[(16384, 3584, 8192)][1]
-    assert lib.smr_ag_matmul_plan(1000, 256, 256, 8, 125, (ctypes.c_int32 * 4)()) == -2      # unsupported shape
+        if sequential:
+            assert grid == lib.smr_ag_matmul_grid(M, N, K, 8, M // 8, 0) and wgs == 256
+        else:
+            assert grid == lib.smr_ag_matmul_grid(M, N, K, 8, M // 8, 1) and grid <= 248
+            assert 1 <= wgs <= 128 and grid + wgs <= 256
+        plans[(M, N, K)] = (grid, wgs, sequential)
+    assert plans[(16384, 3584, 8192)] == (224, 32, 0)
+    assert plans[(4096, 1792, 4096)][2] == 1
+    out = (ctypes.c_int32 * 5)()
+    assert lib.smr_ag_matmul_plan_fp8(16384, 3584, 8192, 8, 2048, out) == 0 and list(out) == [224, 32, 0, 0, 0]
+    assert lib.smr_ag_matmul_plan_fp8(16384, 3584, 8192 + 64, 8, 2048, out) == -2      # K % 128
+    assert lib.smr_ag_matmul_plan(1000, 256, 256, 8, 125, out) == -2                   # unsupported shape
     assert lib.smr_ag_matmul_plan(1024, 256, 256, 8, 128, None) == -1
 
 
