@@ -181,3 +181,73 @@ def gemm_schedule(M: int, N: int, K: int, rank: int, world_size: int, comm_block
     lib.smr_ag_matmul_schedule(M, N, K, rank, world_size, comm_block_m, int(gated), buf, n)
     keys = ("wg", "step", "row0", "col0", "rows", "cols", "comm_block", "local")
     return [dict(zip(keys, buf[8 * i:8 * i + 8])) for i in range(n)]
+
+
+def main(argv=None) -> None:
+    """The reference's harness (triton_all_gather_matmul.py:329-418) with its
+    options (all but --print_ptx: there is no PTX): fused result checked against gather + library matmul, then the four
+    latency lines.  The tile options are accepted and checked as there
+    (rows per flag must divide into BLOCK_SIZE_M * GROUP_SIZE_M); the tile the
+    kernel runs is the library's.  Run as ``python -m symm_mem_recipes.all_gather_matmul``."""
+    import argparse
+
+    from .utils import benchmark_with_event
+
+    ap = argparse.ArgumentParser(description="all-gather matmul: parity check and latencies")
+    ap.add_argument("--M", type=int, default=4096)
+    ap.add_argument("--N", type=int, default=6656)
+    ap.add_argument("--K", type=int, default=16384)
+    ap.add_argument("--BLOCK_SIZE_M", type=int, default=128)
+    ap.add_argument("--BLOCK_SIZE_N", type=int, default=256)
+    ap.add_argument("--BLOCK_SIZE_K", type=int, default=64)
+    ap.add_argument("--GROUP_SIZE_M", type=int, default=4)
+    ap.add_argument("--num_stages", type=int, default=3)
+    ap.add_argument("--num_warps", type=int, default=8)
+    args = ap.parse_args(argv)
+
+    rank = int(os.environ.get("RANK", "0"))
+    world_size = int(os.environ.get("WORLD_SIZE", "8"))
+    device = torch.device("cuda:0")
+    torch.cuda.set_device(device)
+    m, n, k = args.M, args.N, args.K
+
+    a_shard = EmulatedSymmetricMemory.empty_strided_p2p(
+        size=(m // world_size, k), stride=(k, 1), dtype=torch.bfloat16, device=device,
+        world_size=world_size, rank=rank)
+    symm_mem = EmulatedSymmetricMemory.rendezvous(a_shard)
+    for r in range(world_size):
+        torch.manual_seed(42 + r)
+        symm_mem.get_buffer(r, (m // world_size, k), torch.bfloat16).normal_()
+    torch.manual_seed(42 + rank)
+    a = torch.randn((m, k), device=device, dtype=torch.bfloat16)
+    b = torch.randn((k, n), device=device, dtype=torch.bfloat16).T.contiguous()
+    c = torch.randn((m, n), device=device, dtype=torch.bfloat16)
+
+    configs = {
+        "BLOCK_SIZE_M": args.BLOCK_SIZE_M, "BLOCK_SIZE_N": args.BLOCK_SIZE_N,
+        "BLOCK_SIZE_K": args.BLOCK_SIZE_K, "GROUP_SIZE_M": args.GROUP_SIZE_M,
+        "num_stages": args.num_stages, "num_warps": args.num_warps,
+    }
+
+    c0 = all_gather_matmul(a_shard, b.T)
+    c1 = all_gather_matmul_tma_persistent(a_shard, b, a, c, configs)
+    symm_mem.check_status()
+    # two GEMMs that sum K in different orders: bf16's last place (2^-8) of the larger of the
+    # two values is what can differ, plus cancellation noise relative to the row's magnitude
+    assert torch.allclose(c0.float(), c1.float(), rtol=1e-2, atol=1e-2 * c0.float().abs().max().item())
+
+    lat_us = benchmark_with_event(lambda: torch.matmul(a, b.T, out=c), flush_l2=True)
+    print(f"library matmul only: {lat_us} us")
+    lat_us = benchmark_with_event(
+        lambda: all_gather_matmul_tma_persistent(a_shard, b, a, c, configs, mm_only=True), flush_l2=True)
+    print(f"hip matmul only: {lat_us} us")
+    lat_us = benchmark_with_event(lambda: all_gather_matmul(a_shard, b.T), flush_l2=True)
+    print(f"library gather + matmul: {lat_us} us")
+    lat_us = benchmark_with_event(
+        lambda: all_gather_matmul_tma_persistent(a_shard, b, a, c, configs), flush_l2=True)
+    print(f"hip all_gather_matmul: {lat_us} us")
+    symm_mem.check_status()
+
+
+if __name__ == "__main__":
+    main()

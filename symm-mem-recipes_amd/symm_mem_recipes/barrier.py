@@ -51,3 +51,26 @@ def wait_signal(addr: int, symm_mem: EmulatedSymmetricMemory, reset: bool = Fals
     lib = _lib.load()
     fn = lib.smr_wait_signal_reset if reset else lib.smr_wait_signal
     _lib.check(fn(int(addr), symm_mem.status.data_ptr(), _stream(symm_mem.device)), "wait_signal")
+
+
+def main() -> None:
+    """The reference's self-check (triton_barrier.py:172-200): one barrier on 32
+    blocks over zeroed 4096-word buffers must return, and the buffer prints as
+    zeros.  Run as ``python -m symm_mem_recipes.barrier``."""
+    import os
+
+    world_size = int(os.environ.get("WORLD_SIZE", "8"))
+    device = torch.device("cuda:0")
+    torch.cuda.set_device(device)
+
+    t = EmulatedSymmetricMemory.empty_strided_p2p(
+        size=(4096,), stride=(1,), dtype=torch.uint32, device=device, world_size=world_size).fill_(0)
+    symm_mem = EmulatedSymmetricMemory.rendezvous(t)
+    barrier_test(symm_mem)
+    torch.cuda.synchronize(device)
+    symm_mem.check_status()
+    print(t)
+
+
+if __name__ == "__main__":
+    main()

@@ -90,3 +90,36 @@ def one_shot_all_reduce(tensor: torch.Tensor, *, barrier: bool = True, write_all
     if two_shot:
         return symm_mem.all_buffers(tuple(tensor.shape), tensor.dtype)
     return output
+
+
+def main() -> None:
+    """The reference's self-check and latency line
+    (triton_one_shot_all_reduce.py:128-162): 8192 ones per rank must sum to
+    world_size, then the kernel's median device time.  The ranks are emulated in
+    one GPU's memory (WORLD_SIZE, default 8); run as
+    ``python -m symm_mem_recipes.one_shot_all_reduce``."""
+    import os
+
+    from .utils import benchmark_with_profiler
+
+    world_size = int(os.environ.get("WORLD_SIZE", "8"))
+    device = torch.device("cuda:0")
+    torch.cuda.set_device(device)
+
+    tensor = EmulatedSymmetricMemory.empty_strided_p2p(
+        size=(8192,), stride=(1,), dtype=torch.bfloat16, device=device, world_size=world_size)
+    symm_mem = EmulatedSymmetricMemory.rendezvous(tensor)
+    for r in range(world_size):
+        symm_mem.get_buffer(r, (8192,), torch.bfloat16).fill_(1)
+
+    output = one_shot_all_reduce(tensor)
+    assert output.eq(world_size).all().item()
+    symm_mem.check_status()
+
+    lat_us = benchmark_with_profiler(lambda: one_shot_all_reduce(tensor),
+                                     r".*one_shot_all_reduce_kernel", benchmark_iters=200)
+    print(f"Median latency: {lat_us:.2f} us")
+
+
+if __name__ == "__main__":
+    main()

@@ -47,3 +47,19 @@ def test_rank_selection_and_release():
     assert SM.rendezvous(t) is None
     with pytest.raises(AssertionError):
         SM.empty_strided_p2p((8,), (1,), torch.float32, "cpu", world_size=9)
+
+
+def test_reference_import_paths_resolve():
+    """A caller written against the reference's module names gets the same functions."""
+    import importlib
+    import symm_mem_recipes as pkg
+    for module, names in (("triton_one_shot_all_reduce", ("one_shot_all_reduce",)),
+                          ("triton_barrier", ("barrier_test", "blockwise_barrier")),
+                          ("triton_all_gather_matmul", ("all_gather_with_progress", "all_gather_matmul",
+                                                        "all_gather_matmul_tma_persistent")),
+                          ("utils", ("benchmark_with_event", "benchmark_with_profiler"))):
+        mod = importlib.import_module(f"symm_mem_recipes.{module}")
+        for name in names:
+            assert callable(getattr(mod, name))
+            if hasattr(pkg, name):
+                assert getattr(mod, name) is getattr(pkg, name)
