@@ -147,6 +147,32 @@ def test_fused_back_to_back_calls_are_identical(cuda):
         assert torch.equal(c.view(torch.int16), outs[0].view(torch.int16))
 
 
+def test_copy_then_multiply_matches_fused(cuda, lib, monkeypatch):
+    """A GEMM too short to hide the copy behind is planned as copy-then-multiply
+    (M=4096 N=1792 K=4096 is); the planned form and both forced forms give the oracle's
+    product and one another's bits, with the gathered operand complete in each."""
+    import ctypes
+    import importlib
+    agm = importlib.import_module("symm_mem_recipes.all_gather_matmul")
+    M, N, K, ws, rank = 4096, 1792, 4096, 8, 3
+    plan = (ctypes.c_int32 * 5)()
+    assert lib.smr_ag_matmul_plan(M, N, K, ws, M // ws, plan) == 0 and plan[4] == 1
+    a_shard, h, shards, b, b_bits, a_out, c_out = _setup(M, N, K, ws, rank, cuda)
+    want = O.ag_matmul_ref(shards, b_bits)
+    outs = []
+    for fused in (None, True, False):
+        monkeypatch.setattr(agm, "FUSED", fused)
+        a_out.zero_()
+        c = torch.full_like(c_out, float("nan"))
+        agm.all_gather_matmul_tma_persistent(a_shard, b, a_out, c, None)
+        h.check_status()
+        assert np.array_equal(_t_bits(a_out), np.concatenate(shards))
+        _check(_t_bits(c), want)
+        outs.append(c)
+    assert torch.equal(outs[0].view(torch.int16), outs[1].view(torch.int16))
+    assert torch.equal(outs[0].view(torch.int16), outs[2].view(torch.int16))
+
+
 def test_mm_only_is_ungated(cuda, monkeypatch):
     """mm_only multiplies what the buffers already hold, as rank 0, with no flags
     (triton_all_gather_matmul.py:222-224,246-247)."""
