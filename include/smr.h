@@ -167,6 +167,15 @@ int smr_all_gather_with_progress(const uint64_t* buffer_ptrs_dev, void* a_out_de
                                  int world_size, int64_t shard_bytes, int splits_per_rank,
                                  int num_workgroups, void* stream);
 
+/* The same gather for a caller that does not watch the flags on the way (a GEMM queued
+ * behind it in stream order): all chunks are copied together and every flag is raised at
+ * the end.  Same arguments and the same final state of a_out, progress and counters as
+ * smr_all_gather_with_progress (triton_all_gather_matmul.py:20-56 run to completion). */
+int smr_all_gather_at_once(const uint64_t* buffer_ptrs_dev, void* a_out_dev,
+                           uint32_t* progress_dev, uint32_t* counters_dev, int rank,
+                           int world_size, int64_t shard_bytes, int splits_per_rank,
+                           int num_workgroups, void* stream);
+
 /* Pacing of the producer: the first `fast_chunks` chunks are copied by all
  * workgroups, the remaining ones by `slow_workgroups` of them (0 = all, i.e. no
  * pacing).  Default 0 and 0.  No reference counterpart (copy engines pace
@@ -205,12 +214,13 @@ int smr_ag_matmul_fp8(const void* a_shard_dev, const void* a_out_dev, const void
 int smr_ag_matmul_plan_fp8(int M, int N, int K, int world_size, int comm_block_m, int32_t* out5);
 
 /* Host-only: how a fused launch of this shape splits the GPU.  out5 = {GEMM grid,
- * producer workgroups, fast_chunks, slow_workgroups, sequential}.  fast_chunks and
- * slow_workgroups are the arguments of smr_set_gather_pacing ({0, 0}: the copy runs flat
- * out).  sequential = 1: the problem is too small to hide the copy behind the GEMM; copy
- * with the whole GPU first (producer workgroups = all compute units), then call
- * smr_ag_matmul with progress = NULL in stream order behind it.  sequential = 0: launch
- * smr_ag_matmul gated (it uses the grid given here) and the producer beside it.
+ * producer workgroups, fused_us, sequential_us, sequential}.  The first two are the split
+ * of a fused launch: smr_ag_matmul gated uses that grid, the producer
+ * (smr_all_gather_with_progress) gets that many workgroups beside it.  fused_us and
+ * sequential_us are the planner's estimates, in microseconds, of that launch and of the
+ * alternative: gather with the whole GPU (smr_all_gather_at_once, one workgroup per
+ * compute unit), then smr_ag_matmul with progress = NULL behind it in stream order.
+ * sequential = 1 recommends the alternative: the GEMM is too short to hide the copy behind.
  * Replaces the fixed NUM_SMS grid of triton_all_gather_matmul.py:287-294: there the copy
  * engines cost no SMs. */
 int smr_ag_matmul_plan(int M, int N, int K, int world_size, int comm_block_m, int32_t* out5);

@@ -835,6 +835,8 @@ struct FusedEstimate {
   int producer_wgs;
 };
 constexpr int kMaxProducerWgs = 128;
+// copy-then-multiply is chosen when its estimate is below this multiple of the fused one
+constexpr double kSequentialBias = 1.0;
 // every chunk ends with a wait for the stores, a workgroup barrier and an arrival count
 static double copy_us(double bytes, int chunks, int wgs) { return bytes / (wgs * 35.0e3) + 2.5 * chunks; }
 static FusedEstimate estimate_fused(const GemmSchedule& s, int cus, int grid, int elem_bytes = 2) {
@@ -1004,8 +1006,8 @@ int smr_set_ag_matmul_halves(int head, int tail) {
   return 0;
 }
 
-// Fills the plan of a fused launch: {GEMM grid, producer workgroups, fast chunks, slow
-// workgroups, sequential}.
+// Fills the plan of a fused launch: {GEMM grid, producer workgroups, estimated
+// microseconds fused, estimated microseconds copy-then-multiply, sequential}.
 static void fill_plan(int M, int N, int K, int world_size, int comm_block_m, int elem_bytes, int32_t* out5) {
   using namespace smr;
   const int cus = cu_count();
@@ -1014,19 +1016,19 @@ static void fill_plan(int M, int N, int K, int world_size, int comm_block_m, int
   // The alternative for a problem too small to hide the copy behind: copy with the
   // whole GPU, then multiply with the whole GPU.
   const GemmSchedule u = make_schedule(M, N, K, 0, world_size, comm_block_m, cus, false, elem_bytes);
-  const double tile_us = 2.0 * u.BM * u.BN * K / (elem_bytes == 1 ? 12.0e6 : 6.0e6) + 8.0;
+  // (with no copy next to it a GEMM workgroup sustains a little more: 6.4 TFLOP/s)
+  const double tile_us = 2.0 * u.BM * u.BN * K / (elem_bytes == 1 ? 12.8e6 : 6.4e6) + 8.0;
   const int tiles = (M / u.BM) * ceil_div(N, u.BN);
-  const double remote_bytes = 2.0 * elem_bytes * M * K * (world_size - 1) / world_size;
-  const double seq_us = copy_us(remote_bytes, M / comm_block_m, cus) + ceil_div(tiles, u.grid) * tile_us + 5.0;
-  const bool sequential = seq_us < 0.9 * e.total_us;
-  // Fused, the copy runs flat out on what the grid leaves free: with write-through
-  // stores it no longer pays to hold it back (pacing it to two thirds of its width cost
-  // 3 % on the M=16384 N=3584 K=8192 problem, where it used to gain 2 %).
-  out5[0] = sequential ? u.grid : s.grid;
-  out5[1] = sequential ? cus : e.producer_wgs;
-  out5[2] = 0;
-  out5[3] = 0;
-  out5[4] = sequential ? 1 : 0;
+  // the ungated schedule ends on a pass of half tiles when that is shorter: count passes in halves
+  const double passes = ceil_div(2 * tiles, u.grid) * 0.5;
+  // (all chunks at once, the own shard included: read + write at what a copy reaches on the part)
+  const double gather_us = 2.0 * elem_bytes * M * K / 5.0e6 + 4.0;
+  const double seq_us = gather_us + passes * tile_us + 5.0;
+  out5[0] = s.grid;
+  out5[1] = e.producer_wgs;
+  out5[2] = (int32_t)(e.total_us + 0.5);
+  out5[3] = (int32_t)(seq_us + 0.5);
+  out5[4] = seq_us < kSequentialBias * e.total_us ? 1 : 0;
 }
 
 int smr_ag_matmul_plan(int M, int N, int K, int world_size, int comm_block_m, int32_t* out5) {

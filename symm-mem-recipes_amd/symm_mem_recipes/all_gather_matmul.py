@@ -20,7 +20,8 @@ from . import _lib
 from .symm_mem import EmulatedSymmetricMemory, _get_backend_stream
 
 #: Producer width and pacing of a fused launch.  None = the library's plan for the
-#: shape (smr_ag_matmul_plan); a number / a (fast_chunks, slow_workgroups) pair overrides.
+#: shape (smr_ag_matmul_plan) and no pacing; a number / a (fast_chunks, slow_workgroups)
+#: pair overrides.
 MAX_PRODUCER_WORKGROUPS = None
 PRODUCER_PACING = None
 #: None = the plan decides between the fused launch and copy-then-multiply; True / False force one.
@@ -56,10 +57,12 @@ def all_gather_with_progress(output: torch.Tensor, inp: torch.Tensor, progress: 
 
 
 def _launch_producer(symm_mem, output, inp, progress, counters, splits_per_rank, num_workgroups,
-                     stream_handle) -> None:
+                     stream_handle, at_once: bool = False) -> None:
     """The producer kernel on the given stream; ``counters`` (one zeroed int32 per
-    chunk) are its arrival counters."""
-    rc = _lib.load().smr_all_gather_with_progress(
+    chunk) are its arrival counters.  ``at_once`` copies all chunks together and raises
+    the flags at the end, for a consumer that is queued behind the copy."""
+    lib = _lib.load()
+    rc = (lib.smr_all_gather_at_once if at_once else lib.smr_all_gather_with_progress)(
         symm_mem.buffer_ptrs_dev, output.data_ptr(), progress.data_ptr(), counters.data_ptr(),
         symm_mem.rank, symm_mem.world_size, inp.numel() * inp.element_size(), int(splits_per_rank),
         int(num_workgroups), stream_handle)
@@ -126,15 +129,14 @@ def all_gather_matmul_tma_persistent(a_shard: torch.Tensor, b: torch.Tensor, a_o
         planner = lib.smr_ag_matmul_plan_fp8 if fp8 else lib.smr_ag_matmul_plan
         _lib.check(planner(M, N, K, world_size, COMM_BLOCK_SIZE_M, plan), "all_gather_matmul")
         producer_wgs = plan[1] if MAX_PRODUCER_WORKGROUPS is None else min(MAX_PRODUCER_WORKGROUPS, plan[1])
-        pacing = (plan[2], plan[3]) if PRODUCER_PACING is None else PRODUCER_PACING
+        pacing = (0, 0) if PRODUCER_PACING is None else PRODUCER_PACING
         sequential = bool(plan[4]) and FUSED is None or FUSED is False
         if sequential:
             # Too small to hide the copy behind the GEMM: the whole GPU copies, then the whole
             # GPU multiplies, in stream order (the GEMM then needs no flags).
-            _lib.check(lib.smr_set_gather_pacing(0, 0), "all_gather_matmul")
             wide = torch.cuda.get_device_properties(device).multi_processor_count
             _launch_producer(symm_mem, a_out, a_shard, progress, counters, splits_per_rank, wide,
-                             current.cuda_stream)
+                             current.cuda_stream, at_once=True)
             progress_ptr = 0
 
     # The GEMM goes first: its first tiles are local rows and need no flag, so the

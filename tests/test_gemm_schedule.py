@@ -129,27 +129,29 @@ def test_grid_leaves_room_for_the_producer(lib):
 
 def test_fused_plan_splits_the_gpu(lib):
     """smr_ag_matmul_plan: GEMM grid + producer fit the GPU (256 compute units assumed
-    without one); a fused plan's grid is the one the gated GEMM launches; a problem too
-    small to hide the copy behind is planned as copy-then-multiply on the whole GPU."""
+    without one) and the grid is the one the gated GEMM launches; both forms come with an
+    estimate, and a problem too small to hide the copy behind is planned as copy-then-multiply."""
     import ctypes
     plans = {}
-    for (M, N, K) in [(16384, 3584, 8192), (16384, 6656, 16384), (8192, 3584, 8192), (4096, 1792, 4096),
-                      (1024, 256, 256)]:
+    for (M, N, K) in [(16384, 3584, 8192), (16384, 6656, 16384), (8192, 3584, 8192), (16384, 1792, 4096),
+                      (4096, 1792, 4096), (1024, 256, 256)]:
         out = (ctypes.c_int32 * 5)()
         assert lib.smr_ag_matmul_plan(M, N, K, 8, M // 8, out) == 0
-        grid, wgs, fast, slow, sequential = list(out)
-        assert grid % 8 == 0 and 8 <= grid <= 256
-        assert (fast, slow) == (0, 0)
-        if sequential:
-            assert grid == lib.smr_ag_matmul_grid(M, N, K, 8, M // 8, 0) and wgs == 256
-        else:
-            assert grid == lib.smr_ag_matmul_grid(M, N, K, 8, M // 8, 1) and grid <= 248
-            assert 1 <= wgs <= 128 and grid + wgs <= 256
+        grid, wgs, fused_us, sequential_us, sequential = list(out)
+        assert grid % 8 == 0 and 8 <= grid <= 248
+        assert grid == lib.smr_ag_matmul_grid(M, N, K, 8, M // 8, 1)
+        assert 1 <= wgs <= 128 and grid + wgs <= 256
+        assert fused_us > 0 and sequential_us > 0
+        assert sequential == (1 if sequential_us < fused_us else 0)
         plans[(M, N, K)] = (grid, wgs, sequential)
     assert plans[(16384, 3584, 8192)] == (224, 32, 0)
-    assert plans[(4096, 1792, 4096)][2] == 1
+    assert plans[(16384, 6656, 16384)][2] == 0
+    assert plans[(4096, 1792, 4096)][2] == 1 and plans[(1024, 256, 256)][2] == 1
+    # a skinny problem leaves the producer more of the GPU
+    assert plans[(16384, 1792, 4096)][1] > plans[(16384, 3584, 8192)][1]
     out = (ctypes.c_int32 * 5)()
-    assert lib.smr_ag_matmul_plan_fp8(16384, 3584, 8192, 8, 2048, out) == 0 and list(out) == [224, 32, 0, 0, 0]
+    assert lib.smr_ag_matmul_plan_fp8(16384, 3584, 8192, 8, 2048, out) == 0
+    assert list(out)[:2] == [224, 32] and out[4] == 0
     assert lib.smr_ag_matmul_plan_fp8(16384, 3584, 8192 + 64, 8, 2048, out) == -2      # K % 128
     assert lib.smr_ag_matmul_plan(1000, 256, 256, 8, 125, out) == -2                   # unsupported shape
     assert lib.smr_ag_matmul_plan(1024, 256, 256, 8, 128, None) == -1

@@ -47,6 +47,21 @@ def _check(got_bits, want_bits):
     assert np.mean(err <= ulp) >= 0.999
 
 
+@pytest.fixture
+def force_fused(monkeypatch):
+    """Small problems are planned as copy-then-multiply; the tests of the flag-gated
+    launch force it."""
+    import importlib
+    monkeypatch.setattr(importlib.import_module("symm_mem_recipes.all_gather_matmul"), "FUSED", True)
+
+
+@pytest.fixture(params=[True, False], ids=["fused", "copy-then-multiply"])
+def either_form(request, monkeypatch):
+    import importlib
+    monkeypatch.setattr(importlib.import_module("symm_mem_recipes.all_gather_matmul"), "FUSED", request.param)
+    return request.param
+
+
 @pytest.fixture(autouse=True)
 def _release():
     yield
@@ -68,6 +83,30 @@ def test_all_gather_with_progress(cuda, rank, splits):
     assert progress.cpu().tolist() == prog.tolist()
 
 
+@pytest.mark.parametrize("ws,rows,K,splits,wgs", [(8, 96, 200, 1, 3), (8, 96, 200, 2, 256), (3, 64, 72, 4, 1),
+                                                 (8, 8, 8, 1, 256), (8, 512, 4096, 4, 256)])
+def test_all_gather_at_once(cuda, lib, ws, rows, K, splits, wgs):
+    """All chunks copied together (the copy a GEMM is queued behind): the same gathered
+    operand, flags and zeroed counters as the chunk-by-chunk producer leaves."""
+    rank = ws - 1
+    a_shard, h, shards, *_ = _setup(ws * rows, 8, K, ws, rank, cuda)
+    out = torch.zeros(ws * rows, K, dtype=torch.bfloat16, device=cuda)
+    state = torch.zeros(2 * ws * splits, dtype=torch.int32, device=cuda)
+    progress, counters = state[:ws * splits], state[ws * splits:]
+    for _ in range(2):                                   # the counters are left ready for the next call
+        out.zero_()
+        progress.zero_()
+        rc = lib.smr_all_gather_at_once(h.buffer_ptrs_dev, out.data_ptr(), progress.data_ptr(),
+                                        counters.data_ptr(), rank, ws, rows * K * 2, splits, wgs,
+                                        torch.cuda.current_stream(cuda).cuda_stream)
+        assert rc == 0
+        torch.cuda.synchronize()
+        want, prog, _ = O.all_gather_ref(shards, rank, splits)
+        assert np.array_equal(_t_bits(out), want)
+        assert progress.cpu().tolist() == prog.tolist()
+        assert counters.cpu().tolist() == [0] * (ws * splits)
+
+
 @pytest.mark.parametrize("M,N,K,ws,rank", [
     (1024, 256, 256, 8, 0),      # 128x128 tiles
     (1024, 136, 64, 8, 6),       # ragged last column tile, single K step
@@ -75,7 +114,7 @@ def test_all_gather_with_progress(cuda, rank, splits):
     (2048, 128, 1024, 8, 7),     # 256x128 tiles
     (1024, 512, 320, 4, 1),      # world size 4
 ])
-def test_fused_parity_small(cuda, M, N, K, ws, rank):
+def test_fused_parity_small(cuda, either_form, M, N, K, ws, rank):
     from symm_mem_recipes import all_gather_matmul_tma_persistent, all_gather_matmul
     a_shard, h, shards, b, b_bits, a_out, c_out = _setup(M, N, K, ws, rank, cuda)
     configs = {"BLOCK_SIZE_M": 128, "BLOCK_SIZE_N": 128, "BLOCK_SIZE_K": 64, "GROUP_SIZE_M": 1,
@@ -97,7 +136,7 @@ def test_fused_parity_small(cuda, M, N, K, ws, rank):
     (4096, 512, 128, 8, 6, 2),       # comm blocks of 256 rows: 256x256 tiles, 16 flags
     (4096, 384, 192, 4, 1, 4),       # world size 4, four flags per rank
 ])
-def test_fused_parity_splits_per_rank(cuda, M, N, K, ws, rank, splits):
+def test_fused_parity_splits_per_rank(cuda, either_form, M, N, K, ws, rank, splits):
     """Finer flags (triton_all_gather_matmul.py:24,41-49): every rank's shard arrives in
     `splits` chunks with a flag each, and a tile waits for the chunk its rows are in."""
     from symm_mem_recipes import all_gather_matmul_tma_persistent
@@ -110,7 +149,7 @@ def test_fused_parity_splits_per_rank(cuda, M, N, K, ws, rank, splits):
 
 
 @pytest.mark.parametrize("head,tail", [(0, 0), (1, 0), (1, 1), (2, 0), (0, 2), (3, 3)])
-def test_fused_parity_half_tile_phases(cuda, lib, head, tail):
+def test_fused_parity_half_tile_phases(cuda, lib, force_fused, head, tail):
     """Every split of the gated schedule into half-width and full-width phases computes
     the same product (the library picks one by cost; this forces the others)."""
     from symm_mem_recipes import all_gather_matmul_tma_persistent
@@ -126,7 +165,7 @@ def test_fused_parity_half_tile_phases(cuda, lib, head, tail):
     _check(_t_bits(c_out), O.ag_matmul_ref(shards, b_bits))
 
 
-def test_fused_back_to_back_calls_are_identical(cuda):
+def test_fused_back_to_back_calls_are_identical(cuda, either_form):
     """Twenty fused launches in a row without a host synchronisation in between, the
     gathered operand wiped before each: flags, arrival counters and the two streams
     must hand over cleanly from one call to the next, and the result is deterministic."""
@@ -171,6 +210,40 @@ def test_copy_then_multiply_matches_fused(cuda, lib, monkeypatch):
         outs.append(c)
     assert torch.equal(outs[0].view(torch.int16), outs[1].view(torch.int16))
     assert torch.equal(outs[0].view(torch.int16), outs[2].view(torch.int16))
+
+
+@pytest.mark.parametrize("M,N,K", [(8192, 1024, 1024), (4096, 1792, 4096)])
+def test_fused_launch_replays_from_a_graph(cuda, either_form, M, N, K):
+    """The whole call - flag fill, handshake, GEMM, producer on the second stream and the
+    join - captured into a HIP graph (kernel nodes only) and replayed: every replay, with
+    eager work and synchronisations in between, gives the eager result, for the fused form (two concurrent branches) and for copy-then-multiply."""
+    from symm_mem_recipes import all_gather_matmul_tma_persistent
+    ws, rank = 8, 2
+    a_shard, h, shards, b, b_bits, a_out, c_out = _setup(M, N, K, ws, rank, cuda)
+    all_gather_matmul_tma_persistent(a_shard, b, a_out, c_out, None)          # eager: the expected bits
+    torch.cuda.synchronize()
+    h.check_status()
+    want_c, want_a = c_out.clone(), a_out.clone()
+    _check(_t_bits(want_c)[:64], O.ag_matmul_ref([shards[0][:64]], b_bits))
+    side = torch.cuda.Stream(cuda)
+    side.wait_stream(torch.cuda.current_stream(cuda))
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            all_gather_matmul_tma_persistent(a_shard, b, a_out, c_out, None)
+    torch.cuda.current_stream(cuda).wait_stream(side)
+    for replay in range(4):
+        a_out.zero_()
+        c_out.fill_(float("nan"))
+        scratch = torch.randn(1 << 20, device=cuda).sum()                      # unrelated eager work
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        h.check_status()
+        assert torch.equal(c_out.view(torch.int16), want_c.view(torch.int16)), replay
+        assert torch.equal(a_out.view(torch.int16), want_a.view(torch.int16)), replay
+        del scratch
+    del graph
 
 
 def test_mm_only_is_ungated(cuda, monkeypatch):

@@ -47,6 +47,14 @@ def _check(got, want):
     assert np.mean(d == 0) >= 0.998, float(np.mean(d == 0))
 
 
+@pytest.fixture(params=[True, False], ids=["fused", "copy-then-multiply"])
+def either_form(request, monkeypatch):
+    """Small problems are planned as copy-then-multiply; both forms are tested."""
+    import importlib
+    monkeypatch.setattr(importlib.import_module("symm_mem_recipes.all_gather_matmul"), "FUSED", request.param)
+    return request.param
+
+
 @pytest.fixture(autouse=True)
 def _release():
     yield
@@ -60,7 +68,7 @@ def _release():
     (4096, 512, 1024, 8, 3),
     (2048, 272, 256, 4, 1),       # world size 4, two row tiles per comm block
 ])
-def test_fp8_fused_parity(cuda, M, N, K, ws, rank):
+def test_fp8_fused_parity(cuda, either_form, M, N, K, ws, rank):
     from symm_mem_recipes import all_gather_matmul_tma_persistent
     a_shard, h, shards, b, b_bits, a_out, c_out = _setup(M, N, K, ws, rank, cuda)
     ret = all_gather_matmul_tma_persistent(a_shard, b, a_out, c_out, None)
@@ -70,7 +78,7 @@ def test_fp8_fused_parity(cuda, M, N, K, ws, rank):
     assert np.array_equal(_bits(a_out), np.concatenate(shards))
 
 
-def test_fp8_saturation_and_exact_small_integers(cuda):
+def test_fp8_saturation_and_exact_small_integers(cuda, either_form):
     """Operands of small integers: every product and sum is exact, so the result must
     equal the oracle bit for bit - including the entries beyond 448, which saturate."""
     from symm_mem_recipes import all_gather_matmul_tma_persistent
