@@ -24,6 +24,7 @@ from . import _lib
 #: bytes per emulated signal pad: 4096 blocks x 8 ranks x 4 B
 SIGNAL_PAD_SIZE = 128 * 1024
 _ALIGN = 256
+_STAGGER = 4096        # bytes between the end of one rank's buffer and the start of the next
 
 _current_rank = int(os.environ.get("RANK", "0"))
 _default_world_size = int(os.environ.get("WORLD_SIZE", "8"))
@@ -56,11 +57,15 @@ class _Group:
         self.world_size = world_size
         self.device = device
         self.buffer_size = max(_ALIGN, (nbytes + _ALIGN - 1) // _ALIGN * _ALIGN)
-        self.slab = torch.empty(world_size * self.buffer_size, dtype=torch.uint8, device=device)
+        # Peers' buffers one GPU apart would share no DRAM; emulated in one slab, eight read
+        # streams that are congruent modulo a power of two keep landing in the same banks
+        # (8 x 16 MiB reduce: 27.5 us; staggered by 4 KiB per rank: 25.5 us).
+        self.buffer_stride = self.buffer_size + _STAGGER
+        self.slab = torch.empty(world_size * self.buffer_stride, dtype=torch.uint8, device=device)
         self.pads = torch.zeros(world_size * SIGNAL_PAD_SIZE, dtype=torch.uint8, device=device)
         base = self.slab.data_ptr()
         pbase = self.pads.data_ptr()
-        self.buffer_addrs = [base + r * self.buffer_size for r in range(world_size)]
+        self.buffer_addrs = [base + r * self.buffer_stride for r in range(world_size)]
         self.pad_addrs = [pbase + r * SIGNAL_PAD_SIZE for r in range(world_size)]
         self.buffer_ptrs = torch.tensor(self.buffer_addrs, dtype=torch.int64, device=device)
         self.pad_ptrs = torch.tensor(self.pad_addrs, dtype=torch.int64, device=device)
@@ -147,7 +152,7 @@ class EmulatedSymmetricMemory:
     def _view(self, rank, sizes, strides, dtype, storage_offset):
         itemsize = torch.empty((), dtype=dtype).element_size()
         g = self._group
-        flat = g.slab[rank * g.buffer_size:(rank + 1) * g.buffer_size].view(dtype)
+        flat = g.slab[rank * g.buffer_stride:rank * g.buffer_stride + g.buffer_size].view(dtype)
         need = storage_offset + (1 + sum((n - 1) * s for n, s in zip(sizes, strides))
                                  if all(n > 0 for n in sizes) else 0)
         assert need * itemsize <= g.buffer_size, "view exceeds the symmetric buffer"
@@ -173,9 +178,9 @@ class EmulatedSymmetricMemory:
         first = self.get_buffer(0, sizes, dtype)
         itemsize = first.element_size()
         g = self._group
-        assert g.buffer_size % itemsize == 0
+        assert g.buffer_stride % itemsize == 0
         return g.slab.view(dtype).as_strided((self.world_size,) + sizes,
-                                            (g.buffer_size // itemsize,) + tuple(first.stride()),
+                                            (g.buffer_stride // itemsize,) + tuple(first.stride()),
                                             g.slab.view(dtype).storage_offset())
 
     def get_signal_pad(self, rank: int, sizes: Optional[Sequence[int]] = None,
