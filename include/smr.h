@@ -167,6 +167,14 @@ int smr_all_gather_with_progress(const uint64_t* buffer_ptrs_dev, void* a_out_de
                                  int world_size, int64_t shard_bytes, int splits_per_rank,
                                  int num_workgroups, void* stream);
 
+/* The producer starting at the first_chunk-th chunk of its walk (0 = all of it): the
+ * chunks before are delivered by someone else, smr_ag_matmul_pull_first's workgroups
+ * for the first one.  Their flags and their part of a_out are not touched. */
+int smr_all_gather_with_progress_from(const uint64_t* buffer_ptrs_dev, void* a_out_dev,
+                                      uint32_t* progress_dev, uint32_t* counters_dev, int rank,
+                                      int world_size, int64_t shard_bytes, int splits_per_rank,
+                                      int first_chunk, int num_workgroups, void* stream);
+
 /* The same gather for a caller that does not watch the flags on the way (a GEMM queued
  * behind it in stream order): all chunks are copied together and every flag is raised at
  * the end.  Same arguments and the same final state of a_out, progress and counters as
@@ -201,6 +209,24 @@ int smr_ag_matmul(const void* a_shard_dev, const void* a_out_dev, const void* b_
  * Counterpart of the index arithmetic at triton_all_gather_matmul.py:125-174. */
 int smr_ag_matmul_schedule(int M, int N, int K, int rank, int world_size, int comm_block_m,
                            int gated, int32_t* out_records, int max_tiles);
+
+/* smr_ag_matmul (elem_bytes 2) or smr_ag_matmul_fp8 (elem_bytes 1), gated, whose
+ * workgroups copy the first remote chunk themselves.  Half the grid of a gated launch
+ * starts on the first remote comm block and would wait for the producer to deliver it;
+ * those workgroups are idle compute units, so they pull the chunk from
+ * buffer_ptrs_dev[rank + 1] into a_out (a slice each), the last one raises
+ * progress[(rank + 1) * splits], and the producer is started at its second chunk
+ * (smr_all_gather_with_progress_from, first_chunk = 1).  The reference's copy engines
+ * deliver every chunk (triton_all_gather_matmul.py:41-55); this is the part of that loop
+ * the consumer takes over when the copy has to run on compute units.
+ *   pull_counters_dev  uint32 [2], zero on entry, zero again when the kernel is through
+ * Returns the number of pulling workgroups (> 0: start the producer at chunk 1), 0 when
+ * too few workgroups would wait for pulling to pay (plain gated launch: start the producer
+ * at chunk 0), or a negative SMR_E_* code. */
+int smr_ag_matmul_pull_first(const void* a_shard_dev, void* a_out_dev, const void* b_nk_dev, void* c_dev,
+                             uint32_t* progress_dev, uint32_t* pull_counters_dev,
+                             const uint64_t* buffer_ptrs_dev, int elem_bytes, int M, int N, int K, int rank,
+                             int world_size, int comm_block_m, uint32_t* status, void* stream);
 
 /* The same GEMM with e4m3fn (OCP FP8) operands and result, fp32 accumulation: the
  * reference's FP8_OUTPUT switch (triton_all_gather_matmul.py:115,123,188,311).  The cast of

@@ -685,11 +685,69 @@ __device__ __forceinline__ void run_tile_fp8(const TileContext& cx, const TileRe
   }
 }
 
+// The first remote chunk, pulled by the GEMM's own workgroups before their first tile.
+// A gated launch puts as many workgroups on the first remote comm block as on the
+// local one, and a producer that owns an eighth of the GPU needs a third of a tile's
+// time to deliver that chunk; every workgroup has the same number of tiles, so the
+// launch ends late by that wait.  Instead the whole grid copies the chunk first (a
+// slice per workgroup, taken by ticket; 32 MiB in about 15 us), the last workgroup to
+// finish raises the flag, and the producer starts at the second chunk, which it
+// delivers long before the second pass.
+struct PullFirst {
+  const uint64_t* buffer_ptrs;   // the ranks' shard addresses (device array); nullptr = off
+  uint8_t* dst;                  // the chunk's place in the gathered operand
+  uint32_t* flag;                // its progress flag
+  uint32_t* counters;            // [0] tickets, [1] arrivals; zero on entry, zero again on exit
+  int64_t vecs;                  // 16-byte vectors in the chunk
+  int src_rank, comm_block, helpers;
+};
+
+typedef __attribute__((address_space(1))) u32x4 GlobalVec;
+
+__device__ __forceinline__ void pull_first_chunk(const PullFirst& pf, uint32_t lds0) {
+  // one ticket per workgroup, handed to its threads through the (still unused) tile ring
+  if (threadIdx.x == 0) {
+    const uint32_t t = __hip_atomic_fetch_add(&pf.counters[0], 1u, __ATOMIC_RELAXED, kScope);
+    *reinterpret_cast<__attribute__((address_space(3))) uint32_t*>((uintptr_t)lds0) = t;
+  }
+  __syncthreads();
+  const uint32_t ticket = *reinterpret_cast<__attribute__((address_space(3))) uint32_t*>((uintptr_t)lds0);
+  __syncthreads();
+  const GlobalVec* src = (const GlobalVec*)(uintptr_t)pf.buffer_ptrs[pf.src_rank];
+  GlobalVec* dst = (GlobalVec*)(uintptr_t)pf.dst;
+  constexpr int kInFlight = 16;
+  const int64_t stride = (int64_t)pf.helpers * kGemmThreads;
+  int64_t i = (int64_t)ticket * kGemmThreads + threadIdx.x;
+  for (; i + (kInFlight - 1) * stride < pf.vecs; i += kInFlight * stride) {
+    u32x4 v[kInFlight];
+#pragma unroll
+    for (int u = 0; u < kInFlight; ++u) v[u] = __builtin_nontemporal_load(src + i + u * stride);
+#pragma unroll
+    for (int u = 0; u < kInFlight; ++u)
+      asm volatile("global_store_dwordx4 %0, %1, off sc1" : : "v"(dst + i + u * stride), "v"(v[u]) : "memory");
+  }
+  for (; i < pf.vecs; i += stride) {
+    const u32x4 v = __builtin_nontemporal_load(src + i);
+    asm volatile("global_store_dwordx4 %0, %1, off sc1" : : "v"(dst + i), "v"(v) : "memory");
+  }
+  // written through: once acknowledged the slice is where every XCD reads it
+  wait_stores_acknowledged();
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    const uint32_t prev = __hip_atomic_fetch_add(&pf.counters[1], 1u, __ATOMIC_RELAXED, kScope);
+    if (prev + 1u == (uint32_t)pf.helpers) {
+      __hip_atomic_store(&pf.counters[0], 0u, __ATOMIC_RELAXED, kScope);
+      __hip_atomic_store(&pf.counters[1], 0u, __ATOMIC_RELAXED, kScope);
+      __hip_atomic_store(pf.flag, 1u, __ATOMIC_RELAXED, kScope);
+    }
+  }
+}
+
 template <int BM, int BN, bool FP8 = false>
 __global__ __launch_bounds__(kGemmThreads, 1) void ag_matmul_kernel(
     const uint8_t* __restrict__ a_shard, const uint8_t* __restrict__ a_out,
     const uint8_t* __restrict__ b_nk, uint8_t* __restrict__ c, const uint32_t* __restrict__ progress,
-    GemmSchedule s, uint64_t limit_ticks, uint32_t* status, uint64_t* trace) {
+    GemmSchedule s, uint64_t limit_ticks, uint32_t* status, uint64_t* trace, PullFirst pf) {
   __shared__ __attribute__((aligned(1024))) uint8_t lds[GemmTile<BM, BN>::kLdsBytes];
 
   TileContext cx;
@@ -714,6 +772,7 @@ __global__ __launch_bounds__(kGemmThreads, 1) void ag_matmul_kernel(
   bool have = next_tile(s, blockIdx.x, step, tile);
   const uint8_t* a_base = nullptr;
   const uint8_t* b_base = nullptr;
+  if (pf.buffer_ptrs != nullptr) pull_first_chunk(pf, cx.lds0);
   if (have) {
     a_base = a_rows_of(tile);
     b_base = b_nk + (int64_t)tile.col0 * cx.row_stride;
@@ -925,18 +984,35 @@ static GemmSchedule make_schedule(int M, int N, int K, int rank, int world_size,
 
 extern "C" {
 
-int smr_ag_matmul(const void* a_shard_dev, const void* a_out_dev, const void* b_nk_dev, void* c_dev,
-                  const uint32_t* progress_dev, int M, int N, int K, int rank, int world_size,
-                  int comm_block_m, uint32_t* status, void* stream) {
+// Workgroups of a gated launch whose first tile lies in the first remote comm block of
+// the ring order: the ones that would start with a wait.
+static int first_chunk_waiters(const smr::GemmSchedule& s, int comm_block) {
   using namespace smr;
-  const char* why;
-  if (int rc = validate(M, N, K, rank, world_size, comm_block_m, &why)) return fail(rc, why);
+  int n = 0;
+  for (int wg = 0; wg < s.grid; ++wg) {
+    TileRef t;
+    int step = 0;
+    if (next_tile(s, wg, step, t) && !t.local && t.comm_block == comm_block) ++n;
+  }
+  return n;
+}
+
+// With fewer workgroups waiting for the first remote chunk the copy is left to the producer.
+constexpr int kMinPullHelpers = 48;
+
+static int launch_gemm(int elem_bytes, const void* a_shard_dev, const void* a_out_dev, const void* b_nk_dev,
+                       void* c_dev, const uint32_t* progress_dev, int M, int N, int K, int rank,
+                       int world_size, int comm_block_m, uint32_t* status, void* stream,
+                       const uint64_t* buffer_ptrs_dev, uint32_t* pull_counters_dev, int* helpers_out) {
+  using namespace smr;
   if (a_shard_dev == nullptr || a_out_dev == nullptr || b_nk_dev == nullptr || c_dev == nullptr)
-    return fail(SMR_E_INVALID, "smr_ag_matmul: null pointer");
+    return fail(SMR_E_INVALID, elem_bytes == 1 ? "smr_ag_matmul_fp8: null pointer" : "smr_ag_matmul: null pointer");
   if ((reinterpret_cast<uintptr_t>(a_shard_dev) | reinterpret_cast<uintptr_t>(a_out_dev) |
        reinterpret_cast<uintptr_t>(b_nk_dev) | reinterpret_cast<uintptr_t>(c_dev)) & 15u)
-    return fail(SMR_E_INVALID, "smr_ag_matmul: operands must be 16-byte aligned");
-  const GemmSchedule s = make_schedule(M, N, K, rank, world_size, comm_block_m, cu_count(), progress_dev != nullptr);
+    return fail(SMR_E_INVALID, elem_bytes == 1 ? "smr_ag_matmul_fp8: operands must be 16-byte aligned"
+                                               : "smr_ag_matmul: operands must be 16-byte aligned");
+  const GemmSchedule s = make_schedule(M, N, K, rank, world_size, comm_block_m, cu_count(),
+                                       progress_dev != nullptr, elem_bytes);
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
   const uint8_t* a0 = reinterpret_cast<const uint8_t*>(a_shard_dev);
   const uint8_t* a1 = reinterpret_cast<const uint8_t*>(a_out_dev);
@@ -944,16 +1020,71 @@ int smr_ag_matmul(const void* a_shard_dev, const void* a_out_dev, const void* b_
   uint8_t* c = reinterpret_cast<uint8_t*>(c_dev);
   const uint64_t lim = spin_limit_ticks();
   uint64_t* tb = trace_buffer(kTraceProducerWords + kTraceGemmWords);
-  if (s.BM == 256 && s.BN == 256)
+  PullFirst pf = {};
+  if (buffer_ptrs_dev != nullptr && world_size > 1) {
+    // the producer's first chunk: split 0 of rank + 1
+    const int splits = (M / world_size) / comm_block_m;
+    const int src_rank = (rank + 1) % world_size;
+    const int waiters = first_chunk_waiters(s, src_rank * splits);
+    const int helpers = s.grid;
+    if (waiters >= kMinPullHelpers) {
+      const int64_t chunk_bytes = (int64_t)comm_block_m * K * elem_bytes;
+      pf.buffer_ptrs = buffer_ptrs_dev;
+      pf.dst = const_cast<uint8_t*>(a1) + (int64_t)src_rank * splits * chunk_bytes;
+      pf.flag = const_cast<uint32_t*>(progress_dev) + src_rank * splits;
+      pf.counters = pull_counters_dev;
+      pf.vecs = chunk_bytes / 16;
+      pf.src_rank = src_rank;
+      pf.comm_block = src_rank * splits;
+      pf.helpers = helpers;
+    }
+  }
+  if (helpers_out != nullptr) *helpers_out = pf.helpers;
+  if (elem_bytes == 1)
+    hipLaunchKernelGGL((ag_matmul_kernel<256, 256, true>), dim3(s.grid), dim3(kGemmThreads), 0, st, a0, a1, b,
+                       c, progress_dev, s, lim, status, tb, pf);
+  else if (s.BM == 256 && s.BN == 256)
     hipLaunchKernelGGL((ag_matmul_kernel<256, 256>), dim3(s.grid), dim3(kGemmThreads), 0, st, a0, a1, b,
-                       c, progress_dev, s, lim, status, tb);
+                       c, progress_dev, s, lim, status, tb, pf);
   else if (s.BM == 256)
     hipLaunchKernelGGL((ag_matmul_kernel<256, 128>), dim3(s.grid), dim3(kGemmThreads), 0, st, a0, a1, b,
-                       c, progress_dev, s, lim, status, tb);
+                       c, progress_dev, s, lim, status, tb, pf);
   else
     hipLaunchKernelGGL((ag_matmul_kernel<128, 128>), dim3(s.grid), dim3(kGemmThreads), 0, st, a0, a1, b,
-                       c, progress_dev, s, lim, status, tb);
+                       c, progress_dev, s, lim, status, tb, pf);
   return check_hip(hipGetLastError(), "smr_ag_matmul launch");
+}
+
+static int validate_fp8(int M, int N, int K, int rank, int world_size, int comm_block_m, const char** why);
+
+int smr_ag_matmul(const void* a_shard_dev, const void* a_out_dev, const void* b_nk_dev, void* c_dev,
+                  const uint32_t* progress_dev, int M, int N, int K, int rank, int world_size,
+                  int comm_block_m, uint32_t* status, void* stream) {
+  using namespace smr;
+  const char* why;
+  if (int rc = validate(M, N, K, rank, world_size, comm_block_m, &why)) return fail(rc, why);
+  return launch_gemm(2, a_shard_dev, a_out_dev, b_nk_dev, c_dev, progress_dev, M, N, K, rank, world_size,
+                     comm_block_m, status, stream, nullptr, nullptr, nullptr);
+}
+
+int smr_ag_matmul_pull_first(const void* a_shard_dev, void* a_out_dev, const void* b_nk_dev, void* c_dev,
+                             uint32_t* progress_dev, uint32_t* pull_counters_dev,
+                             const uint64_t* buffer_ptrs_dev, int elem_bytes, int M, int N, int K, int rank,
+                             int world_size, int comm_block_m, uint32_t* status, void* stream) {
+  using namespace smr;
+  const char* why;
+  if (elem_bytes != 1 && elem_bytes != 2)
+    return fail(SMR_E_INVALID, "smr_ag_matmul_pull_first: elem_bytes must be 2 (bf16) or 1 (e4m3fn)");
+  if (int rc = elem_bytes == 1 ? validate_fp8(M, N, K, rank, world_size, comm_block_m, &why)
+                               : validate(M, N, K, rank, world_size, comm_block_m, &why))
+    return fail(rc, why);
+  if (progress_dev == nullptr || pull_counters_dev == nullptr || buffer_ptrs_dev == nullptr)
+    return fail(SMR_E_INVALID, "smr_ag_matmul_pull_first: progress, counters and buffer_ptrs are required");
+  int helpers = 0;
+  if (int rc = launch_gemm(elem_bytes, a_shard_dev, a_out_dev, b_nk_dev, c_dev, progress_dev, M, N, K, rank,
+                           world_size, comm_block_m, status, stream, buffer_ptrs_dev, pull_counters_dev, &helpers))
+    return rc;
+  return helpers;
 }
 
 static void fill_plan(int M, int N, int K, int world_size, int comm_block_m, int elem_bytes, int32_t* out5);
@@ -975,19 +1106,8 @@ int smr_ag_matmul_fp8(const void* a_shard_dev, const void* a_out_dev, const void
   using namespace smr;
   const char* why;
   if (int rc = validate_fp8(M, N, K, rank, world_size, comm_block_m, &why)) return fail(rc, why);
-  if (a_shard_dev == nullptr || a_out_dev == nullptr || b_nk_dev == nullptr || c_dev == nullptr)
-    return fail(SMR_E_INVALID, "smr_ag_matmul_fp8: null pointer");
-  if ((reinterpret_cast<uintptr_t>(a_shard_dev) | reinterpret_cast<uintptr_t>(a_out_dev) |
-       reinterpret_cast<uintptr_t>(b_nk_dev) | reinterpret_cast<uintptr_t>(c_dev)) & 15u)
-    return fail(SMR_E_INVALID, "smr_ag_matmul_fp8: operands must be 16-byte aligned");
-  const GemmSchedule s = make_schedule(M, N, K, rank, world_size, comm_block_m, cu_count(),
-                                       progress_dev != nullptr, 1);
-  hipLaunchKernelGGL((ag_matmul_kernel<256, 256, true>), dim3(s.grid), dim3(kGemmThreads), 0,
-                     reinterpret_cast<hipStream_t>(stream), reinterpret_cast<const uint8_t*>(a_shard_dev),
-                     reinterpret_cast<const uint8_t*>(a_out_dev), reinterpret_cast<const uint8_t*>(b_nk_dev),
-                     reinterpret_cast<uint8_t*>(c_dev), progress_dev, s, spin_limit_ticks(), status,
-                     trace_buffer(kTraceProducerWords + kTraceGemmWords));
-  return check_hip(hipGetLastError(), "smr_ag_matmul_fp8 launch");
+  return launch_gemm(1, a_shard_dev, a_out_dev, b_nk_dev, c_dev, progress_dev, M, N, K, rank, world_size,
+                     comm_block_m, status, stream, nullptr, nullptr, nullptr);
 }
 
 int smr_ag_matmul_plan_fp8(int M, int N, int K, int world_size, int comm_block_m, int32_t* out5) {

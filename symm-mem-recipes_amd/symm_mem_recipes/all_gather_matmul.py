@@ -26,6 +26,9 @@ MAX_PRODUCER_WORKGROUPS = None
 PRODUCER_PACING = None
 #: None = the plan decides between the fused launch and copy-then-multiply; True / False force one.
 FUSED = None
+#: A fused launch lets the GEMM's waiting workgroups copy the first remote chunk themselves
+#: (smr_ag_matmul_pull_first); False leaves every chunk to the producer.
+PULL_FIRST = True
 
 
 def all_gather_with_progress(output: torch.Tensor, inp: torch.Tensor, progress: torch.Tensor,
@@ -57,11 +60,19 @@ def all_gather_with_progress(output: torch.Tensor, inp: torch.Tensor, progress: 
 
 
 def _launch_producer(symm_mem, output, inp, progress, counters, splits_per_rank, num_workgroups,
-                     stream_handle, at_once: bool = False) -> None:
+                     stream_handle, at_once: bool = False, first_chunk: int = 0) -> None:
     """The producer kernel on the given stream; ``counters`` (one zeroed int32 per
     chunk) are its arrival counters.  ``at_once`` copies all chunks together and raises
-    the flags at the end, for a consumer that is queued behind the copy."""
+    the flags at the end, for a consumer that is queued behind the copy; ``first_chunk``
+    starts the walk at a later chunk (the ones before are delivered by the consumer)."""
     lib = _lib.load()
+    if first_chunk:
+        rc = lib.smr_all_gather_with_progress_from(
+            symm_mem.buffer_ptrs_dev, output.data_ptr(), progress.data_ptr(), counters.data_ptr(),
+            symm_mem.rank, symm_mem.world_size, inp.numel() * inp.element_size(), int(splits_per_rank),
+            int(first_chunk), int(num_workgroups), stream_handle)
+        _lib.check(rc, "all_gather_with_progress")
+        return
     rc = (lib.smr_all_gather_at_once if at_once else lib.smr_all_gather_with_progress)(
         symm_mem.buffer_ptrs_dev, output.data_ptr(), progress.data_ptr(), counters.data_ptr(),
         symm_mem.rank, symm_mem.world_size, inp.numel() * inp.element_size(), int(splits_per_rank),
@@ -116,8 +127,8 @@ def all_gather_matmul_tma_persistent(a_shard: torch.Tensor, b: torch.Tensor, a_o
     else:
         # flags and the producer's arrival counters, zeroed by one fill ahead of both kernels
         chunks = world_size * splits_per_rank
-        flags = torch.zeros(2 * chunks, dtype=torch.int32, device=device)
-        progress, counters = flags[:chunks], flags[chunks:]
+        flags = torch.zeros(2 * chunks + 2, dtype=torch.int32, device=device)
+        progress, counters, pull_counters = flags[:chunks], flags[chunks:2 * chunks], flags[2 * chunks:]
         progress_ptr = progress.data_ptr()
         symm_mem.barrier(0)
         backend = _get_backend_stream()
@@ -142,15 +153,25 @@ def all_gather_matmul_tma_persistent(a_shard: torch.Tensor, b: torch.Tensor, a_o
     # The GEMM goes first: its first tiles are local rows and need no flag, so the
     # producer's launch latency is hidden behind them instead of delaying the GEMM.
     # (The backend stream waits for what preceded the GEMM, not for the GEMM.)
-    gemm = lib.smr_ag_matmul_fp8 if fp8 else lib.smr_ag_matmul
-    rc = gemm(a_shard.data_ptr(), a_out.data_ptr(), b.data_ptr(), c_out.data_ptr(),
-              progress_ptr, M, N, K, rank, world_size, COMM_BLOCK_SIZE_M, status_ptr,
-              current.cuda_stream)
-    _lib.check(rc, "all_gather_matmul")
+    pulled = 0
+    if not mm_only and not sequential and PULL_FIRST:
+        # the workgroups that would wait for the first remote chunk copy it themselves
+        pulled = lib.smr_ag_matmul_pull_first(
+            a_shard.data_ptr(), a_out.data_ptr(), b.data_ptr(), c_out.data_ptr(), progress_ptr,
+            pull_counters.data_ptr(), symm_mem.buffer_ptrs_dev, 1 if fp8 else 2, M, N, K, rank, world_size,
+            COMM_BLOCK_SIZE_M, status_ptr, current.cuda_stream)
+        if pulled < 0:
+            _lib.check(pulled, "all_gather_matmul")
+    else:
+        gemm = lib.smr_ag_matmul_fp8 if fp8 else lib.smr_ag_matmul
+        rc = gemm(a_shard.data_ptr(), a_out.data_ptr(), b.data_ptr(), c_out.data_ptr(),
+                  progress_ptr, M, N, K, rank, world_size, COMM_BLOCK_SIZE_M, status_ptr,
+                  current.cuda_stream)
+        _lib.check(rc, "all_gather_matmul")
     if not mm_only and not sequential:
         _lib.check(lib.smr_set_gather_pacing(int(pacing[0]), int(pacing[1])), "all_gather_matmul")
         _launch_producer(symm_mem, a_out, a_shard, progress, counters, splits_per_rank, producer_wgs,
-                         backend.cuda_stream)
+                         backend.cuda_stream, first_chunk=1 if pulled > 0 else 0)
         current.wait_stream(backend)
     return c_out
 

@@ -246,6 +246,72 @@ def test_fused_launch_replays_from_a_graph(cuda, either_form, M, N, K):
     del graph
 
 
+@pytest.mark.parametrize("M,N,K,rank,splits", [(16384, 2048, 256, 0, 1), (16384, 2048, 192, 5, 1), (16384, 3072, 128, 7, 2)])
+def test_first_chunk_pulled_by_the_gemm(cuda, lib, force_fused, monkeypatch, M, N, K, rank, splits):
+    """Enough workgroups would wait for the first remote chunk that the GEMM's grid copies
+    it itself and the producer starts at its second chunk: same product, bit for bit, as
+    with every chunk left to the producer; gathered operand complete; all flags raised."""
+    import importlib
+    agm = importlib.import_module("symm_mem_recipes.all_gather_matmul")
+    ws = 8
+    a_shard, h, shards, b, b_bits, a_out, c_out = _setup(M, N, K, ws, rank, cuda)
+    outs = []
+    for pull in (False, True, True):
+        monkeypatch.setattr(agm, "PULL_FIRST", pull)
+        a_out.zero_()
+        c = torch.full_like(c_out, float("nan"))
+        agm.all_gather_matmul_tma_persistent(a_shard, b, a_out, c, None, splits_per_rank=splits)
+        h.check_status()
+        assert np.array_equal(_t_bits(a_out), np.concatenate(shards))
+        outs.append(c)
+    _check(_t_bits(outs[0]), O.ag_matmul_ref(shards, b_bits))
+    assert torch.equal(outs[0].view(torch.int16), outs[1].view(torch.int16))
+    assert torch.equal(outs[0].view(torch.int16), outs[2].view(torch.int16))
+    # through the C ABI: it reports the pulling workgroups, leaves its two counters zero and
+    # raises the first remote chunk's flag itself (no producer is started here, so only that one)
+    chunks = ws * splits
+    state = torch.zeros(chunks + 2, dtype=torch.int32, device=cuda)
+    state[:chunks] = 1                                    # the other chunks are in place already
+    first = ((rank + 1) % ws) * splits
+    state[first] = 0
+    rows = M // ws // splits
+    a_out[first * rows:(first + 1) * rows].zero_()
+    pulled = lib.smr_ag_matmul_pull_first(a_shard.data_ptr(), a_out.data_ptr(), b.data_ptr(), c_out.data_ptr(),
+                                          state.data_ptr(), state[chunks:].data_ptr(), h.buffer_ptrs_dev, 2,
+                                          M, N, K, rank, ws, rows, h.status.data_ptr(),
+                                          torch.cuda.current_stream(cuda).cuda_stream)
+    torch.cuda.synchronize()
+    h.check_status()
+    assert pulled == lib.smr_ag_matmul_grid(M, N, K, ws, rows, 1) > 0
+    assert state.cpu().tolist() == [1] * chunks + [0, 0]
+    assert np.array_equal(_t_bits(a_out), np.concatenate(shards))
+    assert torch.equal(c_out.view(torch.int16), outs[0].view(torch.int16))
+
+
+def test_small_launch_leaves_the_first_chunk_to_the_producer(cuda, lib):
+    """Few waiting workgroups: smr_ag_matmul_pull_first runs as the plain gated GEMM and says so."""
+    M, N, K, ws, rank = 2048, 256, 256, 8, 1
+    a_shard, h, shards, b, b_bits, a_out, c_out = _setup(M, N, K, ws, rank, cuda)
+    a_out.copy_(_bits_t(np.concatenate(shards)))
+    state = torch.ones(ws + 2, dtype=torch.int32, device=cuda)
+    state[ws:] = 0
+    pulled = lib.smr_ag_matmul_pull_first(a_shard.data_ptr(), a_out.data_ptr(), b.data_ptr(), c_out.data_ptr(),
+                                          state.data_ptr(), state[ws:].data_ptr(), h.buffer_ptrs_dev, 2,
+                                          M, N, K, rank, ws, M // ws, h.status.data_ptr(),
+                                          torch.cuda.current_stream(cuda).cuda_stream)
+    torch.cuda.synchronize()
+    h.check_status()
+    assert pulled == 0
+    _check(_t_bits(c_out), O.ag_matmul_ref(shards, b_bits))
+    null = lib.smr_ag_matmul_pull_first(a_shard.data_ptr(), a_out.data_ptr(), b.data_ptr(), c_out.data_ptr(),
+                                        None, state[ws:].data_ptr(), h.buffer_ptrs_dev, 2, M, N, K, rank, ws,
+                                        M // ws, h.status.data_ptr(), None)
+    assert null == -1
+    assert lib.smr_ag_matmul_pull_first(a_shard.data_ptr(), a_out.data_ptr(), b.data_ptr(), c_out.data_ptr(),
+                                        state.data_ptr(), state[ws:].data_ptr(), h.buffer_ptrs_dev, 4, M, N, K,
+                                        rank, ws, M // ws, h.status.data_ptr(), None) == -1
+
+
 def test_mm_only_is_ungated(cuda, monkeypatch):
     """mm_only multiplies what the buffers already hold, as rank 0, with no flags
     (triton_all_gather_matmul.py:222-224,246-247)."""

@@ -41,7 +41,9 @@ def _k_loops(lines):
         if re.search(r"s_waitcnt vmcnt\((8|4)\)", ln):
             start = max(j for j in range(i) if re.match(r"^\.LBB\d+_\d+:", lines[j]))
             end = next(j for j in range(i, len(lines)) if "s_cbranch" in lines[j])
-            loops.append(lines[start:end + 1])
+            body = lines[start:end + 1]
+            if any("v_mfma_" in x for x in body):           # (the copy loop of the pulled first chunk waits too)
+                loops.append(body)
     return loops
 
 
