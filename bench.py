@@ -177,6 +177,30 @@ def bench_reduce_rotating(size_kib, dev, dtype_name="bf16", write_all=False, acc
     return res
 
 
+def _time_interleaved(fns, iters, warm, pre=None):
+    """Median device time in microseconds of each fn in `fns`, the calls taken in turn
+    (a, b, c, a, b, c, ...): variants measured one block after another see different
+    clocks, because the part's power management reacts to the last milliseconds of load."""
+    import torch
+    for _ in range(warm):
+        for fn in fns:
+            fn()
+    torch.cuda.synchronize()
+    ts = [[] for _ in fns]
+    for _ in range(iters):
+        for k, fn in enumerate(fns):
+            if pre is not None:
+                pre()
+            a = torch.cuda.Event(enable_timing=True)
+            b = torch.cuda.Event(enable_timing=True)
+            a.record()
+            fn()
+            b.record()
+            torch.cuda.synchronize()
+            ts[k].append(a.elapsed_time(b) * 1e3)
+    return [_median(t) for t in ts]
+
+
 def bench_ag_matmul(dev, gated=True):
     import torch
     from symm_mem_recipes import EmulatedSymmetricMemory as SM, all_gather_matmul_tma_persistent
@@ -193,12 +217,13 @@ def bench_ag_matmul(dev, gated=True):
     c = torch.empty(M, N, dtype=torch.bfloat16, device=dev)
     flush = torch.empty(1 << 28, dtype=torch.int32, device=dev)      # 1 GiB > last-level cache
     flops = 2.0 * M * N * K
-    us_ungated = _time_events(lambda: all_gather_matmul_tma_persistent(a_shard, b, a_out, c, None, mm_only=True),
-                              25, 20, pre=flush.zero_)
-    us_gated = _time_events(lambda: all_gather_matmul_tma_persistent(a_shard, b, a_out, c, None),
-                            25, 20, pre=flush.zero_) if gated else float("nan")
+    fns = [lambda: all_gather_matmul_tma_persistent(a_shard, b, a_out, c, None, mm_only=True),
+           lambda: torch.matmul(a_out, b.T, out=c)]
+    if gated:
+        fns.append(lambda: all_gather_matmul_tma_persistent(a_shard, b, a_out, c, None))
+    us = _time_interleaved(fns, 25, 10, pre=flush.zero_)
+    us_ungated, us_lib, us_gated = us[0], us[1], (us[2] if gated else float("nan"))
     h.check_status()
-    us_lib = _time_events(lambda: torch.matmul(a_out, b.T, out=c), 25, 20, pre=flush.zero_)
     SM.release()
     return dict(workload="all-gather matmul M=16384 N=3584 K=8192 bf16, 8 shards of [2048, 8192], rank 0",
                 flops=flops, us_gated=us_gated, us_ungated=us_ungated,
@@ -229,10 +254,9 @@ def bench_ag_matmul_fp8(dev):
     c = torch.empty(M, N, dtype=torch.uint8, device=dev).view(f8)
     flush = torch.empty(1 << 28, dtype=torch.int32, device=dev)
     flops = 2.0 * M * N * K
-    us_ungated = _time_events(lambda: all_gather_matmul_tma_persistent(a_shard, b, a_out, c, None, mm_only=True),
-                              25, 20, pre=flush.zero_)
-    us_gated = _time_events(lambda: all_gather_matmul_tma_persistent(a_shard, b, a_out, c, None),
-                            25, 20, pre=flush.zero_)
+    us_ungated, us_gated = _time_interleaved(
+        [lambda: all_gather_matmul_tma_persistent(a_shard, b, a_out, c, None, mm_only=True),
+         lambda: all_gather_matmul_tma_persistent(a_shard, b, a_out, c, None)], 25, 10, pre=flush.zero_)
     h.check_status()
     res = dict(workload="all-gather matmul M=16384 N=3584 K=8192 e4m3fn in and out, 8 shards of [2048, 8192], rank 0",
                flops=flops, us_gated=us_gated, us_ungated=us_ungated,
