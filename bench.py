@@ -35,6 +35,7 @@ MFMA_FP8_PEAK_TFLOPS = 5000.0   # MI355X dense fp8, published
 # run cannot hold the gated launch (it serialises kernels); the gated GEMM reads and writes
 # the same tiles in the same order.
 MEASURED_GEMM_TRAFFIC_BYTES = 1618400051
+MEASURED_GEMM_FP8_TRAFFIC_BYTES = 799597261   # the same two counter runs of `bench.py --gemm-only --fp8`
 WS = 8
 
 
@@ -235,7 +236,7 @@ def bench_ag_matmul(dev, gated=True):
                 torch_matmul_us=us_lib, torch_matmul_tflops=flops / us_lib / 1e6)
 
 
-def bench_ag_matmul_fp8(dev):
+def bench_ag_matmul_fp8(dev, gated=True):
     """The same problem with e4m3fn operands and result (the reference's FP8_OUTPUT switch)."""
     import torch
     from symm_mem_recipes import EmulatedSymmetricMemory as SM, all_gather_matmul_tma_persistent
@@ -254,9 +255,11 @@ def bench_ag_matmul_fp8(dev):
     c = torch.empty(M, N, dtype=torch.uint8, device=dev).view(f8)
     flush = torch.empty(1 << 28, dtype=torch.int32, device=dev)
     flops = 2.0 * M * N * K
-    us_ungated, us_gated = _time_interleaved(
-        [lambda: all_gather_matmul_tma_persistent(a_shard, b, a_out, c, None, mm_only=True),
-         lambda: all_gather_matmul_tma_persistent(a_shard, b, a_out, c, None)], 25, 10, pre=flush.zero_)
+    fns = [lambda: all_gather_matmul_tma_persistent(a_shard, b, a_out, c, None, mm_only=True)]
+    if gated:
+        fns.append(lambda: all_gather_matmul_tma_persistent(a_shard, b, a_out, c, None))
+    us = _time_interleaved(fns, 25, 10, pre=flush.zero_)
+    us_ungated, us_gated = us[0], (us[1] if gated else float("nan"))
     h.check_status()
     res = dict(workload="all-gather matmul M=16384 N=3584 K=8192 e4m3fn in and out, 8 shards of [2048, 8192], rank 0",
                flops=flops, us_gated=us_gated, us_ungated=us_ungated,
@@ -264,7 +267,7 @@ def bench_ag_matmul_fp8(dev):
                gating_overhead=us_gated / us_ungated - 1.0,
                roofline={"bound": "mfma", "achieved": flops / us_gated / 1e6, "peak": MFMA_FP8_PEAK_TFLOPS,
                          "unit": "TFLOP/s", "frac": flops / us_gated / 1e6 / MFMA_FP8_PEAK_TFLOPS,
-                         "traffic": None})
+                         "traffic": MEASURED_GEMM_FP8_TRAFFIC_BYTES})
     try:                                            # the library's fp8 GEMM of the same operands (bf16 result)
         one = torch.ones((), device=dev)
         us_lib = _time_events(lambda: torch._scaled_mm(a_out, b.T, scale_a=one, scale_b=one,
@@ -405,6 +408,7 @@ def main():
                     help="only the ungated GEMM and the library matmul of the same operands: the run to "
                          "collect hardware counters on (a counter run serialises kernels, and a gated GEMM "
                          "whose producer cannot run beside it only times out)")
+    ap.add_argument("--fp8", action="store_true", help="with --gemm-only: the e4m3fn GEMM instead of the bf16 one")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on exactly one GPU (the 8 ranks are emulated in one "
@@ -419,7 +423,7 @@ def main():
     torch.cuda.set_device(dev)
 
     if args.gemm_only:
-        print(json.dumps(bench_ag_matmul(dev, gated=False)))
+        print(json.dumps(bench_ag_matmul_fp8(dev, gated=False) if args.fp8 else bench_ag_matmul(dev, gated=False)))
         return
 
     r = bench_reduce(args.size_mib, args.steps, args.warmup, dev)
