@@ -78,6 +78,38 @@ def test_fp8_fused_parity(cuda, either_form, M, N, K, ws, rank):
     assert np.array_equal(_bits(a_out), np.concatenate(shards))
 
 
+def test_fp8_first_chunk_pulled_by_the_gemm(cuda, lib, monkeypatch):
+    """A launch wide enough that the grid copies the first remote chunk itself: same codes
+    as with every chunk left to the producer, gathered operand complete."""
+    import importlib
+    agm = importlib.import_module("symm_mem_recipes.all_gather_matmul")
+    monkeypatch.setattr(agm, "FUSED", True)
+    M, N, K, ws, rank = 16384, 2048, 256, 8, 6
+    a_shard, h, shards, b, b_bits, a_out, c_out = _setup(M, N, K, ws, rank, cuda)
+    outs = []
+    for pull in (False, True):
+        monkeypatch.setattr(agm, "PULL_FIRST", pull)
+        a_out.view(torch.uint8).zero_()
+        c = torch.full_like(c_out.view(torch.uint8), 0x7F).view(torch.float8_e4m3fn)
+        agm.all_gather_matmul_tma_persistent(a_shard, b, a_out, c, None)
+        h.check_status()
+        assert np.array_equal(_bits(a_out), np.concatenate(shards))
+        outs.append(_bits(c))
+    _check(outs[0], O.ag_matmul_ref_fp8(shards, b_bits))
+    assert np.array_equal(outs[0], outs[1])
+    state = torch.zeros(ws + 2, dtype=torch.int32, device=cuda)
+    state[:ws] = 1
+    state[(rank + 1) % ws] = 0
+    pulled = lib.smr_ag_matmul_pull_first(a_shard.data_ptr(), a_out.data_ptr(), b.data_ptr(), c_out.data_ptr(),
+                                          state.data_ptr(), state[ws:].data_ptr(), h.buffer_ptrs_dev, 1,
+                                          M, N, K, rank, ws, M // ws, h.status.data_ptr(),
+                                          torch.cuda.current_stream(cuda).cuda_stream)
+    torch.cuda.synchronize()
+    h.check_status()
+    assert pulled > 0 and state.cpu().tolist() == [1] * ws + [0, 0]
+    assert np.array_equal(_bits(c_out), outs[0])
+
+
 def test_fp8_saturation_and_exact_small_integers(cuda, either_form):
     """Operands of small integers: every product and sum is exact, so the result must
     equal the oracle bit for bit - including the entries beyond 448, which saturate."""
