@@ -251,6 +251,13 @@ int smr_ag_matmul_plan_fp8(int M, int N, int K, int world_size, int comm_block_m
  * engines cost no SMs. */
 int smr_ag_matmul_plan(int M, int N, int K, int world_size, int comm_block_m, int32_t* out5);
 
+/* 1: the gated GEMM issues an acquire fence (cache invalidate) behind every flag wait, as a
+ * literal reading of wait_signal + the loads that follow (triton_all_gather_matmul.py:72-95,
+ * 170-174) asks for.  0 (default): flag poll past the caches and a workgroup barrier only;
+ * the rows of a comm block cannot be in a cache before its flag is up, because nobody reads
+ * them earlier inside the launch and a launch starts from invalidated caches. */
+int smr_set_ag_matmul_acquire(int on);
+
 /* Tuning knob of the gated schedule: the first `head` and the last `tail` comm blocks
  * of the ring order are computed in tiles of half the width.  Both -1 (the default)
  * means none.  No reference counterpart. */

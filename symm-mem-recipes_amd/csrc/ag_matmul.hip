@@ -51,6 +51,7 @@ struct GemmSchedule {
   int head, tail;
   int steps;                     // trips of the busiest workgroup (passes over all phases)
   int group_m;                   // row tiles per group of the tile order; divides the comm block's
+  int acquire;                   // invalidate the caches behind every flag wait (smr_set_ag_matmul_acquire)
 };
 
 struct TileRef {
@@ -763,7 +764,24 @@ __global__ __launch_bounds__(kGemmThreads, 1) void ag_matmul_kernel(
   // block's flag is up.
   auto a_rows_of = [&](const TileRef& t) -> const uint8_t* {
     if (t.local) return a_shard + (int64_t)t.a_row * cx.row_stride;
-    if (progress != nullptr) wait_signal(progress + t.comm_block, limit_ticks, status, t.comm_block);
+    if (progress != nullptr) {
+      // Thread 0 polls the flag past the caches, the workgroup meets, and only then are the
+      // rows' loads issued.  No cache is invalidated here: a line of this comm block can sit
+      // in this compute unit's L1 or this XCD's L2 only if somebody read or wrote it since
+      // the kernel began (the dispatch itself starts from invalidated caches), nobody reads
+      // a comm block's rows before its flag, and whoever wrote them (the producer, or the
+      // grid pulling the first chunk) wrote whole lines through to memory and saw them
+      // acknowledged before the flag went up.  The invalidate an acquire fence stands for
+      // would throw out the XCD's shared A and B lines at every tile instead: 2 % of the
+      // fused launch.  smr_set_ag_matmul_acquire(1) puts the fence back.
+      if (s.acquire) {
+        wait_signal(progress + t.comm_block, limit_ticks, status, t.comm_block);
+      } else {
+        if (threadIdx.x == 0 && !wait_flag_set(progress + t.comm_block, limit_ticks))
+          report(status, SMR_ST_WAIT_TIMEOUT, t.comm_block, blockIdx.x, 0u);
+        __syncthreads();
+      }
+    }
     return a_out + (int64_t)t.a_row * cx.row_stride;
   };
 
@@ -917,6 +935,7 @@ static FusedEstimate estimate_fused(const GemmSchedule& s, int cus, int grid, in
 // smr_set_ag_matmul_halves: ring positions cut into half tiles at either end of a
 // gated launch, or -1 to let make_schedule choose.
 static int g_force_head = -1, g_force_tail = -1;
+static int g_acquire_after_flag = 0;
 
 static GemmSchedule make_schedule(int M, int N, int K, int rank, int world_size, int comm_block_m,
                                   int cus, bool gated, int elem_bytes = 2) {
@@ -924,6 +943,7 @@ static GemmSchedule make_schedule(int M, int N, int K, int rank, int world_size,
   s.M = M; s.N = N; s.K = K;
   s.rank = rank; s.world_size = world_size; s.comm_block_m = comm_block_m;
   s.head = s.tail = 0;
+  s.acquire = g_acquire_after_flag;
   if (elem_bytes == 1) s.BM = s.BN = 256;        // the e4m3fn tile exists in one shape
   else pick_tile(M, N, comm_block_m, s.BM, s.BN, cus);
   const int tn = (N + s.BN - 1) / s.BN;
@@ -1108,6 +1128,11 @@ int smr_ag_matmul_fp8(const void* a_shard_dev, const void* a_out_dev, const void
   if (int rc = validate_fp8(M, N, K, rank, world_size, comm_block_m, &why)) return fail(rc, why);
   return launch_gemm(1, a_shard_dev, a_out_dev, b_nk_dev, c_dev, progress_dev, M, N, K, rank, world_size,
                      comm_block_m, status, stream, nullptr, nullptr, nullptr);
+}
+
+int smr_set_ag_matmul_acquire(int on) {
+  smr::g_acquire_after_flag = on ? 1 : 0;
+  return 0;
 }
 
 int smr_ag_matmul_plan_fp8(int M, int N, int K, int world_size, int comm_block_m, int32_t* out5) {

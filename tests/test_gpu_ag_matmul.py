@@ -312,6 +312,39 @@ def test_small_launch_leaves_the_first_chunk_to_the_producer(cuda, lib):
                                         rank, ws, M // ws, h.status.data_ptr(), None) == -1
 
 
+@pytest.fixture(params=[0, 1], ids=["flag-only", "acquire"])
+def acquire_mode(request, lib):
+    assert lib.smr_set_ag_matmul_acquire(request.param) == 0
+    yield request.param
+    lib.smr_set_ag_matmul_acquire(0)
+
+
+@pytest.mark.parametrize("M,N,K", [(8192, 1024, 1024), (16384, 2048, 256)])
+def test_fused_reads_fresh_rows_when_buffers_are_reused(cuda, either_form, acquire_mode, M, N, K):
+    """The same gathered buffer, the same output and new shard contents call after call,
+    with no host synchronisation in between: a tile must never be computed from rows that
+    a cache kept from the call before (the gathered operand of these shapes fits the L2s)."""
+    from symm_mem_recipes import all_gather_matmul_tma_persistent
+    ws, rank = 8, 4
+    a_shard, h, shards, b, b_bits, a_out, c_out = _setup(M, N, K, ws, rank, cuda)
+    rows = M // ws
+    versions = []
+    for v in range(4):
+        bits = [O.seeded_normal_bf16_bits(rows * K, seed=1000 * v + r, std=0.02).reshape(rows, K) for r in range(ws)]
+        versions.append((bits, [_bits_t(x).to(cuda) for x in bits]))
+    outs = []
+    for bits, dev_bits in versions:
+        for r in range(ws):
+            h.get_buffer(r, (rows, K), torch.bfloat16).copy_(dev_bits[r])
+        all_gather_matmul_tma_persistent(a_shard, b, a_out, c_out, None)
+        outs.append((c_out.clone(), a_out.clone()))
+    torch.cuda.synchronize()
+    h.check_status()
+    for (bits, _), (c, a) in zip(versions, outs):
+        assert np.array_equal(_t_bits(a), np.concatenate(bits))
+        _check(_t_bits(c), O.ag_matmul_ref(bits, b_bits))
+
+
 def test_mm_only_is_ungated(cuda, monkeypatch):
     """mm_only multiplies what the buffers already hold, as rank 0, with no flags
     (triton_all_gather_matmul.py:222-224,246-247)."""
