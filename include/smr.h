@@ -232,7 +232,7 @@ int smr_ag_matmul_pull_first(const void* a_shard_dev, void* a_out_dev, const voi
  * reference's FP8_OUTPUT switch (triton_all_gather_matmul.py:115,123,188,311).  The cast of
  * the accumulator rounds to nearest even and saturates to +-448, NaN stays NaN (what
  * Triton's cast compiles to on the reference's hardware, cvt.rn.satfinite).
- * K % 128 == 0, N % 16 == 0, comm_block_m % 256 == 0; otherwise as smr_ag_matmul. */
+ * K % 128 == 0, N % 16 == 0; otherwise as smr_ag_matmul (same tile shapes, same schedule). */
 int smr_ag_matmul_fp8(const void* a_shard_dev, const void* a_out_dev, const void* b_nk_dev, void* c_dev,
                       const uint32_t* progress_dev, int M, int N, int K, int rank, int world_size,
                       int comm_block_m, uint32_t* status, void* stream);

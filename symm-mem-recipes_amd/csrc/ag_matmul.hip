@@ -493,7 +493,7 @@ __device__ __forceinline__ void run_tile(const TileContext& cx, const TileRef& t
 // (0 or 1).  Both operands use the same lane -> K mapping, which is all the sum
 // over K needs.  The 8 lanes x 2 that an LDS read serves together are 8 consecutive
 // rows at two chunks that differ by 2: the case row_swizzle is built for.
-// 256x256 tiles only: a wave holds 4 x 4 accumulators of 16 registers.
+// A wave of a 256x256 tile holds 4 x 4 accumulators of 16 registers.
 typedef int i32x8 __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 
@@ -505,11 +505,10 @@ __device__ __forceinline__ uint32_t pack_fp8x4(float a, float b, float c, float 
   return (uint32_t)w;
 }
 
-template <typename Between>
+template <int BM, int BN, typename Between>
 __device__ __forceinline__ void run_tile_fp8(const TileContext& cx, const TileRef& tile,
                                              const uint8_t* a_rows, const uint8_t* b_rows,
                                              bool preloaded, Between&& between) {
-  constexpr int BM = 256, BN = 256;
   using T = GemmTile<BM, BN>;
   const uint8_t* a_base = uniform_ptr(a_rows);
   const uint8_t* b_base = uniform_ptr(b_rows);
@@ -644,7 +643,9 @@ __device__ __forceinline__ void run_tile_fp8(const TileContext& cx, const TileRe
     const uint8_t* ak = a_base + (int64_t)ka * kRowBytes;
     const uint32_t a_dst = a_at >= kSlot ? a_at - kSlot : a_at + (kRingSlots - 1) * kSlot;
     first_step(ak, lds0 + a_dst + wave * (GA * 1024));
-    asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+    static_assert(GA == 8 || GA == 4, "explicit vmcnt below");
+    if constexpr (GA == 8) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+    else asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
     __syncthreads();
     second_step(kt);
   }
@@ -656,11 +657,13 @@ __device__ __forceinline__ void run_tile_fp8(const TileContext& cx, const TileRe
   // Epilogue.  D[n][m]: a lane holds row m = lane & 31 of a 32x32 fragment and, per
   // group g of 4 registers, the 4 consecutive columns g*8 + (lane >> 5)*4 .. +3: one
   // 32-bit word of e4m3fn.  32 rows at a time go through the wave's quarter of ring
-  // slot 4 (128 bytes per row, chunk c of row r at position c ^ ((r >> 1) & 7)) and
-  // leave as whole rows, 16 bytes per lane.
+  // slot 4 (WN bytes per row, chunk c of row r at position c ^ (r >> 1), modulo the
+  // chunks of a row) and leave as whole rows, 16 bytes per lane.
+  constexpr int kChunks = WN / 16;                // 16-byte chunks per wave-tile row
+  constexpr int kRowsPerStore = 64 / kChunks;
   const uint32_t turn = lds0 + (kRingSlots - 1) * kSlot + wave * (32 * WN);
   const int half = ln >> 5, wr_row = ln & 31;
-  const int rd_row = ln >> 3, rd_chunk = ln & 7;
+  const int rd_row = ln / kChunks, rd_chunk = ln % kChunks;
 #pragma unroll
   for (int mi = 0; mi < FM; ++mi) {
 #pragma unroll
@@ -670,14 +673,15 @@ __device__ __forceinline__ void run_tile_fp8(const TileContext& cx, const TileRe
         const f32x16& d = acc[ni][mi];
         const uint32_t w = pack_fp8x4(d[g * 4 + 0], d[g * 4 + 1], d[g * 4 + 2], d[g * 4 + 3]);
         const int chunk = ni * 2 + (g >> 1);
-        const uint32_t addr = turn + wr_row * WN + (((chunk ^ (wr_row >> 1)) & 7) << 4) + ((g & 1) * 2 + half) * 4;
+        const uint32_t addr = turn + wr_row * WN + (((chunk ^ (wr_row >> 1)) & (kChunks - 1)) << 4) +
+                              ((g & 1) * 2 + half) * 4;
         *reinterpret_cast<__attribute__((address_space(3))) uint32_t*>((uintptr_t)addr) = w;
       }
     }
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int r = i * 8 + rd_row;
-      const u32x4 v = lds_read_b128(turn + r * WN + (((rd_chunk ^ (r >> 1)) & 7) << 4));
+    for (int i = 0; i < 32 / kRowsPerStore; ++i) {
+      const int r = i * kRowsPerStore + rd_row;
+      const u32x4 v = lds_read_b128(turn + r * WN + (((rd_chunk ^ (r >> 1)) & (kChunks - 1)) << 4));
       const int m = tile.row0 + wm * WM + mi * 32 + r;
       const int n = tile.col0 + wn * WN + rd_chunk * 16;
       if (n < s.N) *reinterpret_cast<u32x4*>(c + (int64_t)m * s.N + n) = v;
@@ -822,8 +826,11 @@ __global__ __launch_bounds__(kGemmThreads, 1) void ag_matmul_kernel(
         issue_prologue<BM, BN>(cx, a_next, b_next, b_last);
       }
     };
-    if constexpr (FP8) {
-      run_tile_fp8(cx, tile, a_base, b_base, preloaded, between);
+    if constexpr (FP8 && BN == 256) {
+      if (tile.cols != BN) run_tile_fp8<BM, BN / 2>(cx, tile, a_base, b_base, preloaded, between);
+      else run_tile_fp8<BM, BN>(cx, tile, a_base, b_base, preloaded, between);
+    } else if constexpr (FP8) {
+      run_tile_fp8<BM, BN>(cx, tile, a_base, b_base, preloaded, between);
     } else if constexpr (BN == 256) {
       if (tile.cols != BN) run_tile<BM, BN / 2>(cx, tile, a_base, b_base, preloaded, between);
       else run_tile<BM, BN>(cx, tile, a_base, b_base, preloaded, between);
@@ -944,8 +951,7 @@ static GemmSchedule make_schedule(int M, int N, int K, int rank, int world_size,
   s.rank = rank; s.world_size = world_size; s.comm_block_m = comm_block_m;
   s.head = s.tail = 0;
   s.acquire = g_acquire_after_flag;
-  if (elem_bytes == 1) s.BM = s.BN = 256;        // the e4m3fn tile exists in one shape
-  else pick_tile(M, N, comm_block_m, s.BM, s.BN, cus);
+  pick_tile(M, N, comm_block_m, s.BM, s.BN, cus);
   const int tn = (N + s.BN - 1) / s.BN;
   const int total = (M / s.BM) * tn;
   int max_grid = ((gated ? cus - kReservedCus : cus) / 8) * 8;
@@ -1060,8 +1066,14 @@ static int launch_gemm(int elem_bytes, const void* a_shard_dev, const void* a_ou
     }
   }
   if (helpers_out != nullptr) *helpers_out = pf.helpers;
-  if (elem_bytes == 1)
+  if (elem_bytes == 1 && s.BM == 256 && s.BN == 256)
     hipLaunchKernelGGL((ag_matmul_kernel<256, 256, true>), dim3(s.grid), dim3(kGemmThreads), 0, st, a0, a1, b,
+                       c, progress_dev, s, lim, status, tb, pf);
+  else if (elem_bytes == 1 && s.BM == 256)
+    hipLaunchKernelGGL((ag_matmul_kernel<256, 128, true>), dim3(s.grid), dim3(kGemmThreads), 0, st, a0, a1, b,
+                       c, progress_dev, s, lim, status, tb, pf);
+  else if (elem_bytes == 1)
+    hipLaunchKernelGGL((ag_matmul_kernel<128, 128, true>), dim3(s.grid), dim3(kGemmThreads), 0, st, a0, a1, b,
                        c, progress_dev, s, lim, status, tb, pf);
   else if (s.BM == 256 && s.BN == 256)
     hipLaunchKernelGGL((ag_matmul_kernel<256, 256>), dim3(s.grid), dim3(kGemmThreads), 0, st, a0, a1, b,
@@ -1115,8 +1127,6 @@ static int validate_fp8(int M, int N, int K, int rank, int world_size, int comm_
     *why = "smr_ag_matmul_fp8: K must be a multiple of 128";
   else if (N % 16 != 0)
     *why = "smr_ag_matmul_fp8: N must be a multiple of 16";
-  else if (comm_block_m % 256 != 0)
-    *why = "smr_ag_matmul_fp8: rows per progress flag must be a multiple of 256";
   return *why ? SMR_E_UNSUPPORTED : 0;
 }
 

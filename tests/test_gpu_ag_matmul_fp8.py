@@ -67,6 +67,11 @@ def _release():
     (2048, 400, 384, 8, 5),       # ragged last column tile
     (4096, 512, 1024, 8, 3),
     (2048, 272, 256, 4, 1),       # world size 4, two row tiles per comm block
+    (1024, 256, 256, 8, 2),       # comm blocks of 128 rows: 128x128 tiles
+    (1024, 144, 128, 8, 7),       # 128x128 tiles, ragged last column tile, one K slab
+    (2048, 128, 1024, 8, 6),      # 128x128 tiles, eight K slabs
+    (4096, 1280, 256, 8, 4),      # 256x128 tiles
+    (8192, 1280, 128, 8, 1),      # 256x256 tiles, many of them
 ])
 def test_fp8_fused_parity(cuda, either_form, M, N, K, ws, rank):
     from symm_mem_recipes import all_gather_matmul_tma_persistent
