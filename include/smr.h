@@ -213,13 +213,14 @@ int smr_ag_matmul_schedule(int M, int N, int K, int rank, int world_size, int co
 /* smr_ag_matmul (elem_bytes 2) or smr_ag_matmul_fp8 (elem_bytes 1), gated, whose
  * workgroups copy the first remote chunk themselves.  Half the grid of a gated launch
  * starts on the first remote comm block and would wait for the producer to deliver it;
- * those workgroups are idle compute units, so they pull the chunk from
- * buffer_ptrs_dev[rank + 1] into a_out (a slice each), the last one raises
+ * those workgroups are idle compute units, so the grid pulls the chunk from
+ * buffer_ptrs_dev[rank + 1] into a_out first (64 KiB pieces taken by ticket, so a workgroup
+ * that is dispatched late holds nobody up), the one that completes it raises
  * progress[(rank + 1) * splits], and the producer is started at its second chunk
  * (smr_all_gather_with_progress_from, first_chunk = 1).  The reference's copy engines
  * deliver every chunk (triton_all_gather_matmul.py:41-55); this is the part of that loop
  * the consumer takes over when the copy has to run on compute units.
- *   pull_counters_dev  uint32 [2], zero on entry, zero again when the kernel is through
+ *   pull_counters_dev  uint32 [2], zero on entry (not restored: zero them before every call)
  * Returns the number of pulling workgroups (> 0: start the producer at chunk 1), 0 when
  * too few workgroups would wait for pulling to pay (plain gated launch: start the producer
  * at chunk 0), or a negative SMR_E_* code. */

@@ -694,57 +694,64 @@ __device__ __forceinline__ void run_tile_fp8(const TileContext& cx, const TileRe
 // A gated launch puts as many workgroups on the first remote comm block as on the
 // local one, and a producer that owns an eighth of the GPU needs a third of a tile's
 // time to deliver that chunk; every workgroup has the same number of tiles, so the
-// launch ends late by that wait.  Instead the whole grid copies the chunk first (a
-// slice per workgroup, taken by ticket; 32 MiB in about 15 us), the last workgroup to
-// finish raises the flag, and the producer starts at the second chunk, which it
-// delivers long before the second pass.
+// launch ends late by that wait.  Instead the grid copies the chunk first (32 MiB in
+// about 15 us), the workgroup that completes it raises the flag, and the producer
+// starts at the second chunk, which it delivers long before the second pass.
+//
+// The chunk is cut into 64 KiB pieces that the workgroups take by ticket until none
+// is left, so nothing depends on how many workgroups are running: one that is
+// dispatched late (another kernel holds its compute unit) finds the pieces gone and
+// goes on to its tiles, and the ones that are there do all of the copying.
 struct PullFirst {
   const uint64_t* buffer_ptrs;   // the ranks' shard addresses (device array); nullptr = off
   uint8_t* dst;                  // the chunk's place in the gathered operand
   uint32_t* flag;                // its progress flag
-  uint32_t* counters;            // [0] tickets, [1] arrivals; zero on entry, zero again on exit
+  uint32_t* counters;            // [0] tickets, [1] finished pieces; zero on entry
   int64_t vecs;                  // 16-byte vectors in the chunk
-  int src_rank, comm_block, helpers;
+  int src_rank, comm_block, pieces;
 };
 
 typedef __attribute__((address_space(1))) u32x4 GlobalVec;
+constexpr int kPullInFlight = 16;                               // 128-bit loads per thread and piece
+constexpr int kPullPieceVecs = kGemmThreads * kPullInFlight;    // 64 KiB
 
 __device__ __forceinline__ void pull_first_chunk(const PullFirst& pf, uint32_t lds0) {
-  // one ticket per workgroup, handed to its threads through the (still unused) tile ring
-  if (threadIdx.x == 0) {
-    const uint32_t t = __hip_atomic_fetch_add(&pf.counters[0], 1u, __ATOMIC_RELAXED, kScope);
-    *reinterpret_cast<__attribute__((address_space(3))) uint32_t*>((uintptr_t)lds0) = t;
-  }
-  __syncthreads();
-  const uint32_t ticket = *reinterpret_cast<__attribute__((address_space(3))) uint32_t*>((uintptr_t)lds0);
-  __syncthreads();
+  typedef __attribute__((address_space(3))) uint32_t LdsWord;
+  LdsWord* slot = reinterpret_cast<LdsWord*>((uintptr_t)lds0);   // the tile ring is not in use yet
+  // a ticket for the whole workgroup: thread 0 draws it, the others read it
+  auto draw = [&]() -> uint32_t {
+    if (threadIdx.x == 0) *slot = __hip_atomic_fetch_add(&pf.counters[0], 1u, __ATOMIC_RELAXED, kScope);
+    __syncthreads();
+    const uint32_t t = *slot;
+    __syncthreads();
+    return t;
+  };
   const GlobalVec* src = (const GlobalVec*)(uintptr_t)pf.buffer_ptrs[pf.src_rank];
   GlobalVec* dst = (GlobalVec*)(uintptr_t)pf.dst;
-  constexpr int kInFlight = 16;
-  const int64_t stride = (int64_t)pf.helpers * kGemmThreads;
-  int64_t i = (int64_t)ticket * kGemmThreads + threadIdx.x;
-  for (; i + (kInFlight - 1) * stride < pf.vecs; i += kInFlight * stride) {
-    u32x4 v[kInFlight];
+  uint32_t mine = 0;
+  for (uint32_t t = draw(); t < (uint32_t)pf.pieces; t = draw()) {
+    const int64_t i0 = (int64_t)t * kPullPieceVecs + threadIdx.x;
+    u32x4 v[kPullInFlight];
 #pragma unroll
-    for (int u = 0; u < kInFlight; ++u) v[u] = __builtin_nontemporal_load(src + i + u * stride);
+    for (int u = 0; u < kPullInFlight; ++u) {
+      const int64_t i = i0 + u * kGemmThreads;
+      v[u] = __builtin_nontemporal_load(src + (i < pf.vecs ? i : pf.vecs - 1));
+    }
 #pragma unroll
-    for (int u = 0; u < kInFlight; ++u)
-      asm volatile("global_store_dwordx4 %0, %1, off sc1" : : "v"(dst + i + u * stride), "v"(v[u]) : "memory");
+    for (int u = 0; u < kPullInFlight; ++u) {
+      const int64_t i = i0 + u * kGemmThreads;
+      if (i < pf.vecs)
+        asm volatile("global_store_dwordx4 %0, %1, off sc1" : : "v"(dst + i), "v"(v[u]) : "memory");
+    }
+    ++mine;
   }
-  for (; i < pf.vecs; i += stride) {
-    const u32x4 v = __builtin_nontemporal_load(src + i);
-    asm volatile("global_store_dwordx4 %0, %1, off sc1" : : "v"(dst + i), "v"(v) : "memory");
-  }
-  // written through: once acknowledged the slice is where every XCD reads it
+  if (mine == 0) return;
+  // written through: once acknowledged the pieces are where every XCD reads them
   wait_stores_acknowledged();
   __syncthreads();
   if (threadIdx.x == 0) {
-    const uint32_t prev = __hip_atomic_fetch_add(&pf.counters[1], 1u, __ATOMIC_RELAXED, kScope);
-    if (prev + 1u == (uint32_t)pf.helpers) {
-      __hip_atomic_store(&pf.counters[0], 0u, __ATOMIC_RELAXED, kScope);
-      __hip_atomic_store(&pf.counters[1], 0u, __ATOMIC_RELAXED, kScope);
-      __hip_atomic_store(pf.flag, 1u, __ATOMIC_RELAXED, kScope);
-    }
+    const uint32_t prev = __hip_atomic_fetch_add(&pf.counters[1], mine, __ATOMIC_RELAXED, kScope);
+    if (prev + mine == (uint32_t)pf.pieces) __hip_atomic_store(pf.flag, 1u, __ATOMIC_RELAXED, kScope);
   }
 }
 
@@ -1052,7 +1059,6 @@ static int launch_gemm(int elem_bytes, const void* a_shard_dev, const void* a_ou
     const int splits = (M / world_size) / comm_block_m;
     const int src_rank = (rank + 1) % world_size;
     const int waiters = first_chunk_waiters(s, src_rank * splits);
-    const int helpers = s.grid;
     if (waiters >= kMinPullHelpers) {
       const int64_t chunk_bytes = (int64_t)comm_block_m * K * elem_bytes;
       pf.buffer_ptrs = buffer_ptrs_dev;
@@ -1062,10 +1068,10 @@ static int launch_gemm(int elem_bytes, const void* a_shard_dev, const void* a_ou
       pf.vecs = chunk_bytes / 16;
       pf.src_rank = src_rank;
       pf.comm_block = src_rank * splits;
-      pf.helpers = helpers;
+      pf.pieces = (int)((pf.vecs + kPullPieceVecs - 1) / kPullPieceVecs);
     }
   }
-  if (helpers_out != nullptr) *helpers_out = pf.helpers;
+  if (helpers_out != nullptr) *helpers_out = pf.pieces > 0 ? s.grid : 0;
   if (elem_bytes == 1 && s.BM == 256 && s.BN == 256)
     hipLaunchKernelGGL((ag_matmul_kernel<256, 256, true>), dim3(s.grid), dim3(kGemmThreads), 0, st, a0, a1, b,
                        c, progress_dev, s, lim, status, tb, pf);

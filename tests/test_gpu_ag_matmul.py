@@ -267,7 +267,7 @@ def test_first_chunk_pulled_by_the_gemm(cuda, lib, force_fused, monkeypatch, M, 
     _check(_t_bits(outs[0]), O.ag_matmul_ref(shards, b_bits))
     assert torch.equal(outs[0].view(torch.int16), outs[1].view(torch.int16))
     assert torch.equal(outs[0].view(torch.int16), outs[2].view(torch.int16))
-    # through the C ABI: it reports the pulling workgroups, leaves its two counters zero and
+    # through the C ABI: it reports the pulling workgroups, counts every piece of the chunk once and
     # raises the first remote chunk's flag itself (no producer is started here, so only that one)
     chunks = ws * splits
     state = torch.zeros(chunks + 2, dtype=torch.int32, device=cuda)
@@ -283,7 +283,9 @@ def test_first_chunk_pulled_by_the_gemm(cuda, lib, force_fused, monkeypatch, M, 
     torch.cuda.synchronize()
     h.check_status()
     assert pulled == lib.smr_ag_matmul_grid(M, N, K, ws, rows, 1) > 0
-    assert state.cpu().tolist() == [1] * chunks + [0, 0]
+    pieces = -(-rows * K * 2 // 65536)                      # 64 KiB pieces, each taken once and finished once
+    final = state.cpu().tolist()
+    assert final[:chunks] == [1] * chunks and final[chunks] >= pieces and final[chunks + 1] == pieces
     assert np.array_equal(_t_bits(a_out), np.concatenate(shards))
     assert torch.equal(c_out.view(torch.int16), outs[0].view(torch.int16))
 
