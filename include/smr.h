@@ -72,8 +72,8 @@ int smr_set_spin_timeout_us(int64_t us);
  * into which the all-gather producer and the GEMM write time stamps of the
  * GPU's 100 MHz constant clock.  Words 0..62: time progress flag i was raised,
  * word 63: producer start.  Words 64 + (workgroup*16 + step)*4 + k: GEMM
- * workgroup's step-th tile, k = 0 tile picked, 1 flag wait over, 2 K loop done,
- * 3 tile stored.  Needs 64 + 256*16*4 words for the GEMM part.  The reference's
+ * workgroup's step-th tile, k = 0 tile picked (step 0: kernel entry), 1 flag wait
+ * over (step 0: the pull of the first chunk included), 2 K loop done, 3 tile stored.  Needs 64 + 256*16*4 words for the GEMM part.  The reference's
  * counterpart is its profiler hook (symm_mem_recipes/utils.py:41-52). */
 int smr_set_trace_buffer(uint64_t* trace_dev, int64_t words);
 int64_t smr_get_spin_timeout_us(void);

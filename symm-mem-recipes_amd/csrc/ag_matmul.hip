@@ -729,7 +729,8 @@ __device__ __forceinline__ void pull_first_chunk(const PullFirst& pf, uint32_t l
   const GlobalVec* src = (const GlobalVec*)(uintptr_t)pf.buffer_ptrs[pf.src_rank];
   GlobalVec* dst = (GlobalVec*)(uintptr_t)pf.dst;
   uint32_t mine = 0;
-  for (uint32_t t = draw(); t < (uint32_t)pf.pieces; t = draw()) {
+  uint32_t t = draw();
+  while (t < (uint32_t)pf.pieces) {
     const int64_t i0 = (int64_t)t * kPullPieceVecs + threadIdx.x;
     u32x4 v[kPullInFlight];
 #pragma unroll
@@ -737,6 +738,8 @@ __device__ __forceinline__ void pull_first_chunk(const PullFirst& pf, uint32_t l
       const int64_t i = i0 + u * kGemmThreads;
       v[u] = __builtin_nontemporal_load(src + (i < pf.vecs ? i : pf.vecs - 1));
     }
+    // the next ticket is drawn while this piece's loads are in flight
+    t = draw();
 #pragma unroll
     for (int u = 0; u < kPullInFlight; ++u) {
       const int64_t i = i0 + u * kGemmThreads;
@@ -796,6 +799,7 @@ __global__ __launch_bounds__(kGemmThreads, 1) void ag_matmul_kernel(
     return a_out + (int64_t)t.a_row * cx.row_stride;
   };
 
+  const uint64_t t_entry = trace != nullptr ? wall_clock64() : 0;
   TileRef tile;
   int step = 0;
   bool have = next_tile(s, blockIdx.x, step, tile);
@@ -812,6 +816,7 @@ __global__ __launch_bounds__(kGemmThreads, 1) void ag_matmul_kernel(
     if (trace != nullptr && trip < kTraceSteps && blockIdx.x < 256 && threadIdx.x == 0) {
       cx.tr = trace + kTraceProducerWords + ((size_t)blockIdx.x * kTraceSteps + trip) * 4;
       cx.tr[0] = cx.tr[1] = wall_clock64();
+      if (trip == 0) cx.tr[0] = t_entry;     // the first tile's wait includes the pull of the first chunk
     }
     TileRef next;
     bool have_next = false;

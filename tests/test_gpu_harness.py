@@ -50,3 +50,18 @@ def test_module_self_checks(cuda, capsys):
     out = capsys.readouterr().out
     for label in ("library matmul only:", "hip matmul only:", "library gather + matmul:", "hip all_gather_matmul:"):
         assert label in out
+
+
+def test_trace_of_a_launch(cuda):
+    """The kernels' own time stamps: every workgroup's tiles in order, the producer's flags
+    behind its start, and the fused launch's first wait no longer than the whole launch."""
+    from symm_mem_recipes import trace
+    for mode in ("ungated", "fused", "fused-no-pull", "sequential"):
+        r = trace.trace_launch(16384, 2048, 256, mode, warm=2)
+        assert r["end_us"] > 0 and r["steps"], mode
+        assert sum(s["workgroups"] for s in r["steps"]) == (16384 // 256) * (2048 // 256), mode
+        for s in r["steps"]:
+            assert s["k_loop_us"] > 0 and s["wait_us"] >= 0 and s["last_stored_us"] <= r["end_us"]
+        if mode.startswith("fused"):
+            assert r["producer_start_us"] is not None and len(r["flags_us"]) >= 6
+            assert all(v > r["producer_start_us"] for v in r["flags_us"].values())
