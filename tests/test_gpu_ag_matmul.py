@@ -347,6 +347,36 @@ def test_fused_reads_fresh_rows_when_buffers_are_reused(cuda, either_form, acqui
         _check(_t_bits(c), O.ag_matmul_ref(bits, b_bits))
 
 
+def _random_shapes(n, seed):
+    rng = np.random.default_rng(seed)
+    shapes = []
+    while len(shapes) < n:
+        ws = int(rng.choice([2, 3, 4, 5, 8]))
+        splits = int(rng.choice([1, 1, 2, 3]))
+        comm = int(rng.choice([128, 256, 384, 512, 768, 1024]))
+        M = ws * splits * comm
+        N = 8 * int(rng.integers(1, 190))
+        K = 64 * int(rng.integers(1, 17))
+        if M * N * K > 8e9:
+            continue
+        shapes.append((M, N, K, ws, int(rng.integers(0, ws)), splits))
+    return shapes
+
+
+@pytest.mark.parametrize("M,N,K,ws,rank,splits", _random_shapes(14, seed=2024))
+def test_fused_parity_random_shapes(cuda, either_form, M, N, K, ws, rank, splits):
+    """Shapes drawn at random from what the kernel accepts (every world size, ragged column
+    tiles, one to sixteen K slabs, one to three flags per rank): product and gathered operand
+    against the oracle in both forms of the launch."""
+    from symm_mem_recipes import all_gather_matmul_tma_persistent
+    a_shard, h, shards, b, b_bits, a_out, c_out = _setup(M, N, K, ws, rank, cuda)
+    a_out.zero_()
+    all_gather_matmul_tma_persistent(a_shard, b, a_out, c_out, None, splits_per_rank=splits)
+    h.check_status()
+    assert np.array_equal(_t_bits(a_out), np.concatenate(shards))
+    _check(_t_bits(c_out), O.ag_matmul_ref(shards, b_bits))
+
+
 def test_mm_only_is_ungated(cuda, monkeypatch):
     """mm_only multiplies what the buffers already hold, as rank 0, with no flags
     (triton_all_gather_matmul.py:222-224,246-247)."""
