@@ -83,6 +83,29 @@ def test_fp8_fused_parity(cuda, either_form, M, N, K, ws, rank):
     assert np.array_equal(_bits(a_out), np.concatenate(shards))
 
 
+def _random_shapes(n, seed):
+    rng = np.random.default_rng(seed)
+    shapes = []
+    while len(shapes) < n:
+        ws = int(rng.choice([2, 4, 5, 8]))
+        comm = int(rng.choice([128, 256, 384, 512, 1024]))
+        M = ws * comm
+        N = 16 * int(rng.integers(1, 90))
+        K = 128 * int(rng.integers(1, 9))
+        shapes.append((M, N, K, ws, int(rng.integers(0, ws))))
+    return shapes
+
+
+@pytest.mark.parametrize("M,N,K,ws,rank", _random_shapes(10, seed=77))
+def test_fp8_parity_random_shapes(cuda, either_form, M, N, K, ws, rank):
+    from symm_mem_recipes import all_gather_matmul_tma_persistent
+    a_shard, h, shards, b, b_bits, a_out, c_out = _setup(M, N, K, ws, rank, cuda)
+    all_gather_matmul_tma_persistent(a_shard, b, a_out, c_out, None)
+    h.check_status()
+    assert np.array_equal(_bits(a_out), np.concatenate(shards))
+    _check(_bits(c_out), O.ag_matmul_ref_fp8(shards, b_bits))
+
+
 def test_fp8_first_chunk_pulled_by_the_gemm(cuda, lib, monkeypatch):
     """A launch wide enough that the grid copies the first remote chunk itself: same codes
     as with every chunk left to the producer, gathered operand complete."""
