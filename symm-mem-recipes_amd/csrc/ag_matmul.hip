@@ -23,7 +23,11 @@
 //     non-local comm block first waits for that block's progress flag.  Within
 //     one pass over the grid, XCD x (workgroups with id % 8 == x) takes a
 //     contiguous run of the tile order - a patch about as wide as it is high - so
-//     the workgroups that share an L2 also share A rows and B columns.
+//     the workgroups that share an L2 also share A rows and B columns;
+//   * a launch wide enough that many workgroups would start with a wait copies the
+//     first remote chunk itself before its first tiles (pull_first_chunk);
+//   * the same kernel in e4m3fn (run_tile_fp8): the bytes move the same way, the
+//     tile is built from v_mfma_f32_32x32x64_f8f6f4.
 #include <type_traits>
 
 #include "smr_device.hpp"
