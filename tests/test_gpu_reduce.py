@@ -297,3 +297,37 @@ def test_golden_vectors(cuda):
         h.get_buffer(r, (256,), torch.float32).copy_(torch.from_numpy(g["fp32_in"][r]))
     assert np.array_equal(_bits(one_shot_all_reduce(t)).view(np.uint32), g["fp32_out"].view(np.uint32))
     h.check_status()
+
+
+@pytest.mark.parametrize("barrier", [False, True])
+def test_reduce_replays_from_a_graph(cuda, barrier):
+    """Launches captured into a HIP graph (kernel nodes only) give the eager bits on every
+    replay, with eager work and synchronisations between the replays; with the barrier the
+    signal pads must come back to zero after each replay for the next one to pass."""
+    from symm_mem_recipes import one_shot_all_reduce
+    numel = 1 << 18
+    t, h = _alloc(numel, torch.bfloat16, cuda)
+    bufs = _fill(h, numel, torch.bfloat16, seed0=11)
+    want = O.reduce_ref(bufs, "bf16")
+    eager = one_shot_all_reduce(t, barrier=barrier)
+    torch.cuda.synchronize()
+    assert np.array_equal(_bits(eager), want)
+    side = torch.cuda.Stream(cuda)
+    side.wait_stream(torch.cuda.current_stream(cuda))
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            outs = [one_shot_all_reduce(t, barrier=barrier) for _ in range(3)]
+    torch.cuda.current_stream(cuda).wait_stream(side)
+    for replay in range(4):
+        for o in outs:
+            o.zero_()
+        noise = torch.randn(1 << 18, device=cuda).sum()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        h.check_status()
+        for o in outs:
+            assert np.array_equal(_bits(o), want), replay
+        del noise
+    del graph
