@@ -124,3 +124,39 @@ def test_golden_vectors(cuda):
     ref = O.bf16_bits_to_f32(g["out"]).astype(np.float64)
     terms = np.abs(O.bf16_bits_to_f32(g["x"])).astype(np.float64) @ np.abs(O.bf16_bits_to_f32(g["w"])).astype(np.float64)
     assert _within_one_ulp(got, ref, terms)
+
+
+def test_gemv_replays_from_a_graph(cuda):
+    """Three launches on one workspace captured into a HIP graph (kernel nodes only):
+    every replay, with eager work and synchronisations in between, gives the eager bits,
+    and the flags are back to zero for the next."""
+    from symm_mem_recipes import gemv_all_reduce, GemvWorkspace
+    batch, K, N, ws = 4, 2048, 1024, 8
+    g = torch.Generator(device=cuda)
+    g.manual_seed(5)
+    x = torch.empty(batch, K, device=cuda).normal_(0, 1, generator=g).to(torch.bfloat16)
+    w = torch.empty(K, N, device=cuda).normal_(0, 0.02, generator=g).to(torch.bfloat16)
+    work = GemvWorkspace(batch, N, ws, cuda, K)
+    eager = gemv_all_reduce(x, w, ws, work).clone()
+    work.check_status()
+    outs = [torch.empty(batch, N, dtype=torch.bfloat16, device=cuda) for _ in range(3)]
+    side = torch.cuda.Stream(cuda)
+    side.wait_stream(torch.cuda.current_stream(cuda))
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            for o in outs:
+                gemv_all_reduce(x, w, ws, work, out=o)
+    torch.cuda.current_stream(cuda).wait_stream(side)
+    for replay in range(4):
+        for o in outs:
+            o.zero_()
+        noise = torch.randn(1 << 18, device=cuda).sum()
+        torch.cuda.synchronize()
+        graph.replay()
+        work.check_status()
+        assert int(work.flags.abs().sum()) == 0
+        for o in outs:
+            assert torch.equal(o.view(torch.int16), eager.view(torch.int16)), replay
+        del noise
+    del graph
