@@ -286,6 +286,21 @@ int smr_gemv_allreduce(const void* x_dev, const void* w_dev, float* partials_dev
                        int world_size, uint32_t* status, void* stream);
 int smr_gemv_flag_blocks(int N);
 int smr_gemv_senders(int N, int K, int world_size);
+
+/* smr_gemv_allreduce for callers that cannot allocate device memory (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the
+ * reference.  Same kernels, same result bit for bit; the fp32 partials and the flags live in
+ * a fixed array inside the library (one copy per GPU, 4 MiB + 16 KiB, held until the process
+ * ends) instead of caller-provided scratch, and the call allocates nothing.
+ *   Limits: smr_gemv_senders(N, K, ws) * batch * N * 4 <= smr_gemv_static_scratch_bytes()
+ *   (4 MiB; K = N = 8192, batch 8, ws 8 needs 2 MiB) and at most 4096 workgroups; beyond
+ *   them SMR_E_UNSUPPORTED.
+ *   Every call on a GPU uses that GPU's one array: calls that overlap on one GPU (two
+ *   streams, two threads) race and must be serialised by the caller.  The flags are cleared
+ *   by a small kernel ahead of the launch, so a call that timed out leaves nothing behind. */
+int smr_gemv_allreduce_static(const void* x_dev, const void* w_dev, void* out_dev, int batch, int K,
+                              int N, int world_size, uint32_t* status, void* stream);
+int64_t smr_gemv_static_scratch_bytes(void);
 /* Tuning knob: threads per contiguous row segment (16 or 64; 0 = default 16) and
  * sub-shards per rank (1..8; 0 = chosen so that at least 256 workgroups run). */
 int smr_set_gemv_launch(int threads_per_row, int sub_shards);

@@ -19,6 +19,10 @@
 // are zero again on exit) and adds the partials in sender order, i.e. rank by
 // rank.  The partials travel with agent-coherent stores and loads, so no cache
 // write-back or invalidate surrounds the flags.
+#include <atomic>
+#include <cstdio>
+#include <mutex>
+
 #include "smr_device.hpp"
 
 namespace smr {
@@ -32,8 +36,16 @@ constexpr int kGemvKChunk = 1024;            // K rows of x staged in LDS at a t
 // chip.  Measured on MI355X at K = N = 8192: 16 threads per segment (512
 // workgroups, 64 of them combining) beat 64-thread segments at every batch size.
 // smr_set_gemv_launch overrides.
-static int g_gemv_tpr = 16;
-static int g_gemv_sub = 0;                   // 0 = pick so that >= 256 workgroups run
+// Both knobs in one word (threads per row in the low half, sub-shards in the high half), so
+// that a launch reads a consistent pair with one load whoever sets them meanwhile.
+static std::atomic<uint32_t> g_gemv_launch{16u};   // sub-shards 0 = pick so that >= 256 workgroups run
+struct GemvLaunch {
+  int tpr, sub;
+};
+static GemvLaunch gemv_launch_knobs() {
+  const uint32_t v = g_gemv_launch.load(std::memory_order_relaxed);
+  return {(int)(v & 0xFFFFu), (int)(v >> 16)};
+}
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef __attribute__((address_space(1))) u32x4 GlobalVec;
@@ -205,13 +217,105 @@ __global__ __launch_bounds__(kGemvThreads) void gemv_allreduce_kernel(
   }
 }
 
-static int gemv_sub_for(int N, int K, int world_size) {
-  if (g_gemv_sub > 0) return g_gemv_sub;
-  const int cols = g_gemv_tpr * 8;
+static int gemv_sub_for(const GemvLaunch& knobs, int N, int K, int world_size) {
+  if (knobs.sub > 0) return knobs.sub;
+  const int cols = knobs.tpr * 8;
   const int cblocks = (N + cols - 1) / cols;
   int sub = 1;
   while (sub < 8 && cblocks * world_size * sub < 256 && (K / world_size) / (sub * 2) >= 64) sub *= 2;
   return sub;
+}
+
+// Words [0, n) of `p` set to zero: a kernel, not a memset, so that a caller who captures
+// the launch into a graph records kernel nodes only.
+__global__ void gemv_clear_words_kernel(uint32_t* p, int n) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) p[i] = 0u;
+}
+
+// Scratch of smr_gemv_allreduce_static: the flags, then the fp32 partials.  One copy per GPU the
+// library runs on, held until the process ends.
+constexpr int kStaticFlagWords = 4096;                               // one per workgroup at most
+constexpr int64_t kStaticPartialBytes = (int64_t)4 << 20;
+constexpr int64_t kStaticScratchBytes = kStaticFlagWords * 4 + kStaticPartialBytes;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+// The device address of `scratch` on the current GPU.  The array's name is only a handle on
+// the host; every GPU has its own copy at its own address, looked up once per device.
+constexpr int kMaxDevices = 64;
+static std::mutex g_scratch_mutex;
+static unsigned char* g_scratch_ptr[kMaxDevices] = {};
+
+static int static_scratch(unsigned char** out) {
+  int dev = -1;
+  if (int rc = check_hip(hipGetDevice(&dev), "smr_gemv_allreduce_static: hipGetDevice")) return rc;
+  if (dev < 0 || dev >= kMaxDevices) return fail(SMR_E_UNSUPPORTED, "smr_gemv_allreduce_static: device index beyond 63");
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (g_scratch_ptr[dev] == nullptr) {
+    void* p = nullptr;
+    if (int rc = check_hip(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)),
+                           "smr_gemv_allreduce_static: hipGetSymbolAddress"))
+      return rc;
+    if (p == nullptr) return fail(SMR_E_INVALID, "smr_gemv_allreduce_static: no address for the scratch array");
+    g_scratch_ptr[dev] = static_cast<unsigned char*>(p);
+  }
+  *out = g_scratch_ptr[dev];
+  return 0;
+}
+
+// Validation and launch shared by the entry points.  `flag_capacity` (words) and
+// `partial_capacity` (bytes) bound what the kernel may touch of the two scratch arrays;
+// negative = the caller vouches for them.
+static int launch_gemv(const char* who, const void* x_dev, const void* w_dev, float* partials_dev,
+                       uint32_t* flags_dev, int64_t flag_capacity, int64_t partial_capacity, void* out_dev,
+                       int batch, int K, int N, int world_size, uint32_t* status, void* stream,
+                       bool clear_flags) {
+  char msg[160];
+  auto bad = [&](int code, const char* what) {
+    snprintf(msg, sizeof(msg), "%s: %s", who, what);
+    return fail(code, msg);
+  };
+  if (x_dev == nullptr || w_dev == nullptr || partials_dev == nullptr || flags_dev == nullptr ||
+      out_dev == nullptr)
+    return bad(SMR_E_INVALID, "null pointer");
+  if (world_size < 1 || world_size > SMR_MAX_WORLD_SIZE) return bad(SMR_E_INVALID, "world_size must be 1..8");
+  if (batch < 1 || batch > 8) return bad(SMR_E_UNSUPPORTED, "batch must be 1..8");
+  if (K <= 0 || N <= 0 || K % world_size != 0) return bad(SMR_E_INVALID, "K must split evenly over the ranks");
+  if (N % 8 != 0 || (reinterpret_cast<uintptr_t>(w_dev) & 15u))
+    return bad(SMR_E_UNSUPPORTED, "N must be a multiple of 8 and W 16-byte aligned");
+  const GemvLaunch knobs = gemv_launch_knobs();          // one consistent pair for the whole call
+  const int sub = gemv_sub_for(knobs, N, K, world_size);
+  const int cblocks = (N + knobs.tpr * 8 - 1) / (knobs.tpr * 8);
+  const int64_t grid64 = (int64_t)cblocks * world_size * sub;
+  if (grid64 > 4096) return bad(SMR_E_UNSUPPORTED, "more than 4096 workgroups cannot be co-resident");
+  const unsigned grid = (unsigned)grid64;
+  if (flag_capacity >= 0 && grid64 > flag_capacity) return bad(SMR_E_UNSUPPORTED, "too many workgroups for the flag array");
+  if (partial_capacity >= 0 && (int64_t)world_size * sub * batch * N * 4 > partial_capacity)
+    return bad(SMR_E_UNSUPPORTED, "partial sums exceed the scratch array (senders * batch * N * 4 bytes)");
+  hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+  const uint16_t* x = reinterpret_cast<const uint16_t*>(x_dev);
+  const uint8_t* w = reinterpret_cast<const uint8_t*>(w_dev);
+  uint16_t* out = reinterpret_cast<uint16_t*>(out_dev);
+  const uint64_t lim = spin_limit_ticks();
+  if (clear_flags) {
+    hipLaunchKernelGGL(gemv_clear_words_kernel, dim3((grid + 255) / 256), dim3(256), 0, st, flags_dev, (int)grid);
+    if (int rc = check_hip(hipGetLastError(), who)) return rc;
+  }
+#define SMR_GEMV_LAUNCH(BP, TPR)                                                                   \
+  hipLaunchKernelGGL((gemv_allreduce_kernel<BP, TPR>), dim3(grid), dim3(kGemvThreads), 0, st, x, w, \
+                     partials_dev, flags_dev, out, batch, K, N, world_size, sub, lim, status)
+#define SMR_GEMV_BATCH(TPR)                                                                        \
+  do {                                                                                             \
+    if (batch == 1) SMR_GEMV_LAUNCH(1, TPR);                                                       \
+    else if (batch == 2) SMR_GEMV_LAUNCH(2, TPR);                                                  \
+    else if (batch <= 4) SMR_GEMV_LAUNCH(4, TPR);                                                  \
+    else SMR_GEMV_LAUNCH(8, TPR);                                                                  \
+  } while (0)
+  if (knobs.tpr == 16) SMR_GEMV_BATCH(16);
+  else SMR_GEMV_BATCH(64);
+#undef SMR_GEMV_BATCH
+#undef SMR_GEMV_LAUNCH
+  return check_hip(hipGetLastError(), who);
 }
 
 }  // namespace smr
@@ -225,58 +329,40 @@ int smr_set_gemv_launch(int threads_per_row, int sub_shards) {
     return fail(SMR_E_INVALID, "smr_set_gemv_launch: threads_per_row must be 16 or 64");
   if (sub_shards < 0 || sub_shards > 8)
     return fail(SMR_E_INVALID, "smr_set_gemv_launch: sub_shards must be 0..8");
-  g_gemv_tpr = threads_per_row;
-  g_gemv_sub = sub_shards;
+  g_gemv_launch.store((uint32_t)threads_per_row | ((uint32_t)sub_shards << 16), std::memory_order_relaxed);
   return 0;
 }
 
 int smr_gemv_flag_blocks(int N) {
-  return N <= 0 ? 0 : (N + smr::g_gemv_tpr * 8 - 1) / (smr::g_gemv_tpr * 8);
+  const int cols = smr::gemv_launch_knobs().tpr * 8;
+  return N <= 0 ? 0 : (N + cols - 1) / cols;
 }
 
 int smr_gemv_senders(int N, int K, int world_size) {
   if (N <= 0 || K <= 0 || world_size < 1 || world_size > SMR_MAX_WORLD_SIZE) return 0;
-  return world_size * smr::gemv_sub_for(N, K, world_size);
+  return world_size * smr::gemv_sub_for(smr::gemv_launch_knobs(), N, K, world_size);
 }
 
 int smr_gemv_allreduce(const void* x_dev, const void* w_dev, float* partials_dev, uint32_t* flags_dev,
                        void* out_dev, int batch, int K, int N, int world_size, uint32_t* status,
                        void* stream) {
-  using namespace smr;
-  if (x_dev == nullptr || w_dev == nullptr || partials_dev == nullptr || flags_dev == nullptr ||
-      out_dev == nullptr)
-    return fail(SMR_E_INVALID, "smr_gemv_allreduce: null pointer");
-  if (world_size < 1 || world_size > SMR_MAX_WORLD_SIZE)
-    return fail(SMR_E_INVALID, "smr_gemv_allreduce: world_size must be 1..8");
-  if (batch < 1 || batch > 8) return fail(SMR_E_UNSUPPORTED, "smr_gemv_allreduce: batch must be 1..8");
-  if (K <= 0 || N <= 0 || K % world_size != 0)
-    return fail(SMR_E_INVALID, "smr_gemv_allreduce: K must split evenly over the ranks");
-  if (N % 8 != 0 || (reinterpret_cast<uintptr_t>(w_dev) & 15u))
-    return fail(SMR_E_UNSUPPORTED, "smr_gemv_allreduce: N must be a multiple of 8 and W 16-byte aligned");
-  const int sub = gemv_sub_for(N, K, world_size);
-  const unsigned grid = (unsigned)smr_gemv_flag_blocks(N) * (unsigned)world_size * (unsigned)sub;
-  if (grid > 4096u)
-    return fail(SMR_E_UNSUPPORTED, "smr_gemv_allreduce: more than 4096 workgroups cannot be co-resident");
-  hipStream_t st = reinterpret_cast<hipStream_t>(stream);
-  const uint16_t* x = reinterpret_cast<const uint16_t*>(x_dev);
-  const uint8_t* w = reinterpret_cast<const uint8_t*>(w_dev);
-  uint16_t* out = reinterpret_cast<uint16_t*>(out_dev);
-  const uint64_t lim = spin_limit_ticks();
-#define SMR_GEMV_LAUNCH(BP, TPR)                                                                   \
-  hipLaunchKernelGGL((gemv_allreduce_kernel<BP, TPR>), dim3(grid), dim3(kGemvThreads), 0, st, x, w, \
-                     partials_dev, flags_dev, out, batch, K, N, world_size, sub, lim, status)
-#define SMR_GEMV_BATCH(TPR)                                                                        \
-  do {                                                                                             \
-    if (batch == 1) SMR_GEMV_LAUNCH(1, TPR);                                                       \
-    else if (batch == 2) SMR_GEMV_LAUNCH(2, TPR);                                                  \
-    else if (batch <= 4) SMR_GEMV_LAUNCH(4, TPR);                                                  \
-    else SMR_GEMV_LAUNCH(8, TPR);                                                                  \
-  } while (0)
-  if (g_gemv_tpr == 16) SMR_GEMV_BATCH(16);
-  else SMR_GEMV_BATCH(64);
-#undef SMR_GEMV_BATCH
-#undef SMR_GEMV_LAUNCH
-  return check_hip(hipGetLastError(), "smr_gemv_allreduce launch");
+  return smr::launch_gemv("smr_gemv_allreduce", x_dev, w_dev, partials_dev, flags_dev, -1, -1, out_dev, batch,
+                          K, N, world_size, status, stream, false);
 }
+
+int smr_gemv_allreduce_static(const void* x_dev, const void* w_dev, void* out_dev, int batch, int K, int N,
+                              int world_size, uint32_t* status, void* stream) {
+  using namespace smr;
+  unsigned char* base = nullptr;
+  if (int rc = static_scratch(&base)) return rc;
+  uint32_t* flags = reinterpret_cast<uint32_t*>(base);
+  float* partials = reinterpret_cast<float*>(base + kStaticFlagWords * 4);
+  // The array keeps whatever the last call left: a call that timed out may have left flags
+  // up, so they are cleared (by a kernel) ahead of every launch.
+  return launch_gemv("smr_gemv_allreduce_static", x_dev, w_dev, partials, flags, kStaticFlagWords,
+                     kStaticPartialBytes, out_dev, batch, K, N, world_size, status, stream, true);
+}
+
+int64_t smr_gemv_static_scratch_bytes(void) { return smr::kStaticPartialBytes; }
 
 }  // extern "C"
