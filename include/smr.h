@@ -98,6 +98,15 @@ int smr_one_shot_all_reduce(const uint64_t* buffer_ptrs_dev, const uint64_t* sig
                             void* out, int64_t numel, int dtype, int rank, int world_size,
                             int write_all, int barrier_mode, uint32_t* status, void* stream);
 
+/* The same call for a host that knows the peers' buffer addresses: `buffer_ptrs_host` is a
+ * HOST array of world_size device addresses, read during the call and passed to the kernel
+ * as arguments, so no thread starts with a dependent load from the device table that the
+ * reference's kernel reads (triton_one_shot_all_reduce.py:86-87).  Everything else, results
+ * included, as smr_one_shot_all_reduce. */
+int smr_one_shot_all_reduce_addrs(const uint64_t* buffer_ptrs_host, const uint64_t* signal_pad_ptrs_dev,
+                                  void* out, int64_t numel, int dtype, int rank, int world_size,
+                                  int write_all, int barrier_mode, uint32_t* status, void* stream);
+
 /* Number of workgroups (= barrier blocks per rank) the reduce launches for a
  * message; host-only.  Counterpart of the grid formula at
  * triton_one_shot_all_reduce.py:97-109, resized for 256 CUs. */
@@ -263,6 +272,11 @@ int smr_set_ag_matmul_acquire(int on);
  * of the ring order are computed in tiles of half the width.  Both -1 (the default)
  * means none.  No reference counterpart. */
 int smr_set_ag_matmul_halves(int head, int tail);
+
+/* Tuning knob: cap on the workgroups of the GEMM's persistent grid (rounded down to a multiple
+ * of 8; 0 = none), for measuring how the kernel scales with the compute units it is given.
+ * Process-wide.  No reference counterpart (its grid is NUM_SMS, triton_all_gather_matmul.py:287-294). */
+int smr_set_ag_matmul_grid_limit(int workgroups);
 
 /* Workgroups smr_ag_matmul launches on the current device for this shape; a
  * gated launch (progress_dev != NULL) keeps at least 8 compute units free for the

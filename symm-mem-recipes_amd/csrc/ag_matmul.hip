@@ -182,6 +182,16 @@ __device__ __forceinline__ void load_group(const uint8_t* base, uint32_t voff, u
                : "memory", "m0");
 }
 
+// D += A x B on a 16x16x32 bf16 fragment pair, the accumulator named as an accumulation
+// register.  Through the builtin the register allocator is free to keep an accumulator in
+// either register file, and with 256 of them next to 128 fragment registers it would, on
+// details of code far from the loop, park some in vector registers and move them back and
+// forth inside the K loop (every result still right, 9 % slower).  The compiler still sees
+// the operands, so the waits for the fragment reads that feed them are its own.
+__device__ __forceinline__ void mfma_bf16(f32x4& acc, const bf16x8& first, const bf16x8& second) {
+  asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(acc) : "v"(first), "v"(second));
+}
+
 // LDS holds a ring of five slots.  A K-slab of A and a K-slab of B take one slot each,
 // in the order A0 B0 A1 B1 A2 ..., so slab number i lives in slot i % 5: the two slabs
 // of the K step being multiplied, and up to three slabs that are landing.
@@ -372,7 +382,7 @@ __device__ __forceinline__ void run_tile(const TileContext& cx, const TileRef& t
 #pragma unroll
       for (int mi = 0; mi < FM; ++mi) {
         const int slot = ni * FM + mi;
-        acc[ni][mi] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(bf0[ni], af0[mi], acc[ni][mi], 0, 0, 0);
+        mfma_bf16(acc[ni][mi], bf0[ni], af0[mi]);
 #pragma unroll
         for (int r = 0; r < FM; ++r)
           if (r * kReadSpan / kReads == slot)
@@ -407,7 +417,7 @@ __device__ __forceinline__ void run_tile(const TileContext& cx, const TileRef& t
 #pragma unroll
       for (int mi = 0; mi < FM; ++mi) {
         const int slot = ni * FM + mi;
-        acc[ni][mi] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(bf1[ni], af1[mi], acc[ni][mi], 0, 0, 0);
+        mfma_bf16(acc[ni][mi], bf1[ni], af1[mi]);
 #pragma unroll
         for (int g = 0; g < GB; ++g)
           if (g * (kMfma / 2) / GB == slot) load_group(bk, b_off[g], lb + g * 1024);
@@ -439,8 +449,9 @@ __device__ __forceinline__ void run_tile(const TileContext& cx, const TileRef& t
     second_step(kt);
   }
   // The repeated loads of the last K steps must not land on top of the next
-  // tile's first slabs.
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  // tile's first slabs.  (The MFMAs are assembly the compiler does not time: the explicit
+  // idle slots cover the distance the last of them needs before its result may be read.)
+  asm volatile("s_waitcnt vmcnt(0)\n\ts_nop 15\n\ts_nop 15" ::: "memory");
   __syncthreads();       // the next tile's prologue overwrites the ring
   if (tr != nullptr) tr[2] = wall_clock64();
   between();
@@ -959,6 +970,7 @@ static FusedEstimate estimate_fused(const GemmSchedule& s, int cus, int grid, in
 // gated launch, or -1 to let make_schedule choose.
 static int g_force_head = -1, g_force_tail = -1;
 static int g_acquire_after_flag = 0;
+static int g_grid_limit = 0;            // smr_set_ag_matmul_grid_limit: 0 = none
 
 static GemmSchedule make_schedule(int M, int N, int K, int rank, int world_size, int comm_block_m,
                                   int cus, bool gated, int elem_bytes = 2) {
@@ -971,6 +983,7 @@ static GemmSchedule make_schedule(int M, int N, int K, int rank, int world_size,
   const int tn = (N + s.BN - 1) / s.BN;
   const int total = (M / s.BM) * tn;
   int max_grid = ((gated ? cus - kReservedCus : cus) / 8) * 8;
+  if (g_grid_limit > 0 && g_grid_limit < max_grid) max_grid = g_grid_limit / 8 * 8;
   if (max_grid < 8) max_grid = 8;
   const int passes = (total + max_grid - 1) / max_grid;
   const int need = ((total + passes - 1) / passes + 7) / 8 * 8;
@@ -1166,6 +1179,12 @@ int smr_ag_matmul_plan_fp8(int M, int N, int K, int world_size, int comm_block_m
   if (int rc = validate_fp8(M, N, K, 0, world_size, comm_block_m, &why)) return fail(rc, why);
   if (out5 == nullptr) return fail(SMR_E_INVALID, "smr_ag_matmul_plan_fp8: out5 is NULL");
   fill_plan(M, N, K, world_size, comm_block_m, 1, out5);
+  return 0;
+}
+
+int smr_set_ag_matmul_grid_limit(int workgroups) {
+  if (workgroups < 0) return smr::fail(SMR_E_INVALID, "smr_set_ag_matmul_grid_limit: negative");
+  smr::g_grid_limit = workgroups;
   return 0;
 }
 

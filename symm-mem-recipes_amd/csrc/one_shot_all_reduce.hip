@@ -18,6 +18,8 @@
 // In kAllRanks adjacent ids hold the partners of one handshake, so in-order
 // dispatch makes every partner resident by the time a later workgroup starts:
 // the spins end.
+#include <atomic>
+
 #include "smr_device.hpp"
 
 namespace smr {
@@ -30,13 +32,37 @@ constexpr int kReduceMaxThreads = 1024;
 // Defaults from a sweep on MI355X: one workgroup per compute unit streams best
 // (8 contiguous read streams of 1 MiB-strided chunks keep the DRAM pages open);
 // 512 threads below 32 MiB per buffer, 256 above.  0 = pick by size.
-static int g_reduce_threads = 0;
-static int g_reduce_max_blocks = 256;
+// Both knobs in one word (threads in the low half, cap in the high half): a launch reads the
+// pair once, so a setter on another thread cannot hand it half of an update.
+static std::atomic<uint32_t> g_reduce_launch{256u << 16};
+struct ReduceLaunch {
+  int threads, max_blocks;
+};
+static ReduceLaunch reduce_launch_knobs() {
+  const uint32_t v = g_reduce_launch.load(std::memory_order_relaxed);
+  return {(int)(v & 0xFFFFu), (int)(v >> 16)};
+}
 
-static int reduce_threads_for(int64_t nvec) {
-  if (g_reduce_threads != 0) return g_reduce_threads;
+static int reduce_threads_for(const ReduceLaunch& knobs, int64_t nvec) {
+  if (knobs.threads != 0) return knobs.threads;
   return nvec >= (int64_t)(32 << 20) / 16 ? 256 : 512;
 }
+
+static int reduce_blocks_for(const ReduceLaunch& knobs, int64_t nvec) {
+  if (nvec <= 0) return 0;
+  const int threads = reduce_threads_for(knobs, nvec);
+  int64_t nb = (nvec + threads - 1) / threads;
+  if (nb > knobs.max_blocks) nb = knobs.max_blocks;
+  return nb < 1 ? 1 : (int)nb;
+}
+
+// The peers' buffer addresses as kernel arguments.  The reference's kernel reads them from a
+// table in device memory (triton_one_shot_all_reduce.py:87): a dependent memory round trip
+// in front of every thread's first data load, which a launch of a few microseconds notices.
+// A host that knows the addresses passes them by value; all-zero = read the device table.
+struct PeerPtrs {
+  uint64_t p[SMR_MAX_WORLD_SIZE];
+};
 
 struct alignas(16) Vec16 {
   uint32_t w[4];
@@ -123,7 +149,7 @@ __device__ __forceinline__ Vec16 sum_in_rank_order(const Vec16 (&v)[WS]) {
 
 template <int KIND, int WS, bool WRITE_ALL>
 __global__ __launch_bounds__(kReduceMaxThreads) void one_shot_all_reduce_kernel(
-    const uint64_t* __restrict__ buffer_ptrs, const uint64_t* __restrict__ signal_pad_ptrs,
+    const uint64_t* __restrict__ buffer_ptrs, PeerPtrs by_value, const uint64_t* __restrict__ signal_pad_ptrs,
     Vec16* __restrict__ out, int64_t nvec, int rank, int layout, int nblocks, int do_barrier,
     uint64_t limit_ticks, uint32_t* status) {
   int block = blockIdx.x;
@@ -170,8 +196,13 @@ __global__ __launch_bounds__(kReduceMaxThreads) void one_shot_all_reduce_kernel(
   if (do_barrier) blockwise_barrier(signal_pad_ptrs, block, rank, WS, limit_ticks, status, false);
 
   GlobalVec* src[WS];
+  if (buffer_ptrs != nullptr) {
 #pragma unroll
-  for (int r = 0; r < WS; ++r) src[r] = (GlobalVec*)(uintptr_t)buffer_ptrs[r];
+    for (int r = 0; r < WS; ++r) src[r] = (GlobalVec*)(uintptr_t)buffer_ptrs[r];
+  } else {
+#pragma unroll
+    for (int r = 0; r < WS; ++r) src[r] = (GlobalVec*)(uintptr_t)by_value.p[r];
+  }
   GlobalVec* dst = (GlobalVec*)(uintptr_t)out;
 
   const int64_t stride = (int64_t)nblocks * nthreads;
@@ -193,26 +224,27 @@ __global__ __launch_bounds__(kReduceMaxThreads) void one_shot_all_reduce_kernel(
 }
 
 template <int KIND, int WS>
-static int launch_ws(bool write_all, dim3 grid, int threads, hipStream_t s, const uint64_t* bp, const uint64_t* sp,
+static int launch_ws(bool write_all, dim3 grid, int threads, hipStream_t s, const uint64_t* bp,
+                     const PeerPtrs& pv, const uint64_t* sp,
                      Vec16* out, int64_t nvec, int rank, int layout, int nblocks, int do_barrier,
                      uint32_t* status) {
   const uint64_t lim = spin_limit_ticks();
   if (write_all)
     hipLaunchKernelGGL((one_shot_all_reduce_kernel<KIND, WS, true>), grid, dim3(threads), 0, s,
-                       bp, sp, out, nvec, rank, layout, nblocks, do_barrier, lim, status);
+                       bp, pv, sp, out, nvec, rank, layout, nblocks, do_barrier, lim, status);
   else
     hipLaunchKernelGGL((one_shot_all_reduce_kernel<KIND, WS, false>), grid, dim3(threads), 0, s,
-                       bp, sp, out, nvec, rank, layout, nblocks, do_barrier, lim, status);
+                       bp, pv, sp, out, nvec, rank, layout, nblocks, do_barrier, lim, status);
   return check_hip(hipGetLastError(), "smr_one_shot_all_reduce launch");
 }
 
 template <int KIND>
 static int launch_dtype(int ws, bool write_all, dim3 grid, int threads, hipStream_t s, const uint64_t* bp,
-                        const uint64_t* sp, Vec16* out, int64_t nvec, int rank, int layout,
+                        const PeerPtrs& pv, const uint64_t* sp, Vec16* out, int64_t nvec, int rank, int layout,
                         int nblocks, int do_barrier, uint32_t* status) {
 #define SMR_WS_CASE(W)                                                                          \
   case W:                                                                                       \
-    return launch_ws<KIND, W>(write_all, grid, threads, s, bp, sp, out, nvec, rank, layout, nblocks,     \
+    return launch_ws<KIND, W>(write_all, grid, threads, s, bp, pv, sp, out, nvec, rank, layout, nblocks, \
                               do_barrier, status);
   switch (ws) {
     SMR_WS_CASE(1) SMR_WS_CASE(2) SMR_WS_CASE(3) SMR_WS_CASE(4)
@@ -224,33 +256,11 @@ static int launch_dtype(int ws, bool write_all, dim3 grid, int threads, hipStrea
 
 }  // namespace smr
 
-extern "C" {
-
-int smr_set_reduce_launch(int threads, int max_blocks) {
-  if (max_blocks == 0) max_blocks = 256;
-  if (threads != 0 && (threads < 64 || threads > smr::kReduceMaxThreads || (threads & 63) != 0))
-    return smr::fail(SMR_E_INVALID, "smr_set_reduce_launch: threads must be a multiple of 64 in 64..1024");
-  if (max_blocks < 1 || max_blocks > 4096)
-    return smr::fail(SMR_E_INVALID, "smr_set_reduce_launch: max_blocks must be 1..4096");
-  smr::g_reduce_threads = threads;
-  smr::g_reduce_max_blocks = max_blocks;
-  return 0;
-}
-
-int smr_reduce_num_blocks(int64_t numel, int dtype) {
-  const int per_vec = dtype == SMR_DTYPE_FP32 ? 4 : 8;
-  if (numel <= 0) return 0;
-  const int64_t nvec = numel / per_vec;
-  const int threads = smr::reduce_threads_for(nvec);
-  int64_t nb = (nvec + threads - 1) / threads;
-  if (nb > smr::g_reduce_max_blocks) nb = smr::g_reduce_max_blocks;
-  if (nb < 1) nb = 1;
-  return (int)nb;
-}
-
-int smr_one_shot_all_reduce(const uint64_t* buffer_ptrs_dev, const uint64_t* signal_pad_ptrs_dev,
-                            void* out, int64_t numel, int dtype, int rank, int world_size,
-                            int write_all, int barrier_mode, uint32_t* status, void* stream) {
+// Validation and launch behind both entry points: the peers' addresses come either from the
+// device table (`buffer_ptrs_dev`) or, by value, from the host array `buffer_ptrs_host`.
+static int reduce_entry(const uint64_t* buffer_ptrs_dev, const uint64_t* buffer_ptrs_host,
+                        const uint64_t* signal_pad_ptrs_dev, void* out, int64_t numel, int dtype, int rank,
+                        int world_size, int write_all, int barrier_mode, uint32_t* status, void* stream) {
   using namespace smr;
   if (dtype != SMR_DTYPE_BF16 && dtype != SMR_DTYPE_FP32 && dtype != SMR_DTYPE_BF16_STEPWISE)
     return fail(SMR_E_INVALID, "smr_one_shot_all_reduce: dtype must be bf16 (0), fp32 (1) or stepwise bf16 (2)");
@@ -261,8 +271,16 @@ int smr_one_shot_all_reduce(const uint64_t* buffer_ptrs_dev, const uint64_t* sig
   const int per_vec = dtype == SMR_DTYPE_FP32 ? 4 : 8;
   if (numel < 0 || numel % per_vec != 0)
     return fail(SMR_E_INVALID, "smr_one_shot_all_reduce: The number of elements must be 128-bit aligned.");
-  if (buffer_ptrs_dev == nullptr)
-    return fail(SMR_E_INVALID, "smr_one_shot_all_reduce: buffer_ptrs_dev is NULL");
+  if (buffer_ptrs_dev == nullptr && buffer_ptrs_host == nullptr)
+    return fail(SMR_E_INVALID, "smr_one_shot_all_reduce: the buffer address table is NULL");
+  PeerPtrs pv = {};
+  if (buffer_ptrs_host != nullptr) {
+    for (int r = 0; r < world_size; ++r) {
+      if (buffer_ptrs_host[r] == 0 || (buffer_ptrs_host[r] & 15u))
+        return fail(SMR_E_INVALID, "smr_one_shot_all_reduce_addrs: buffer addresses must be non-zero and 16-byte aligned");
+      pv.p[r] = buffer_ptrs_host[r];
+    }
+  }
   if (barrier_mode != SMR_BARRIER_NONE && barrier_mode != SMR_BARRIER_PROXY && barrier_mode != SMR_BARRIER_BOTH)
     return fail(SMR_E_INVALID, "smr_one_shot_all_reduce: unknown barrier_mode");
   if (barrier_mode != SMR_BARRIER_NONE && signal_pad_ptrs_dev == nullptr)
@@ -275,9 +293,10 @@ int smr_one_shot_all_reduce(const uint64_t* buffer_ptrs_dev, const uint64_t* sig
     return fail(SMR_E_INVALID, "smr_one_shot_all_reduce: out must be 16-byte aligned");
   if (numel == 0) return 0;
 
+  const ReduceLaunch knobs = reduce_launch_knobs();       // one consistent pair for the whole call
   const int64_t nvec = numel / per_vec;
-  const int nblocks = smr_reduce_num_blocks(numel, dtype);
-  const int threads = reduce_threads_for(nvec);
+  const int nblocks = reduce_blocks_for(knobs, nvec);
+  const int threads = reduce_threads_for(knobs, nvec);
   const int do_barrier = barrier_mode == SMR_BARRIER_BOTH ? 2 : (barrier_mode != SMR_BARRIER_NONE ? 1 : 0);
   int layout = kPlain;
   unsigned grid = (unsigned)nblocks;
@@ -291,15 +310,50 @@ int smr_one_shot_all_reduce(const uint64_t* buffer_ptrs_dev, const uint64_t* sig
   }
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
   Vec16* o = reinterpret_cast<Vec16*>(out);
+  const uint64_t* table = buffer_ptrs_host != nullptr ? nullptr : buffer_ptrs_dev;
   if (dtype == SMR_DTYPE_BF16)
-    return launch_dtype<SMR_DTYPE_BF16>(world_size, write_all != 0, dim3(grid), threads, s, buffer_ptrs_dev,
+    return launch_dtype<SMR_DTYPE_BF16>(world_size, write_all != 0, dim3(grid), threads, s, table, pv,
                                         signal_pad_ptrs_dev, o, nvec, rank, layout, nblocks, do_barrier, status);
   if (dtype == SMR_DTYPE_BF16_STEPWISE)
-    return launch_dtype<SMR_DTYPE_BF16_STEPWISE>(world_size, write_all != 0, dim3(grid), threads, s,
-                                                 buffer_ptrs_dev, signal_pad_ptrs_dev, o, nvec, rank, layout,
-                                                 nblocks, do_barrier, status);
-  return launch_dtype<SMR_DTYPE_FP32>(world_size, write_all != 0, dim3(grid), threads, s, buffer_ptrs_dev,
-                             signal_pad_ptrs_dev, o, nvec, rank, layout, nblocks, do_barrier, status);
+    return launch_dtype<SMR_DTYPE_BF16_STEPWISE>(world_size, write_all != 0, dim3(grid), threads, s, table, pv,
+                                                 signal_pad_ptrs_dev, o, nvec, rank, layout, nblocks, do_barrier,
+                                                 status);
+  return launch_dtype<SMR_DTYPE_FP32>(world_size, write_all != 0, dim3(grid), threads, s, table, pv,
+                                      signal_pad_ptrs_dev, o, nvec, rank, layout, nblocks, do_barrier, status);
+}
+
+extern "C" {
+
+int smr_set_reduce_launch(int threads, int max_blocks) {
+  if (max_blocks == 0) max_blocks = 256;
+  if (threads != 0 && (threads < 64 || threads > smr::kReduceMaxThreads || (threads & 63) != 0))
+    return smr::fail(SMR_E_INVALID, "smr_set_reduce_launch: threads must be a multiple of 64 in 64..1024");
+  if (max_blocks < 1 || max_blocks > 4096)
+    return smr::fail(SMR_E_INVALID, "smr_set_reduce_launch: max_blocks must be 1..4096");
+  smr::g_reduce_launch.store((uint32_t)threads | ((uint32_t)max_blocks << 16), std::memory_order_relaxed);
+  return 0;
+}
+
+int smr_reduce_num_blocks(int64_t numel, int dtype) {
+  const int per_vec = dtype == SMR_DTYPE_FP32 ? 4 : 8;
+  if (numel <= 0) return 0;
+  return smr::reduce_blocks_for(smr::reduce_launch_knobs(), numel / per_vec);
+}
+
+int smr_one_shot_all_reduce(const uint64_t* buffer_ptrs_dev, const uint64_t* signal_pad_ptrs_dev,
+                            void* out, int64_t numel, int dtype, int rank, int world_size,
+                            int write_all, int barrier_mode, uint32_t* status, void* stream) {
+  return reduce_entry(buffer_ptrs_dev, nullptr, signal_pad_ptrs_dev, out, numel, dtype, rank, world_size,
+                      write_all, barrier_mode, status, stream);
+}
+
+int smr_one_shot_all_reduce_addrs(const uint64_t* buffer_ptrs_host, const uint64_t* signal_pad_ptrs_dev,
+                                  void* out, int64_t numel, int dtype, int rank, int world_size,
+                                  int write_all, int barrier_mode, uint32_t* status, void* stream) {
+  if (buffer_ptrs_host == nullptr)
+    return smr::fail(SMR_E_INVALID, "smr_one_shot_all_reduce_addrs: buffer_ptrs_host is NULL");
+  return reduce_entry(nullptr, buffer_ptrs_host, signal_pad_ptrs_dev, out, numel, dtype, rank, world_size,
+                      write_all, barrier_mode, status, stream);
 }
 
 }  // extern "C"

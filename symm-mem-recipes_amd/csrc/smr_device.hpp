@@ -36,8 +36,13 @@ __device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {
   uint32_t q = (u >> 16) | 0x40u;
   return ((u & 0x7FFFFFFFu) > 0x7F800000u) ? q : r;
 }
+// Two at once through the hardware conversion (v_cvt_pk_bf16_f32: round-to-nearest-even,
+// NaN quieted): one instruction instead of a dozen integer operations per pair.
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef float f32x2_t __attribute__((ext_vector_type(2)));
 __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
-  return f32_to_bf16_bits(lo) | (f32_to_bf16_bits(hi) << 16);
+  const f32x2_t v = {lo, hi};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));
 }
 
 // ---------------------------------------------------------------- status

@@ -38,6 +38,7 @@ SIGNATURES = {
     "smr_get_spin_timeout_us": (_i64, []),
     "smr_set_trace_buffer": (_i, [_p, _i64]),
     "smr_one_shot_all_reduce": (_i, [_p, _p, _p, _i64, _i, _i, _i, _i, _i, _p, _p]),
+    "smr_one_shot_all_reduce_addrs": (_i, [_p, _p, _p, _i64, _i, _i, _i, _i, _i, _p, _p]),
     "smr_reduce_num_blocks": (_i, [_i64, _i]),
     "smr_set_reduce_launch": (_i, [_i, _i]),
     "smr_barrier": (_i, [_p, _i, _i, _i, _i, _i, _p, _p]),
@@ -56,6 +57,7 @@ SIGNATURES = {
     "smr_ag_matmul_schedule": (_i, [_i, _i, _i, _i, _i, _i, _i, _p, _i]),
     "smr_ag_matmul_grid": (_i, [_i, _i, _i, _i, _i, _i]),
     "smr_set_ag_matmul_halves": (_i, [_i, _i]),
+    "smr_set_ag_matmul_grid_limit": (_i, [_i]),
     "smr_ag_matmul_plan": (_i, [_i, _i, _i, _i, _i, _p]),
     "smr_ag_matmul_fp8": (_i, [_p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _p, _p]),
     "smr_ag_matmul_plan_fp8": (_i, [_i, _i, _i, _i, _i, _p]),

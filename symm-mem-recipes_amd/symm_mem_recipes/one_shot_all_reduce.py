@@ -24,7 +24,7 @@ def num_blocks(numel: int, dtype: torch.dtype = torch.bfloat16) -> int:
 
 def one_shot_all_reduce(tensor: torch.Tensor, *, barrier: bool = True, write_all: bool = False,
                         all_ranks: bool = False, accumulate: str = "fp32",
-                        trailing_barrier: bool = False) -> torch.Tensor:
+                        trailing_barrier: bool = False, device_table: bool = False) -> torch.Tensor:
     """Sum the symmetric buffers of all ranks element-wise (fp32 accumulator,
     rank order 0..world_size-1) and return the calling rank's result.
 
@@ -42,6 +42,10 @@ def one_shot_all_reduce(tensor: torch.Tensor, *, barrier: bool = True, write_all
     ``trailing_barrier`` a second handshake after the last store (the reference
                    has none behind triton_one_shot_all_reduce.py:93): no peer
                    can overwrite its buffer while another still reads it.
+    ``device_table`` let the kernel read the peers' addresses from the table in device
+                   memory, as the reference's does (triton_one_shot_all_reduce.py:86-87);
+                   by default they are passed as kernel arguments, which saves every
+                   thread a dependent load in front of its first data load.
     ``accumulate`` "fp32" (default) keeps an fp32 accumulator and rounds once;
                    "bf16" rounds the accumulator to bf16 after every add, which is
                    bit for bit the reference's add.bf16x2 chain
@@ -72,8 +76,10 @@ def one_shot_all_reduce(tensor: torch.Tensor, *, barrier: bool = True, write_all
     else:
         output = torch.empty_like(tensor)
         out_ptr = output.data_ptr()
-    rc = lib.smr_one_shot_all_reduce(
-        symm_mem.buffer_ptrs_dev,
+    entry, table = ((lib.smr_one_shot_all_reduce, symm_mem.buffer_ptrs_dev) if device_table
+                    else (lib.smr_one_shot_all_reduce_addrs, symm_mem.buffer_ptrs_host))
+    rc = entry(
+        table,
         symm_mem.signal_pad_ptrs_dev,
         out_ptr,
         tensor.numel(),

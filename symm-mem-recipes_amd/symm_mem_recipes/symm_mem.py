@@ -13,6 +13,7 @@ rank is process-wide state (``set_rank``), since one process plays every rank.
 """
 from __future__ import annotations
 
+import ctypes
 import math
 import os
 from typing import Dict, List, Optional, Sequence, Tuple
@@ -67,6 +68,8 @@ class _Group:
         pbase = self.pads.data_ptr()
         self.buffer_addrs = [base + r * self.buffer_stride for r in range(world_size)]
         self.pad_addrs = [pbase + r * SIGNAL_PAD_SIZE for r in range(world_size)]
+        # the same addresses as a host array, for entry points that take them by value
+        self.buffer_addrs_host = (ctypes.c_uint64 * _lib.MAX_WORLD_SIZE)(*self.buffer_addrs)
         self.buffer_ptrs = torch.tensor(self.buffer_addrs, dtype=torch.int64, device=device)
         self.pad_ptrs = torch.tensor(self.pad_addrs, dtype=torch.int64, device=device)
         self.status = torch.zeros(_lib.STATUS_WORDS, dtype=torch.int32, device=device)
@@ -94,6 +97,11 @@ class EmulatedSymmetricMemory:
     @property
     def signal_pad_ptrs_dev(self) -> int:
         return self._group.pad_ptrs.data_ptr()
+
+    @property
+    def buffer_ptrs_host(self):
+        """ctypes array of the ranks' buffer addresses in host memory."""
+        return self._group.buffer_addrs_host
 
     @property
     def buffer_ptrs(self) -> List[int]:

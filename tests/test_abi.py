@@ -63,6 +63,17 @@ def test_reduce_argument_errors_before_launch(lib):
     assert bad(p, p, p + 4, 16, 0, 0, 8, 0, 0, None, None) == -1   # misaligned output
     assert bad(p, p, None, 16, 0, -1, 8, 1, 0, None, None) == -1   # write_all needs a rank
     assert bad(p, p, p, 0, 0, 0, 8, 0, 0, None, None) == 0         # empty message: no launch
+    # the variant that takes the addresses from a host array
+    by_value = lib.smr_one_shot_all_reduce_addrs
+    addrs = (ctypes.c_uint64 * 8)(*[0x10000 * (r + 1) for r in range(8)])
+    assert by_value(None, p, p, 16, 0, 0, 8, 0, 0, None, None) == -1
+    assert by_value(addrs, p, p, 12, 0, 0, 8, 0, 0, None, None) == -1
+    assert by_value(addrs, p, p, 0, 0, 0, 8, 0, 0, None, None) == 0
+    addrs[5] = 0x10008                                             # not 16-byte aligned
+    assert by_value(addrs, p, p, 16, 0, 0, 8, 0, 0, None, None) == -1
+    assert b"16-byte aligned" in lib.smr_last_error_string()
+    addrs[5] = 0
+    assert by_value(addrs, p, p, 16, 0, 0, 8, 0, 0, None, None) == -1
 
 
 def test_barrier_argument_errors(lib):

@@ -68,12 +68,15 @@ def test_known_answer_ones(cuda):
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
 @pytest.mark.parametrize("nbytes", [16, 4096, 16 << 10, 64 << 10, (1 << 20) + 16 * 37, 2 << 20])
 @pytest.mark.parametrize("barrier", [True, False])
-def test_parity_single_output(cuda, dtype, nbytes, barrier):
+@pytest.mark.parametrize("device_table", [False, True], ids=["addrs-by-value", "device-table"])
+def test_parity_single_output(cuda, dtype, nbytes, barrier, device_table):
+    """Both ways the kernel learns the peers' addresses: as kernel arguments (the default) and
+    from the table in device memory, as the reference's kernel does."""
     from symm_mem_recipes import one_shot_all_reduce
     numel = nbytes // (2 if dtype == torch.bfloat16 else 4)
     t, h = _alloc(numel, dtype, cuda, rank=3)
     bufs = _fill(h, numel, dtype)
-    out = one_shot_all_reduce(t, barrier=barrier)
+    out = one_shot_all_reduce(t, barrier=barrier, device_table=device_table)
     h.check_status()
     want = O.reduce_ref(bufs, "bf16" if dtype == torch.bfloat16 else "fp32")
     assert _same(_bits(out), want)
