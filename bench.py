@@ -405,9 +405,8 @@ def main():
     ap.add_argument("--no-extra", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=10.0)
     ap.add_argument("--gemm-only", action="store_true",
-                    help="only the ungated GEMM and the library matmul of the same operands: the run to "
-                         "collect hardware counters on (a counter run serialises kernels, and a gated GEMM "
-                         "whose producer cannot run beside it only times out)")
+                    help="only the GEMM of the all-gather matmul (ungated, the library's matmul of the same "
+                         "operands, and the fused launch): the run to collect hardware counters on")
     ap.add_argument("--fp8", action="store_true", help="with --gemm-only: the e4m3fn GEMM instead of the bf16 one")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -423,7 +422,7 @@ def main():
     torch.cuda.set_device(dev)
 
     if args.gemm_only:
-        print(json.dumps(bench_ag_matmul_fp8(dev, gated=False) if args.fp8 else bench_ag_matmul(dev, gated=False)))
+        print(json.dumps(bench_ag_matmul_fp8(dev) if args.fp8 else bench_ag_matmul(dev)))
         return
 
     r = bench_reduce(args.size_mib, args.steps, args.warmup, dev)

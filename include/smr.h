@@ -176,14 +176,6 @@ int smr_all_gather_with_progress(const uint64_t* buffer_ptrs_dev, void* a_out_de
                                  int world_size, int64_t shard_bytes, int splits_per_rank,
                                  int num_workgroups, void* stream);
 
-/* The producer starting at the first_chunk-th chunk of its walk (0 = all of it): the
- * chunks before are delivered by someone else, smr_ag_matmul_pull_first's workgroups
- * for the first one.  Their flags and their part of a_out are not touched. */
-int smr_all_gather_with_progress_from(const uint64_t* buffer_ptrs_dev, void* a_out_dev,
-                                      uint32_t* progress_dev, uint32_t* counters_dev, int rank,
-                                      int world_size, int64_t shard_bytes, int splits_per_rank,
-                                      int first_chunk, int num_workgroups, void* stream);
-
 /* The same gather for a caller that does not watch the flags on the way (a GEMM queued
  * behind it in stream order): all chunks are copied together and every flag is raised at
  * the end.  Same arguments and the same final state of a_out, progress and counters as
@@ -219,24 +211,33 @@ int smr_ag_matmul(const void* a_shard_dev, const void* a_out_dev, const void* b_
 int smr_ag_matmul_schedule(int M, int N, int K, int rank, int world_size, int comm_block_m,
                            int gated, int32_t* out_records, int max_tiles);
 
-/* smr_ag_matmul (elem_bytes 2) or smr_ag_matmul_fp8 (elem_bytes 1), gated, whose
- * workgroups copy the first remote chunk themselves.  Half the grid of a gated launch
- * starts on the first remote comm block and would wait for the producer to deliver it;
- * those workgroups are idle compute units, so the grid pulls the chunk from
- * buffer_ptrs_dev[rank + 1] into a_out first (64 KiB pieces taken by ticket, so a workgroup
- * that is dispatched late holds nobody up), the one that completes it raises
- * progress[(rank + 1) * splits], and the producer is started at its second chunk
- * (smr_all_gather_with_progress_from, first_chunk = 1).  The reference's copy engines
- * deliver every chunk (triton_all_gather_matmul.py:41-55); this is the part of that loop
- * the consumer takes over when the copy has to run on compute units.
- *   pull_counters_dev  uint32 [2], zero on entry (not restored: zero them before every call)
- * Returns the number of pulling workgroups (> 0: start the producer at chunk 1), 0 when
- * too few workgroups would wait for pulling to pay (plain gated launch: start the producer
- * at chunk 0), or a negative SMR_E_* code. */
-int smr_ag_matmul_pull_first(const void* a_shard_dev, void* a_out_dev, const void* b_nk_dev, void* c_dev,
-                             uint32_t* progress_dev, uint32_t* pull_counters_dev,
-                             const uint64_t* buffer_ptrs_dev, int elem_bytes, int M, int N, int K, int rank,
-                             int world_size, int comm_block_m, uint32_t* status, void* stream);
+/* The whole all-gather matmul in one launch on one stream.  Replaces the body of
+ * all_gather_matmul_tma_persistent (symm_mem_recipes/triton_all_gather_matmul.py:246-318:
+ * fresh flags, producer on a second stream, persistent GEMM, stream join).  The reference's
+ * producer is a copy engine and costs no SMs; on one GPU the copy runs on compute units, and
+ * here it runs inside the GEMM's own grid:
+ *   - `producer_workgroups` extra workgroups (0 = the plan's, see smr_ag_matmul_plan) only
+ *     copy: the peers' shards from buffer_ptrs_dev into a_out in the reference's order
+ *     (sources rank+1, ..., rank+ws-1, rank; :43-44), in 64 KiB pieces taken by ticket;
+ *   - a GEMM workgroup whose next tile's chunk is not in place takes pieces of that chunk
+ *     too instead of spinning, so the launch finishes whichever of its workgroups are
+ *     resident, and needs no second stream and no kernel running beside it;
+ *   - pull_first 1: every GEMM workgroup starts by copying at the first remote chunk (as many
+ *     workgroups begin on that comm block as on the local one); 0: never; -1: when at least
+ *     48 workgroups would otherwise start with a wait.
+ *   elem_bytes 2 = smr_ag_matmul's arithmetic (bf16), 1 = smr_ag_matmul_fp8's (e4m3fn).
+ *   state_dev  uint32 [smr_ag_matmul_fused_state_words(ws, splits)]: flags, tickets and
+ *              counters.  Zero before the first launch; the last workgroup to finish zeroes
+ *              it again, so the next launch (or the next replay of a captured graph) needs no
+ *              fill.  One launch at a time per state array; after a launch that reported a
+ *              timeout in `status` the caller must zero it.
+ * On return a_out holds all ws shards and c the product; c is identical, bit for bit, to
+ * smr_ag_matmul on the gathered operand. */
+int smr_ag_matmul_fused(const void* a_shard_dev, void* a_out_dev, const void* b_nk_dev, void* c_dev,
+                        uint32_t* state_dev, const uint64_t* buffer_ptrs_dev, int elem_bytes, int M,
+                        int N, int K, int rank, int world_size, int comm_block_m,
+                        int producer_workgroups, int pull_first, uint32_t* status, void* stream);
+int smr_ag_matmul_fused_state_words(int world_size, int splits_per_rank);
 
 /* The same GEMM with e4m3fn (OCP FP8) operands and result, fp32 accumulation: the
  * reference's FP8_OUTPUT switch (triton_all_gather_matmul.py:115,123,188,311).  The cast of

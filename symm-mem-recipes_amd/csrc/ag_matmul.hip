@@ -24,8 +24,9 @@
 //     one pass over the grid, XCD x (workgroups with id % 8 == x) takes a
 //     contiguous run of the tile order - a patch about as wide as it is high - so
 //     the workgroups that share an L2 also share A rows and B columns;
-//   * a launch wide enough that many workgroups would start with a wait copies the
-//     first remote chunk itself before its first tiles (pull_first_chunk);
+//   * a fused launch gathers the peers' shards itself (CopyJob): extra workgroups of the
+//     same grid only copy, and a GEMM workgroup that finds its tile's chunk missing copies
+//     along instead of spinning;
 //   * the same kernel in e4m3fn (run_tile_fp8): the bytes move the same way, the
 //     tile is built from v_mfma_f32_32x32x64_f8f6f4.
 #include <type_traits>
@@ -705,87 +706,168 @@ __device__ __forceinline__ void run_tile_fp8(const TileContext& cx, const TileRe
   }
 }
 
-// The first remote chunk, pulled by the GEMM's own workgroups before their first tile.
-// A gated launch puts as many workgroups on the first remote comm block as on the
-// local one, and a producer that owns an eighth of the GPU needs a third of a tile's
-// time to deliver that chunk; every workgroup has the same number of tiles, so the
-// launch ends late by that wait.  Instead the grid copies the chunk first (32 MiB in
-// about 15 us), the workgroup that completes it raises the flag, and the producer
-// starts at the second chunk, which it delivers long before the second pass.
+// The gather done by the launch itself.  The reference's copy engines deliver every chunk and
+// cost no SMs (triton_all_gather_matmul.py:41-55); on one GPU the copy runs on compute units,
+// and here it runs inside the GEMM's own launch: workgroups [gemm_grid, gridDim.x) do nothing
+// but copy, in the reference's chunk order, and a GEMM workgroup whose next tile's chunk is
+// not there yet copies along instead of spinning.  One launch, one stream, no flag fill.
 //
-// The chunk is cut into 64 KiB pieces that the workgroups take by ticket until none
-// is left, so nothing depends on how many workgroups are running: one that is
-// dispatched late (another kernel holds its compute unit) finds the pieces gone and
-// goes on to its tiles, and the ones that are there do all of the copying.
-struct PullFirst {
-  const uint64_t* buffer_ptrs;   // the ranks' shard addresses (device array); nullptr = off
-  uint8_t* dst;                  // the chunk's place in the gathered operand
-  uint32_t* flag;                // its progress flag
-  uint32_t* counters;            // [0] tickets, [1] finished pieces; zero on entry
-  int64_t vecs;                  // 16-byte vectors in the chunk
-  int src_rank, comm_block, pieces;
+// Every chunk is cut into 64 KiB pieces that are taken by ticket until none is left, so
+// nothing depends on which workgroups are running: a copy-only workgroup that is dispatched
+// late (another kernel holds its compute unit) finds the pieces gone, and if none of them
+// ever runs the GEMM's workgroups copy everything themselves, only later.  Pieces are written
+// through to memory; whoever completes a chunk's count raises its flag.
+//
+// A launch wide enough that many workgroups would start with a wait has all of its GEMM
+// workgroups copy the first remote chunk before their first tiles (32 MiB in about 15 us):
+// as many workgroups sit on the first remote comm block as on the local one and all have the
+// same number of tiles, so the launch would end late by whatever the later half waits.
+//
+// State (uint32 words, zero before the first launch): flags[chunks], tickets[chunks],
+// finished[chunks], exits[1].  The last workgroup to leave zeroes all of it, so the next
+// launch - or the next replay of a captured graph - starts from zero again with no fill.
+struct CopyJob {
+  const uint64_t* buffer_ptrs;   // the ranks' shard addresses (device array); nullptr = this launch copies nothing
+  uint8_t* a_out;                // the gathered operand
+  uint32_t* flags;               // progress flags, one per chunk
+  uint32_t* tickets;             // next piece of a chunk
+  uint32_t* finished;            // pieces of a chunk that are in place
+  uint32_t* exits;               // workgroups that are through
+  int64_t chunk_vecs;            // 16-byte vectors per chunk
+  int pieces;                    // per chunk
+  int chunks, splits, rank, world_size;
+  int gemm_grid;                 // workgroups from here on only copy
+  int pull_chunk;                // chunk every GEMM workgroup copies at before its first tile, or -1
 };
 
 typedef __attribute__((address_space(1))) u32x4 GlobalVec;
+typedef __attribute__((address_space(3))) uint32_t LdsWord;
 constexpr int kPullInFlight = 16;                               // 128-bit loads per thread and piece
 constexpr int kPullPieceVecs = kGemmThreads * kPullInFlight;    // 64 KiB
 
-__device__ __forceinline__ void pull_first_chunk(const PullFirst& pf, uint32_t lds0) {
-  typedef __attribute__((address_space(3))) uint32_t LdsWord;
-  LdsWord* slot = reinterpret_cast<LdsWord*>((uintptr_t)lds0);   // the tile ring is not in use yet
-  // a ticket for the whole workgroup: thread 0 draws it, the others read it
+// One value from thread 0 to the whole workgroup through the first word of the tile ring
+// (not in use where this is called: before a tile's first loads).
+template <typename F>
+__device__ __forceinline__ uint32_t from_thread0(uint32_t lds0, F&& f) {
+  LdsWord* slot = reinterpret_cast<LdsWord*>((uintptr_t)lds0);
+  if (threadIdx.x == 0) *slot = f();
+  __syncthreads();
+  const uint32_t v = *slot;
+  __syncthreads();
+  return v;
+}
+
+// Takes pieces of chunk `c` by ticket and copies them until none is left.  SETS = 2 keeps two
+// pieces in flight (a copy-only workgroup has the registers; 128 KiB per compute unit is what
+// a streaming copy needs), SETS = 1 one (a GEMM workgroup between two tiles).
+template <int SETS>
+__device__ __forceinline__ void copy_pieces(const CopyJob& job, int c, uint32_t lds0, uint64_t* trace) {
+  const GlobalVec* src = (const GlobalVec*)(uintptr_t)job.buffer_ptrs[c / job.splits] +
+                         (int64_t)(c % job.splits) * job.chunk_vecs;
+  GlobalVec* dst = (GlobalVec*)(uintptr_t)job.a_out + (int64_t)c * job.chunk_vecs;
+  const uint32_t pieces = (uint32_t)job.pieces;
   auto draw = [&]() -> uint32_t {
-    if (threadIdx.x == 0) *slot = __hip_atomic_fetch_add(&pf.counters[0], 1u, __ATOMIC_RELAXED, kScope);
-    __syncthreads();
-    const uint32_t t = *slot;
-    __syncthreads();
-    return t;
+    return from_thread0(lds0, [&]() { return __hip_atomic_fetch_add(&job.tickets[c], 1u, __ATOMIC_RELAXED, kScope); });
   };
-  const GlobalVec* src = (const GlobalVec*)(uintptr_t)pf.buffer_ptrs[pf.src_rank];
-  GlobalVec* dst = (GlobalVec*)(uintptr_t)pf.dst;
-  uint32_t mine = 0;
-  uint32_t t = draw();
-  while (t < (uint32_t)pf.pieces) {
+  auto load = [&](u32x4 (&v)[kPullInFlight], uint32_t t) {
     const int64_t i0 = (int64_t)t * kPullPieceVecs + threadIdx.x;
-    u32x4 v[kPullInFlight];
 #pragma unroll
     for (int u = 0; u < kPullInFlight; ++u) {
       const int64_t i = i0 + u * kGemmThreads;
-      v[u] = __builtin_nontemporal_load(src + (i < pf.vecs ? i : pf.vecs - 1));
+      v[u] = __builtin_nontemporal_load(src + (i < job.chunk_vecs ? i : job.chunk_vecs - 1));
     }
-    // the next ticket is drawn while this piece's loads are in flight
-    t = draw();
+  };
+  auto store = [&](const u32x4 (&v)[kPullInFlight], uint32_t t) {
+    const int64_t i0 = (int64_t)t * kPullPieceVecs + threadIdx.x;
 #pragma unroll
     for (int u = 0; u < kPullInFlight; ++u) {
       const int64_t i = i0 + u * kGemmThreads;
-      if (i < pf.vecs)
+      if (i < job.chunk_vecs)
         asm volatile("global_store_dwordx4 %0, %1, off sc1" : : "v"(dst + i), "v"(v[u]) : "memory");
     }
-    ++mine;
+  };
+  uint32_t mine = 0;
+  u32x4 v0[kPullInFlight];
+  uint32_t t0 = draw();
+  if (t0 < pieces) load(v0, t0);
+  if constexpr (SETS == 2) {
+    u32x4 v1[kPullInFlight];
+    while (t0 < pieces) {
+      // the next ticket is drawn, and its piece's loads issued, while this piece's are in flight
+      const uint32_t t1 = draw();
+      if (t1 < pieces) load(v1, t1);
+      store(v0, t0);
+      ++mine;
+      if (t1 >= pieces) break;
+      t0 = draw();
+      if (t0 < pieces) load(v0, t0);
+      store(v1, t1);
+      ++mine;
+    }
+  } else {
+    while (t0 < pieces) {
+      const uint32_t t1 = draw();
+      store(v0, t0);
+      ++mine;
+      t0 = t1;
+      if (t0 < pieces) load(v0, t0);
+    }
   }
   if (mine == 0) return;
   // written through: once acknowledged the pieces are where every XCD reads them
   wait_stores_acknowledged();
   __syncthreads();
   if (threadIdx.x == 0) {
-    const uint32_t prev = __hip_atomic_fetch_add(&pf.counters[1], mine, __ATOMIC_RELAXED, kScope);
-    if (prev + mine == (uint32_t)pf.pieces) __hip_atomic_store(pf.flag, 1u, __ATOMIC_RELAXED, kScope);
+    const uint32_t prev = __hip_atomic_fetch_add(&job.finished[c], mine, __ATOMIC_RELAXED, kScope);
+    if (prev + mine == pieces) {
+      __hip_atomic_store(&job.flags[c], 1u, __ATOMIC_RELAXED, kScope);
+      if (trace != nullptr && c < kTraceProducerWords - 1) trace[c] = wall_clock64();
+    }
   }
+}
+
+// A workgroup is through: the last one puts the launch's state back to zero.
+__device__ __forceinline__ void leave(const CopyJob& job) {
+  if (threadIdx.x != 0) return;
+  const uint32_t prev = __hip_atomic_fetch_add(job.exits, 1u, __ATOMIC_RELAXED, kScope);
+  if (prev + 1u != gridDim.x) return;
+  // every other workgroup's last access to these words lies before its count above
+  for (int c = 0; c < job.chunks; ++c) {
+    __hip_atomic_store(&job.flags[c], 0u, __ATOMIC_RELAXED, kScope);
+    __hip_atomic_store(&job.tickets[c], 0u, __ATOMIC_RELAXED, kScope);
+    __hip_atomic_store(&job.finished[c], 0u, __ATOMIC_RELAXED, kScope);
+  }
+  __hip_atomic_store(job.exits, 0u, __ATOMIC_RELAXED, kScope);
 }
 
 template <int BM, int BN, bool FP8 = false>
 __global__ __launch_bounds__(kGemmThreads, 1) void ag_matmul_kernel(
     const uint8_t* __restrict__ a_shard, const uint8_t* __restrict__ a_out,
-    const uint8_t* __restrict__ b_nk, uint8_t* __restrict__ c, const uint32_t* __restrict__ progress,
-    GemmSchedule s, uint64_t limit_ticks, uint32_t* status, uint64_t* trace, PullFirst pf) {
+    const uint8_t* __restrict__ b_nk, uint8_t* __restrict__ c, const uint32_t* progress,
+    GemmSchedule s, uint64_t limit_ticks, uint32_t* status, uint64_t* trace, CopyJob job) {
   __shared__ __attribute__((aligned(1024))) uint8_t lds[GemmTile<BM, BN>::kLdsBytes];
+  const uint32_t lds0 = lds_offset_of(lds);
+
+  // Copy-only workgroups of a fused launch: the chunks in the reference's order (sources
+  // rank+1, ..., rank+ws-1, rank: triton_all_gather_matmul.py:43-44), then out.
+  if (job.buffer_ptrs != nullptr && (int)blockIdx.x >= job.gemm_grid) {
+    if (trace != nullptr && (int)blockIdx.x == job.gemm_grid && threadIdx.x == 0)
+      trace[kTraceProducerWords - 1] = wall_clock64();
+    for (int step = 0; step < job.world_size; ++step) {
+      const int src_rank = (job.rank + step + 1) % job.world_size;
+      for (int split = 0; split < job.splits; ++split)
+        copy_pieces<2>(job, src_rank * job.splits + split, lds0, trace);
+    }
+    leave(job);
+    return;
+  }
 
   TileContext cx;
   cx.lane = threadIdx.x & 63;
   cx.wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   cx.row_stride = (uint32_t)s.K * (FP8 ? 1u : 2u);        // K values per row, 1 or 2 bytes each
   cx.nk = (int)(cx.row_stride / kRowBytes);
-  cx.lds0 = lds_offset_of(lds);
+  cx.lds0 = lds0;
   cx.N = s.N;
   cx.c = c;
 
@@ -794,19 +876,26 @@ __global__ __launch_bounds__(kGemmThreads, 1) void ag_matmul_kernel(
   auto a_rows_of = [&](const TileRef& t) -> const uint8_t* {
     if (t.local) return a_shard + (int64_t)t.a_row * cx.row_stride;
     if (progress != nullptr) {
+      const uint32_t* flag = progress + t.comm_block;
+      // A launch that gathers for itself: if the chunk is not there, take part in copying it.
+      bool up = false;
+      if (job.buffer_ptrs != nullptr) {
+        up = from_thread0(lds0, [&]() { return __hip_atomic_load(flag, __ATOMIC_RELAXED, kScope) == 1u ? 1u : 0u; }) != 0u;
+        if (!up) copy_pieces<1>(job, t.comm_block, lds0, trace);
+      }
       // Thread 0 polls the flag past the caches, the workgroup meets, and only then are the
       // rows' loads issued.  No cache is invalidated here: a line of this comm block can sit
       // in this compute unit's L1 or this XCD's L2 only if somebody read or wrote it since
       // the kernel began (the dispatch itself starts from invalidated caches), nobody reads
-      // a comm block's rows before its flag, and whoever wrote them (the producer, or the
-      // grid pulling the first chunk) wrote whole lines through to memory and saw them
+      // a comm block's rows before its flag, and whoever wrote them (a producer, or this
+      // launch's own copying) wrote whole lines through to memory and saw them
       // acknowledged before the flag went up.  The invalidate an acquire fence stands for
       // would throw out the XCD's shared A and B lines at every tile instead: 2 % of the
       // fused launch.  smr_set_ag_matmul_acquire(1) puts the fence back.
       if (s.acquire) {
-        wait_signal(progress + t.comm_block, limit_ticks, status, t.comm_block);
-      } else {
-        if (threadIdx.x == 0 && !wait_flag_set(progress + t.comm_block, limit_ticks))
+        wait_signal(flag, limit_ticks, status, t.comm_block);
+      } else if (!up) {
+        if (threadIdx.x == 0 && !wait_flag_set(flag, limit_ticks))
           report(status, SMR_ST_WAIT_TIMEOUT, t.comm_block, blockIdx.x, 0u);
         __syncthreads();
       }
@@ -820,7 +909,7 @@ __global__ __launch_bounds__(kGemmThreads, 1) void ag_matmul_kernel(
   bool have = next_tile(s, blockIdx.x, step, tile);
   const uint8_t* a_base = nullptr;
   const uint8_t* b_base = nullptr;
-  if (pf.buffer_ptrs != nullptr) pull_first_chunk(pf, cx.lds0);
+  if (job.buffer_ptrs != nullptr && job.pull_chunk >= 0) copy_pieces<1>(job, job.pull_chunk, lds0, trace);
   if (have) {
     a_base = a_rows_of(tile);
     b_base = b_nk + (int64_t)tile.col0 * cx.row_stride;
@@ -871,6 +960,7 @@ __global__ __launch_bounds__(kGemmThreads, 1) void ag_matmul_kernel(
     b_base = b_next;
     preloaded = true;
   }
+  if (job.buffer_ptrs != nullptr) leave(job);
 }
 
 // Tile shape: the largest the flags' granularity allows, stepped down while the
@@ -1055,10 +1145,18 @@ static int first_chunk_waiters(const smr::GemmSchedule& s, int comm_block) {
 // With fewer workgroups waiting for the first remote chunk the copy is left to the producer.
 constexpr int kMinPullHelpers = 48;
 
+// What a fused launch adds to the GEMM's: who copies (see CopyJob).
+struct FusedArgs {
+  const uint64_t* buffer_ptrs_dev;
+  uint32_t* state_dev;           // flags, tickets, finished, exits
+  int producer_wgs;              // copy-only workgroups; 0 = the plan's
+  int pull_first;                // 1 / 0 / -1 = decide by the number of workgroups that would wait
+};
+
 static int launch_gemm(int elem_bytes, const void* a_shard_dev, const void* a_out_dev, const void* b_nk_dev,
                        void* c_dev, const uint32_t* progress_dev, int M, int N, int K, int rank,
                        int world_size, int comm_block_m, uint32_t* status, void* stream,
-                       const uint64_t* buffer_ptrs_dev, uint32_t* pull_counters_dev, int* helpers_out) {
+                       const FusedArgs* fused) {
   using namespace smr;
   if (a_shard_dev == nullptr || a_out_dev == nullptr || b_nk_dev == nullptr || c_dev == nullptr)
     return fail(SMR_E_INVALID, elem_bytes == 1 ? "smr_ag_matmul_fp8: null pointer" : "smr_ag_matmul: null pointer");
@@ -1066,8 +1164,9 @@ static int launch_gemm(int elem_bytes, const void* a_shard_dev, const void* a_ou
        reinterpret_cast<uintptr_t>(b_nk_dev) | reinterpret_cast<uintptr_t>(c_dev)) & 15u)
     return fail(SMR_E_INVALID, elem_bytes == 1 ? "smr_ag_matmul_fp8: operands must be 16-byte aligned"
                                                : "smr_ag_matmul: operands must be 16-byte aligned");
-  const GemmSchedule s = make_schedule(M, N, K, rank, world_size, comm_block_m, cu_count(),
-                                       progress_dev != nullptr, elem_bytes);
+  const int cus = cu_count();
+  const GemmSchedule s = make_schedule(M, N, K, rank, world_size, comm_block_m, cus,
+                                       progress_dev != nullptr || fused != nullptr, elem_bytes);
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
   const uint8_t* a0 = reinterpret_cast<const uint8_t*>(a_shard_dev);
   const uint8_t* a1 = reinterpret_cast<const uint8_t*>(a_out_dev);
@@ -1075,43 +1174,60 @@ static int launch_gemm(int elem_bytes, const void* a_shard_dev, const void* a_ou
   uint8_t* c = reinterpret_cast<uint8_t*>(c_dev);
   const uint64_t lim = spin_limit_ticks();
   uint64_t* tb = trace_buffer(kTraceProducerWords + kTraceGemmWords);
-  PullFirst pf = {};
-  if (buffer_ptrs_dev != nullptr && world_size > 1) {
-    // the producer's first chunk: split 0 of rank + 1
+  CopyJob job = {};
+  unsigned grid = (unsigned)s.grid;
+  if (fused != nullptr) {
     const int splits = (M / world_size) / comm_block_m;
-    const int src_rank = (rank + 1) % world_size;
-    const int waiters = first_chunk_waiters(s, src_rank * splits);
-    if (waiters >= kMinPullHelpers) {
-      const int64_t chunk_bytes = (int64_t)comm_block_m * K * elem_bytes;
-      pf.buffer_ptrs = buffer_ptrs_dev;
-      pf.dst = const_cast<uint8_t*>(a1) + (int64_t)src_rank * splits * chunk_bytes;
-      pf.flag = const_cast<uint32_t*>(progress_dev) + src_rank * splits;
-      pf.counters = pull_counters_dev;
-      pf.vecs = chunk_bytes / 16;
-      pf.src_rank = src_rank;
-      pf.comm_block = src_rank * splits;
-      pf.pieces = (int)((pf.vecs + kPullPieceVecs - 1) / kPullPieceVecs);
+    const int chunks = world_size * splits;
+    const int64_t chunk_bytes = (int64_t)comm_block_m * K * elem_bytes;
+    job.buffer_ptrs = fused->buffer_ptrs_dev;
+    job.a_out = const_cast<uint8_t*>(a1);
+    job.flags = fused->state_dev;
+    job.tickets = fused->state_dev + chunks;
+    job.finished = fused->state_dev + 2 * chunks;
+    job.exits = fused->state_dev + 3 * chunks;
+    job.chunk_vecs = chunk_bytes / 16;
+    job.pieces = (int)((job.chunk_vecs + kPullPieceVecs - 1) / kPullPieceVecs);
+    job.chunks = chunks;
+    job.splits = splits;
+    job.rank = rank;
+    job.world_size = world_size;
+    job.gemm_grid = s.grid;
+    job.pull_chunk = -1;
+    if (world_size > 1) {
+      // the first remote chunk of the walk: split 0 of rank + 1
+      const int first = ((rank + 1) % world_size) * splits;
+      const bool pull = fused->pull_first > 0 ||
+                        (fused->pull_first < 0 && first_chunk_waiters(s, first) >= kMinPullHelpers);
+      if (pull) job.pull_chunk = first;
     }
+    int producers = fused->producer_wgs > 0 ? fused->producer_wgs
+                                            : estimate_fused(s, cus, s.grid, elem_bytes).producer_wgs;
+    // a workgroup of this kernel fills a compute unit: more of them than there are compute
+    // units would only queue up behind the GEMM's
+    if (producers > cus - s.grid) producers = cus - s.grid;
+    if (producers < 0) producers = 0;
+    grid += (unsigned)producers;
+    progress_dev = job.flags;
   }
-  if (helpers_out != nullptr) *helpers_out = pf.pieces > 0 ? s.grid : 0;
   if (elem_bytes == 1 && s.BM == 256 && s.BN == 256)
-    hipLaunchKernelGGL((ag_matmul_kernel<256, 256, true>), dim3(s.grid), dim3(kGemmThreads), 0, st, a0, a1, b,
-                       c, progress_dev, s, lim, status, tb, pf);
+    hipLaunchKernelGGL((ag_matmul_kernel<256, 256, true>), dim3(grid), dim3(kGemmThreads), 0, st, a0, a1, b,
+                       c, progress_dev, s, lim, status, tb, job);
   else if (elem_bytes == 1 && s.BM == 256)
-    hipLaunchKernelGGL((ag_matmul_kernel<256, 128, true>), dim3(s.grid), dim3(kGemmThreads), 0, st, a0, a1, b,
-                       c, progress_dev, s, lim, status, tb, pf);
+    hipLaunchKernelGGL((ag_matmul_kernel<256, 128, true>), dim3(grid), dim3(kGemmThreads), 0, st, a0, a1, b,
+                       c, progress_dev, s, lim, status, tb, job);
   else if (elem_bytes == 1)
-    hipLaunchKernelGGL((ag_matmul_kernel<128, 128, true>), dim3(s.grid), dim3(kGemmThreads), 0, st, a0, a1, b,
-                       c, progress_dev, s, lim, status, tb, pf);
+    hipLaunchKernelGGL((ag_matmul_kernel<128, 128, true>), dim3(grid), dim3(kGemmThreads), 0, st, a0, a1, b,
+                       c, progress_dev, s, lim, status, tb, job);
   else if (s.BM == 256 && s.BN == 256)
-    hipLaunchKernelGGL((ag_matmul_kernel<256, 256>), dim3(s.grid), dim3(kGemmThreads), 0, st, a0, a1, b,
-                       c, progress_dev, s, lim, status, tb, pf);
+    hipLaunchKernelGGL((ag_matmul_kernel<256, 256>), dim3(grid), dim3(kGemmThreads), 0, st, a0, a1, b,
+                       c, progress_dev, s, lim, status, tb, job);
   else if (s.BM == 256)
-    hipLaunchKernelGGL((ag_matmul_kernel<256, 128>), dim3(s.grid), dim3(kGemmThreads), 0, st, a0, a1, b,
-                       c, progress_dev, s, lim, status, tb, pf);
+    hipLaunchKernelGGL((ag_matmul_kernel<256, 128>), dim3(grid), dim3(kGemmThreads), 0, st, a0, a1, b,
+                       c, progress_dev, s, lim, status, tb, job);
   else
-    hipLaunchKernelGGL((ag_matmul_kernel<128, 128>), dim3(s.grid), dim3(kGemmThreads), 0, st, a0, a1, b,
-                       c, progress_dev, s, lim, status, tb, pf);
+    hipLaunchKernelGGL((ag_matmul_kernel<128, 128>), dim3(grid), dim3(kGemmThreads), 0, st, a0, a1, b,
+                       c, progress_dev, s, lim, status, tb, job);
   return check_hip(hipGetLastError(), "smr_ag_matmul launch");
 }
 
@@ -1124,27 +1240,34 @@ int smr_ag_matmul(const void* a_shard_dev, const void* a_out_dev, const void* b_
   const char* why;
   if (int rc = validate(M, N, K, rank, world_size, comm_block_m, &why)) return fail(rc, why);
   return launch_gemm(2, a_shard_dev, a_out_dev, b_nk_dev, c_dev, progress_dev, M, N, K, rank, world_size,
-                     comm_block_m, status, stream, nullptr, nullptr, nullptr);
+                     comm_block_m, status, stream, nullptr);
 }
 
-int smr_ag_matmul_pull_first(const void* a_shard_dev, void* a_out_dev, const void* b_nk_dev, void* c_dev,
-                             uint32_t* progress_dev, uint32_t* pull_counters_dev,
-                             const uint64_t* buffer_ptrs_dev, int elem_bytes, int M, int N, int K, int rank,
-                             int world_size, int comm_block_m, uint32_t* status, void* stream) {
+int smr_ag_matmul_fused_state_words(int world_size, int splits_per_rank) {
+  if (world_size < 1 || world_size > SMR_MAX_WORLD_SIZE || splits_per_rank < 1) return 0;
+  return 3 * world_size * splits_per_rank + 1;
+}
+
+int smr_ag_matmul_fused(const void* a_shard_dev, void* a_out_dev, const void* b_nk_dev, void* c_dev,
+                        uint32_t* state_dev, const uint64_t* buffer_ptrs_dev, int elem_bytes, int M, int N,
+                        int K, int rank, int world_size, int comm_block_m, int producer_workgroups,
+                        int pull_first, uint32_t* status, void* stream) {
   using namespace smr;
   const char* why;
   if (elem_bytes != 1 && elem_bytes != 2)
-    return fail(SMR_E_INVALID, "smr_ag_matmul_pull_first: elem_bytes must be 2 (bf16) or 1 (e4m3fn)");
+    return fail(SMR_E_INVALID, "smr_ag_matmul_fused: elem_bytes must be 2 (bf16) or 1 (e4m3fn)");
   if (int rc = elem_bytes == 1 ? validate_fp8(M, N, K, rank, world_size, comm_block_m, &why)
                                : validate(M, N, K, rank, world_size, comm_block_m, &why))
     return fail(rc, why);
-  if (progress_dev == nullptr || pull_counters_dev == nullptr || buffer_ptrs_dev == nullptr)
-    return fail(SMR_E_INVALID, "smr_ag_matmul_pull_first: progress, counters and buffer_ptrs are required");
-  int helpers = 0;
-  if (int rc = launch_gemm(elem_bytes, a_shard_dev, a_out_dev, b_nk_dev, c_dev, progress_dev, M, N, K, rank,
-                           world_size, comm_block_m, status, stream, buffer_ptrs_dev, pull_counters_dev, &helpers))
-    return rc;
-  return helpers;
+  if (state_dev == nullptr || buffer_ptrs_dev == nullptr)
+    return fail(SMR_E_INVALID, "smr_ag_matmul_fused: state and buffer_ptrs are required");
+  if (((int64_t)comm_block_m * K * elem_bytes) % 16 != 0)
+    return fail(SMR_E_INVALID, "smr_ag_matmul_fused: chunks must be 16-byte multiples");
+  if (producer_workgroups < 0 || producer_workgroups > 1024)
+    return fail(SMR_E_INVALID, "smr_ag_matmul_fused: producer_workgroups must be 0..1024");
+  const FusedArgs fa = {buffer_ptrs_dev, state_dev, producer_workgroups, pull_first};
+  return launch_gemm(elem_bytes, a_shard_dev, a_out_dev, b_nk_dev, c_dev, nullptr, M, N, K, rank, world_size,
+                     comm_block_m, status, stream, &fa);
 }
 
 static void fill_plan(int M, int N, int K, int world_size, int comm_block_m, int elem_bytes, int32_t* out5);
@@ -1165,7 +1288,7 @@ int smr_ag_matmul_fp8(const void* a_shard_dev, const void* a_out_dev, const void
   const char* why;
   if (int rc = validate_fp8(M, N, K, rank, world_size, comm_block_m, &why)) return fail(rc, why);
   return launch_gemm(1, a_shard_dev, a_out_dev, b_nk_dev, c_dev, progress_dev, M, N, K, rank, world_size,
-                     comm_block_m, status, stream, nullptr, nullptr, nullptr);
+                     comm_block_m, status, stream, nullptr);
 }
 
 int smr_set_ag_matmul_acquire(int on) {

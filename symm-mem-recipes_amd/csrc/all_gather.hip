@@ -42,17 +42,13 @@ __device__ __forceinline__ void store_through(GlobalVec* p, u32x4 v) {
 __global__ __launch_bounds__(kGatherThreads) void all_gather_kernel(
     const uint64_t* __restrict__ buffer_ptrs, uint8_t* __restrict__ a_out,
     uint32_t* __restrict__ progress, uint32_t* __restrict__ counters, int rank, int world_size,
-    int64_t chunk_vecs, int splits_per_rank, uint64_t* trace, int fast_chunks, int slow_wgs,
-    int skip_chunks) {
+    int64_t chunk_vecs, int splits_per_rank, uint64_t* trace, int fast_chunks, int slow_wgs) {
   int done_chunks = 0;
   if (trace != nullptr && blockIdx.x == 0 && threadIdx.x == 0) trace[kTraceProducerWords - 1] = wall_clock64();
   for (int step = 0; step < world_size; ++step) {
     const int src_rank = (rank + step + 1) % world_size;
     for (int split = 0; split < splits_per_rank; ++split) {
       const int idx = src_rank * splits_per_rank + split;
-      // (the first chunks of the walk may be somebody else's job: the GEMM's own
-      // workgroups pull the first one, smr_ag_matmul_pull_first)
-      if (step * splits_per_rank + split < skip_chunks) continue;
       // workgroups taking part in this chunk
       const int nwg = done_chunks++ < fast_chunks ? (int)gridDim.x : slow_wgs;
       if ((int)blockIdx.x >= nwg) continue;
@@ -145,8 +141,7 @@ extern "C" int smr_set_gather_pacing(int fast_chunks, int slow_workgroups) {
 
 static int launch_gather(const uint64_t* buffer_ptrs_dev, void* a_out_dev, uint32_t* progress_dev,
                          uint32_t* counters_dev, int rank, int world_size, int64_t shard_bytes,
-                         int splits_per_rank, int num_workgroups, void* stream, bool at_once,
-                         int skip_chunks = 0) {
+                         int splits_per_rank, int num_workgroups, void* stream, bool at_once) {
   using namespace smr;
   if (buffer_ptrs_dev == nullptr || a_out_dev == nullptr || progress_dev == nullptr ||
       counters_dev == nullptr)
@@ -158,8 +153,6 @@ static int launch_gather(const uint64_t* buffer_ptrs_dev, void* a_out_dev, uint3
   const int64_t chunk_bytes = shard_bytes / splits_per_rank;
   if (chunk_bytes % 16 != 0 || (reinterpret_cast<uintptr_t>(a_out_dev) & 15u))
     return fail(SMR_E_INVALID, "smr_all_gather_with_progress: chunks must be 16-byte multiples");
-  if (skip_chunks < 0 || skip_chunks > world_size * splits_per_rank)
-    return fail(SMR_E_INVALID, "smr_all_gather_with_progress_from: first_chunk out of range");
   if (num_workgroups < 0 || num_workgroups > 1024)
     return fail(SMR_E_INVALID, "smr_all_gather_with_progress: num_workgroups must be 0..1024");
   const int nwg = num_workgroups == 0 ? kGatherDefaultWorkgroups : num_workgroups;
@@ -174,8 +167,7 @@ static int launch_gather(const uint64_t* buffer_ptrs_dev, void* a_out_dev, uint3
                      reinterpret_cast<hipStream_t>(stream), buffer_ptrs_dev,
                      reinterpret_cast<uint8_t*>(a_out_dev), progress_dev, counters_dev, rank,
                      world_size, chunk_bytes / 16, splits_per_rank, trace_buffer(kTraceProducerWords),
-                     g_gather_fast_chunks, g_gather_slow_workgroups < nwg ? g_gather_slow_workgroups : nwg,
-                     skip_chunks);
+                     g_gather_fast_chunks, g_gather_slow_workgroups < nwg ? g_gather_slow_workgroups : nwg);
   return check_hip(hipGetLastError(), "smr_all_gather_with_progress launch");
 }
 
@@ -193,12 +185,4 @@ extern "C" int smr_all_gather_at_once(const uint64_t* buffer_ptrs_dev, void* a_o
                                       int num_workgroups, void* stream) {
   return launch_gather(buffer_ptrs_dev, a_out_dev, progress_dev, counters_dev, rank, world_size,
                        shard_bytes, splits_per_rank, num_workgroups, stream, true);
-}
-
-extern "C" int smr_all_gather_with_progress_from(const uint64_t* buffer_ptrs_dev, void* a_out_dev,
-                                                 uint32_t* progress_dev, uint32_t* counters_dev, int rank,
-                                                 int world_size, int64_t shard_bytes, int splits_per_rank,
-                                                 int first_chunk, int num_workgroups, void* stream) {
-  return launch_gather(buffer_ptrs_dev, a_out_dev, progress_dev, counters_dev, rank, world_size,
-                       shard_bytes, splits_per_rank, num_workgroups, stream, false, first_chunk);
 }

@@ -50,8 +50,8 @@ SIGNATURES = {
     "smr_all_gather_with_progress": (_i, [_p, _p, _p, _p, _i, _i, _i64, _i, _i, _p]),
     "smr_all_gather_at_once": (_i, [_p, _p, _p, _p, _i, _i, _i64, _i, _i, _p]),
     "smr_set_ag_matmul_acquire": (_i, [_i]),
-    "smr_all_gather_with_progress_from": (_i, [_p, _p, _p, _p, _i, _i, _i64, _i, _i, _i, _p]),
-    "smr_ag_matmul_pull_first": (_i, [_p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _p, _p]),
+    "smr_ag_matmul_fused": (_i, [_p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _i, _p, _p]),
+    "smr_ag_matmul_fused_state_words": (_i, [_i, _i]),
     "smr_set_gather_pacing": (_i, [_i, _i]),
     "smr_ag_matmul": (_i, [_p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _p, _p]),
     "smr_ag_matmul_schedule": (_i, [_i, _i, _i, _i, _i, _i, _i, _p, _i]),

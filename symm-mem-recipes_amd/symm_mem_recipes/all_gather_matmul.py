@@ -17,18 +17,24 @@ from typing import Optional
 import torch
 
 from . import _lib
-from .symm_mem import EmulatedSymmetricMemory, _get_backend_stream
+from .symm_mem import EmulatedSymmetricMemory
 
-#: Producer width and pacing of a fused launch.  None = the library's plan for the
-#: shape (smr_ag_matmul_plan) and no pacing; a number / a (fast_chunks, slow_workgroups)
-#: pair overrides.
-MAX_PRODUCER_WORKGROUPS = None
-PRODUCER_PACING = None
-#: None = the plan decides between the fused launch and copy-then-multiply; True / False force one.
-FUSED = None
-#: A fused launch lets the GEMM's waiting workgroups copy the first remote chunk themselves
-#: (smr_ag_matmul_pull_first); False leaves every chunk to the producer.
-PULL_FIRST = True
+#: Flags, tickets and counters of the fused launch, one array per (device, stream, size): the
+#: kernel leaves it zeroed, so it is filled once when it is made and never again.
+_fused_state = {}
+
+
+def _state_for(device: torch.device, stream: int, words: int) -> torch.Tensor:
+    if torch.cuda.is_current_stream_capturing():
+        # memory allocated under capture belongs to the graph: a fresh array, whose fill is
+        # recorded with the launch (a fill kernel, replayed with it), and nothing cached
+        return torch.zeros(words, dtype=torch.int32, device=device)
+    key = (device.index, int(stream), int(words))
+    st = _fused_state.get(key)
+    if st is None:
+        st = torch.zeros(words, dtype=torch.int32, device=device)
+        _fused_state[key] = st
+    return st
 
 
 def all_gather_with_progress(output: torch.Tensor, inp: torch.Tensor, progress: torch.Tensor,
@@ -60,19 +66,11 @@ def all_gather_with_progress(output: torch.Tensor, inp: torch.Tensor, progress: 
 
 
 def _launch_producer(symm_mem, output, inp, progress, counters, splits_per_rank, num_workgroups,
-                     stream_handle, at_once: bool = False, first_chunk: int = 0) -> None:
+                     stream_handle, at_once: bool = False) -> None:
     """The producer kernel on the given stream; ``counters`` (one zeroed int32 per
     chunk) are its arrival counters.  ``at_once`` copies all chunks together and raises
-    the flags at the end, for a consumer that is queued behind the copy; ``first_chunk``
-    starts the walk at a later chunk (the ones before are delivered by the consumer)."""
+    the flags at the end, for a consumer that is queued behind the copy."""
     lib = _lib.load()
-    if first_chunk:
-        rc = lib.smr_all_gather_with_progress_from(
-            symm_mem.buffer_ptrs_dev, output.data_ptr(), progress.data_ptr(), counters.data_ptr(),
-            symm_mem.rank, symm_mem.world_size, inp.numel() * inp.element_size(), int(splits_per_rank),
-            int(first_chunk), int(num_workgroups), stream_handle)
-        _lib.check(rc, "all_gather_with_progress")
-        return
     rc = (lib.smr_all_gather_at_once if at_once else lib.smr_all_gather_with_progress)(
         symm_mem.buffer_ptrs_dev, output.data_ptr(), progress.data_ptr(), counters.data_ptr(),
         symm_mem.rank, symm_mem.world_size, inp.numel() * inp.element_size(), int(splits_per_rank),
@@ -82,12 +80,25 @@ def _launch_producer(symm_mem, output, inp, progress, counters, splits_per_rank,
 
 def all_gather_matmul_tma_persistent(a_shard: torch.Tensor, b: torch.Tensor, a_out: torch.Tensor,
                                      c_out: torch.Tensor, configs: Optional[dict] = None,
-                                     mm_only: bool = False, *, splits_per_rank: int = 1) -> torch.Tensor:
+                                     mm_only: bool = False, *, splits_per_rank: int = 1,
+                                     fused: Optional[bool] = None, pull_first: Optional[bool] = None,
+                                     producer_workgroups: Optional[int] = None,
+                                     check: bool = False) -> torch.Tensor:
     """``c_out = cat(all ranks' a_shard) @ b.T`` with ``b`` of shape [N, K]
     (K-contiguous), bf16 or - all four tensors - float8_e4m3fn.  ``mm_only`` skips the gather and the flags and multiplies
     what ``a_shard`` (rank 0's rows) and ``a_out`` already hold: the ungated
     comparator.  ``configs`` is accepted for compatibility; the tile shape is the
-    library's choice."""
+    library's choice.
+
+    Keyword arguments beyond the reference's signature (triton_all_gather_matmul.py:219-221):
+    ``fused``      None: the library's plan decides between the fused launch and, for a GEMM too
+                   short to hide the copy behind, copy-then-multiply; True / False force one.
+    ``pull_first`` None: the GEMM's workgroups copy the first remote chunk themselves when enough
+                   of them would otherwise start with a wait; True / False force it.
+    ``producer_workgroups`` copy-only workgroups of the fused launch; None = the plan's.
+    ``check``      synchronise and raise if a bounded wait inside the kernel expired (the result
+                   is then not valid); without it the caller looks at ``check_status()`` later.
+    """
     if mm_only:
         symm_mem = None
         rank = 0
@@ -122,57 +133,48 @@ def all_gather_matmul_tma_persistent(a_shard: torch.Tensor, b: torch.Tensor, a_o
     device = a_shard.device
     current = torch.cuda.current_stream(device)
     status_ptr = symm_mem.status.data_ptr() if symm_mem is not None else 0
-    if mm_only:
-        progress_ptr = 0
-    else:
-        # flags and the producer's arrival counters, zeroed by one fill ahead of both kernels
-        chunks = world_size * splits_per_rank
-        flags = torch.zeros(2 * chunks + 2, dtype=torch.int32, device=device)
-        progress, counters, pull_counters = flags[:chunks], flags[chunks:2 * chunks], flags[2 * chunks:]
-        progress_ptr = progress.data_ptr()
-        symm_mem.barrier(0)
-        backend = _get_backend_stream()
-        backend.wait_stream(current)
-        flags.record_stream(backend)
-        assert a_out.dtype == a_shard.dtype and a_out.is_contiguous()
-        # the producer takes (some of) the compute units the GEMM's grid leaves free
-        plan = (ctypes.c_int32 * 5)()
-        planner = lib.smr_ag_matmul_plan_fp8 if fp8 else lib.smr_ag_matmul_plan
-        _lib.check(planner(M, N, K, world_size, COMM_BLOCK_SIZE_M, plan), "all_gather_matmul")
-        producer_wgs = plan[1] if MAX_PRODUCER_WORKGROUPS is None else min(MAX_PRODUCER_WORKGROUPS, plan[1])
-        pacing = (0, 0) if PRODUCER_PACING is None else PRODUCER_PACING
-        sequential = bool(plan[4]) and FUSED is None or FUSED is False
-        if sequential:
-            # Too small to hide the copy behind the GEMM: the whole GPU copies, then the whole
-            # GPU multiplies, in stream order (the GEMM then needs no flags).
-            wide = torch.cuda.get_device_properties(device).multi_processor_count
-            _launch_producer(symm_mem, a_out, a_shard, progress, counters, splits_per_rank, wide,
-                             current.cuda_stream, at_once=True)
-            progress_ptr = 0
+    gemm = lib.smr_ag_matmul_fp8 if fp8 else lib.smr_ag_matmul
 
-    # The GEMM goes first: its first tiles are local rows and need no flag, so the
-    # producer's launch latency is hidden behind them instead of delaying the GEMM.
-    # (The backend stream waits for what preceded the GEMM, not for the GEMM.)
-    pulled = 0
-    if not mm_only and not sequential and PULL_FIRST:
-        # the workgroups that would wait for the first remote chunk copy it themselves
-        pulled = lib.smr_ag_matmul_pull_first(
-            a_shard.data_ptr(), a_out.data_ptr(), b.data_ptr(), c_out.data_ptr(), progress_ptr,
-            pull_counters.data_ptr(), symm_mem.buffer_ptrs_dev, 1 if fp8 else 2, M, N, K, rank, world_size,
-            COMM_BLOCK_SIZE_M, status_ptr, current.cuda_stream)
-        if pulled < 0:
-            _lib.check(pulled, "all_gather_matmul")
-    else:
-        gemm = lib.smr_ag_matmul_fp8 if fp8 else lib.smr_ag_matmul
-        rc = gemm(a_shard.data_ptr(), a_out.data_ptr(), b.data_ptr(), c_out.data_ptr(),
-                  progress_ptr, M, N, K, rank, world_size, COMM_BLOCK_SIZE_M, status_ptr,
-                  current.cuda_stream)
+    if mm_only:
+        rc = gemm(a_shard.data_ptr(), a_out.data_ptr(), b.data_ptr(), c_out.data_ptr(), 0, M, N, K, rank,
+                  world_size, COMM_BLOCK_SIZE_M, status_ptr, current.cuda_stream)
         _lib.check(rc, "all_gather_matmul")
-    if not mm_only and not sequential:
-        _lib.check(lib.smr_set_gather_pacing(int(pacing[0]), int(pacing[1])), "all_gather_matmul")
-        _launch_producer(symm_mem, a_out, a_shard, progress, counters, splits_per_rank, producer_wgs,
-                         backend.cuda_stream, first_chunk=1 if pulled > 0 else 0)
-        current.wait_stream(backend)
+        return c_out
+
+    symm_mem.barrier(0)
+    plan = (ctypes.c_int32 * 5)()
+    planner = lib.smr_ag_matmul_plan_fp8 if fp8 else lib.smr_ag_matmul_plan
+    _lib.check(planner(M, N, K, world_size, COMM_BLOCK_SIZE_M, plan), "all_gather_matmul")
+    sequential = bool(plan[4]) if fused is None else not fused
+    chunks = world_size * splits_per_rank
+    state = None
+    if sequential:
+        # Too small to hide the copy behind the GEMM: the whole GPU copies, then the whole
+        # GPU multiplies, in stream order (the GEMM then needs no flags).
+        scratch = torch.zeros(2 * chunks, dtype=torch.int32, device=device)
+        wide = torch.cuda.get_device_properties(device).multi_processor_count
+        _launch_producer(symm_mem, a_out, a_shard, scratch[:chunks], scratch[chunks:], splits_per_rank, wide,
+                         current.cuda_stream, at_once=True)
+        rc = gemm(a_shard.data_ptr(), a_out.data_ptr(), b.data_ptr(), c_out.data_ptr(), 0, M, N, K, rank,
+                  world_size, COMM_BLOCK_SIZE_M, status_ptr, current.cuda_stream)
+    else:
+        # One launch on the current stream: GEMM workgroups and copy-only workgroups in one
+        # grid, flags in an array the kernel itself leaves zeroed (no fill, no second stream;
+        # the reference needs both, :249-253,318, because its producer is a copy engine).
+        state = _state_for(device, current.cuda_stream, lib.smr_ag_matmul_fused_state_words(world_size, splits_per_rank))
+        rc = lib.smr_ag_matmul_fused(
+            a_shard.data_ptr(), a_out.data_ptr(), b.data_ptr(), c_out.data_ptr(), state.data_ptr(),
+            symm_mem.buffer_ptrs_dev, 1 if fp8 else 2, M, N, K, rank, world_size, COMM_BLOCK_SIZE_M,
+            0 if producer_workgroups is None else int(producer_workgroups),
+            -1 if pull_first is None else int(bool(pull_first)), status_ptr, current.cuda_stream)
+    _lib.check(rc, "all_gather_matmul")
+    if check:
+        try:
+            symm_mem.check_status()
+        except _lib.SmrError:
+            if state is not None:
+                state.zero_()          # a launch that gave up leaves flags and tickets behind
+            raise
     return c_out
 
 

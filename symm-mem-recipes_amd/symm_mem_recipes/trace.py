@@ -54,19 +54,17 @@ def trace_launch(M: int, N: int, K: int, mode: str = "fused", world_size: int = 
     words = PRODUCER_WORDS + GEMM_WORDS
     trace = torch.zeros(words, dtype=torch.int64, device=device)
 
-    saved = (agm.FUSED, agm.PULL_FIRST)
-    agm.FUSED = {"sequential": False, "ungated": None}.get(mode, True)
-    agm.PULL_FIRST = mode != "fused-no-pull"
+    kwargs = {"fused": {"sequential": False, "ungated": None}.get(mode, True),
+              "pull_first": mode != "fused-no-pull"}
     try:
         _lib.check(lib.smr_set_trace_buffer(trace.data_ptr(), words), "trace")
         for _ in range(warm):
             flush.zero_()
-            agm.all_gather_matmul_tma_persistent(a_shard, b, a_out, c, None, mm_only=(mode == "ungated"))
+            agm.all_gather_matmul_tma_persistent(a_shard, b, a_out, c, None, mm_only=(mode == "ungated"), **kwargs)
         torch.cuda.synchronize(device)
         h.check_status()
     finally:
         lib.smr_set_trace_buffer(None, 0)
-        agm.FUSED, agm.PULL_FIRST = saved
         EmulatedSymmetricMemory.release(a_shard)
 
     t = trace.cpu().tolist()

@@ -48,18 +48,15 @@ def _check(got_bits, want_bits):
 
 
 @pytest.fixture
-def force_fused(monkeypatch):
+def force_fused():
     """Small problems are planned as copy-then-multiply; the tests of the flag-gated
-    launch force it."""
-    import importlib
-    monkeypatch.setattr(importlib.import_module("symm_mem_recipes.all_gather_matmul"), "FUSED", True)
+    launch force it (keyword arguments for all_gather_matmul_tma_persistent)."""
+    return {"fused": True}
 
 
 @pytest.fixture(params=[True, False], ids=["fused", "copy-then-multiply"])
-def either_form(request, monkeypatch):
-    import importlib
-    monkeypatch.setattr(importlib.import_module("symm_mem_recipes.all_gather_matmul"), "FUSED", request.param)
-    return request.param
+def either_form(request):
+    return {"fused": request.param}
 
 
 @pytest.fixture(autouse=True)
@@ -119,7 +116,7 @@ def test_fused_parity_small(cuda, either_form, M, N, K, ws, rank):
     a_shard, h, shards, b, b_bits, a_out, c_out = _setup(M, N, K, ws, rank, cuda)
     configs = {"BLOCK_SIZE_M": 128, "BLOCK_SIZE_N": 128, "BLOCK_SIZE_K": 64, "GROUP_SIZE_M": 1,
                "num_stages": 3, "num_warps": 8}
-    ret = all_gather_matmul_tma_persistent(a_shard, b, a_out, c_out, configs)
+    ret = all_gather_matmul_tma_persistent(a_shard, b, a_out, c_out, configs, **either_form)
     h.check_status()
     assert ret.data_ptr() == c_out.data_ptr()
     want = O.ag_matmul_ref(shards, b_bits)
@@ -142,7 +139,7 @@ def test_fused_parity_splits_per_rank(cuda, either_form, M, N, K, ws, rank, spli
     from symm_mem_recipes import all_gather_matmul_tma_persistent
     a_shard, h, shards, b, b_bits, a_out, c_out = _setup(M, N, K, ws, rank, cuda)
     a_out.zero_()
-    all_gather_matmul_tma_persistent(a_shard, b, a_out, c_out, None, splits_per_rank=splits)
+    all_gather_matmul_tma_persistent(a_shard, b, a_out, c_out, None, splits_per_rank=splits, **either_form)
     h.check_status()
     _check(_t_bits(c_out), O.ag_matmul_ref(shards, b_bits))
     assert np.array_equal(_t_bits(a_out), np.concatenate(shards))
@@ -158,7 +155,7 @@ def test_fused_parity_half_tile_phases(cuda, lib, force_fused, head, tail):
     try:
         assert lib.smr_set_ag_matmul_halves(head, tail) == 0
         c_out.zero_()
-        all_gather_matmul_tma_persistent(a_shard, b, a_out, c_out, None)
+        all_gather_matmul_tma_persistent(a_shard, b, a_out, c_out, None, **force_fused)
         h.check_status()
     finally:
         lib.smr_set_ag_matmul_halves(-1, -1)
@@ -176,7 +173,7 @@ def test_fused_back_to_back_calls_are_identical(cuda, either_form):
     for i in range(20):
         a_out.zero_()
         c = torch.empty_like(c_out)
-        all_gather_matmul_tma_persistent(a_shard, b, a_out, c, None)
+        all_gather_matmul_tma_persistent(a_shard, b, a_out, c, None, **either_form)
         outs.append(c)
     torch.cuda.synchronize()
     h.check_status()
@@ -186,7 +183,7 @@ def test_fused_back_to_back_calls_are_identical(cuda, either_form):
         assert torch.equal(c.view(torch.int16), outs[0].view(torch.int16))
 
 
-def test_copy_then_multiply_matches_fused(cuda, lib, monkeypatch):
+def test_copy_then_multiply_matches_fused(cuda, lib):
     """A GEMM too short to hide the copy behind is planned as copy-then-multiply
     (M=4096 N=1792 K=4096 is); the planned form and both forced forms give the oracle's
     product and one another's bits, with the gathered operand complete in each."""
@@ -200,10 +197,9 @@ def test_copy_then_multiply_matches_fused(cuda, lib, monkeypatch):
     want = O.ag_matmul_ref(shards, b_bits)
     outs = []
     for fused in (None, True, False):
-        monkeypatch.setattr(agm, "FUSED", fused)
         a_out.zero_()
         c = torch.full_like(c_out, float("nan"))
-        agm.all_gather_matmul_tma_persistent(a_shard, b, a_out, c, None)
+        agm.all_gather_matmul_tma_persistent(a_shard, b, a_out, c, None, fused=fused)
         h.check_status()
         assert np.array_equal(_t_bits(a_out), np.concatenate(shards))
         _check(_t_bits(c), want)
@@ -214,13 +210,14 @@ def test_copy_then_multiply_matches_fused(cuda, lib, monkeypatch):
 
 @pytest.mark.parametrize("M,N,K", [(8192, 1024, 1024), (4096, 1792, 4096)])
 def test_fused_launch_replays_from_a_graph(cuda, either_form, M, N, K):
-    """The whole call - flag fill, handshake, GEMM, producer on the second stream and the
-    join - captured into a HIP graph (kernel nodes only) and replayed: every replay, with
-    eager work and synchronisations in between, gives the eager result, for the fused form (two concurrent branches) and for copy-then-multiply."""
+    """The whole call captured into a HIP graph (kernel nodes only) and replayed: every
+    replay, with eager work and synchronisations in between, gives the eager result, for the
+    fused form (one launch whose flags the kernel itself leaves zeroed) and for
+    copy-then-multiply."""
     from symm_mem_recipes import all_gather_matmul_tma_persistent
     ws, rank = 8, 2
     a_shard, h, shards, b, b_bits, a_out, c_out = _setup(M, N, K, ws, rank, cuda)
-    all_gather_matmul_tma_persistent(a_shard, b, a_out, c_out, None)          # eager: the expected bits
+    all_gather_matmul_tma_persistent(a_shard, b, a_out, c_out, None, **either_form)          # eager: the expected bits
     torch.cuda.synchronize()
     h.check_status()
     want_c, want_a = c_out.clone(), a_out.clone()
@@ -230,7 +227,7 @@ def test_fused_launch_replays_from_a_graph(cuda, either_form, M, N, K):
     graph = torch.cuda.CUDAGraph()
     with torch.cuda.stream(side):
         with torch.cuda.graph(graph, stream=side):
-            all_gather_matmul_tma_persistent(a_shard, b, a_out, c_out, None)
+            all_gather_matmul_tma_persistent(a_shard, b, a_out, c_out, None, **either_form)
     torch.cuda.current_stream(cuda).wait_stream(side)
     for replay in range(4):
         a_out.zero_()
@@ -247,71 +244,91 @@ def test_fused_launch_replays_from_a_graph(cuda, either_form, M, N, K):
 
 
 @pytest.mark.parametrize("M,N,K,rank,splits", [(16384, 2048, 256, 0, 1), (16384, 2048, 192, 5, 1), (16384, 3072, 128, 7, 2)])
-def test_first_chunk_pulled_by_the_gemm(cuda, lib, force_fused, monkeypatch, M, N, K, rank, splits):
-    """Enough workgroups would wait for the first remote chunk that the GEMM's grid copies
-    it itself and the producer starts at its second chunk: same product, bit for bit, as
-    with every chunk left to the producer; gathered operand complete; all flags raised."""
-    import importlib
-    agm = importlib.import_module("symm_mem_recipes.all_gather_matmul")
+def test_first_chunk_pulled_by_the_gemm(cuda, lib, M, N, K, rank, splits):
+    """Enough workgroups would wait for the first remote chunk that every GEMM workgroup copies
+    at it before its first tile: same product, bit for bit, as with the copying left to the
+    copy-only workgroups and the waiters; gathered operand complete; state zero again."""
+    from symm_mem_recipes import all_gather_matmul_tma_persistent
     ws = 8
     a_shard, h, shards, b, b_bits, a_out, c_out = _setup(M, N, K, ws, rank, cuda)
     outs = []
-    for pull in (False, True, True):
-        monkeypatch.setattr(agm, "PULL_FIRST", pull)
+    for pull in (False, True, None):
         a_out.zero_()
         c = torch.full_like(c_out, float("nan"))
-        agm.all_gather_matmul_tma_persistent(a_shard, b, a_out, c, None, splits_per_rank=splits)
+        all_gather_matmul_tma_persistent(a_shard, b, a_out, c, None, splits_per_rank=splits, fused=True,
+                                         pull_first=pull)
         h.check_status()
         assert np.array_equal(_t_bits(a_out), np.concatenate(shards))
         outs.append(c)
     _check(_t_bits(outs[0]), O.ag_matmul_ref(shards, b_bits))
     assert torch.equal(outs[0].view(torch.int16), outs[1].view(torch.int16))
     assert torch.equal(outs[0].view(torch.int16), outs[2].view(torch.int16))
-    # through the C ABI: it reports the pulling workgroups, counts every piece of the chunk once and
-    # raises the first remote chunk's flag itself (no producer is started here, so only that one)
-    chunks = ws * splits
-    state = torch.zeros(chunks + 2, dtype=torch.int32, device=cuda)
-    state[:chunks] = 1                                    # the other chunks are in place already
-    first = ((rank + 1) % ws) * splits
-    state[first] = 0
-    rows = M // ws // splits
-    a_out[first * rows:(first + 1) * rows].zero_()
-    pulled = lib.smr_ag_matmul_pull_first(a_shard.data_ptr(), a_out.data_ptr(), b.data_ptr(), c_out.data_ptr(),
-                                          state.data_ptr(), state[chunks:].data_ptr(), h.buffer_ptrs_dev, 2,
-                                          M, N, K, rank, ws, rows, h.status.data_ptr(),
-                                          torch.cuda.current_stream(cuda).cuda_stream)
-    torch.cuda.synchronize()
-    h.check_status()
-    assert pulled == lib.smr_ag_matmul_grid(M, N, K, ws, rows, 1) > 0
-    pieces = -(-rows * K * 2 // 65536)                      # 64 KiB pieces, each taken once and finished once
-    final = state.cpu().tolist()
-    assert final[:chunks] == [1] * chunks and final[chunks] >= pieces and final[chunks + 1] == pieces
-    assert np.array_equal(_t_bits(a_out), np.concatenate(shards))
-    assert torch.equal(c_out.view(torch.int16), outs[0].view(torch.int16))
 
 
-def test_small_launch_leaves_the_first_chunk_to_the_producer(cuda, lib):
-    """Few waiting workgroups: smr_ag_matmul_pull_first runs as the plain gated GEMM and says so."""
-    M, N, K, ws, rank = 2048, 256, 256, 8, 1
+@pytest.mark.parametrize("producers", [1, 8, 64])
+def test_fused_entry_through_the_abi(cuda, lib, producers):
+    """smr_ag_matmul_fused called directly, twice on one state array that is zeroed once:
+    product as the oracle's, gathered operand complete, and every word of the state (flags,
+    tickets, counters) zero again after each launch."""
+    M, N, K, ws, rank, splits = 4096, 512, 256, 8, 3, 2
     a_shard, h, shards, b, b_bits, a_out, c_out = _setup(M, N, K, ws, rank, cuda)
-    a_out.copy_(_bits_t(np.concatenate(shards)))
-    state = torch.ones(ws + 2, dtype=torch.int32, device=cuda)
-    state[ws:] = 0
-    pulled = lib.smr_ag_matmul_pull_first(a_shard.data_ptr(), a_out.data_ptr(), b.data_ptr(), c_out.data_ptr(),
-                                          state.data_ptr(), state[ws:].data_ptr(), h.buffer_ptrs_dev, 2,
-                                          M, N, K, rank, ws, M // ws, h.status.data_ptr(),
-                                          torch.cuda.current_stream(cuda).cuda_stream)
-    torch.cuda.synchronize()
-    h.check_status()
-    assert pulled == 0
-    _check(_t_bits(c_out), O.ag_matmul_ref(shards, b_bits))
-    null = lib.smr_ag_matmul_pull_first(a_shard.data_ptr(), a_out.data_ptr(), b.data_ptr(), c_out.data_ptr(),
-                                        None, state[ws:].data_ptr(), h.buffer_ptrs_dev, 2, M, N, K, rank, ws,
-                                        M // ws, h.status.data_ptr(), None)
-    assert null == -1
-    assert lib.smr_ag_matmul_pull_first(a_shard.data_ptr(), a_out.data_ptr(), b.data_ptr(), c_out.data_ptr(),
-                                        state.data_ptr(), state[ws:].data_ptr(), h.buffer_ptrs_dev, 4, M, N, K,
-                                        rank, ws, M // ws, h.status.data_ptr(), None) == -1
+    words = lib.smr_ag_matmul_fused_state_words(ws, splits)
+    assert words == 3 * ws * splits + 1
+    state = torch.zeros(words, dtype=torch.int32, device=cuda)
+    want = O.ag_matmul_ref(shards, b_bits)
+    for call in range(2):
+        a_out.zero_()
+        c_out.fill_(float("nan"))
+        rc = lib.smr_ag_matmul_fused(a_shard.data_ptr(), a_out.data_ptr(), b.data_ptr(), c_out.data_ptr(),
+                                     state.data_ptr(), h.buffer_ptrs_dev, 2, M, N, K, rank, ws, M // ws // splits,
+                                     producers, -1, h.status.data_ptr(), torch.cuda.current_stream(cuda).cuda_stream)
+        assert rc == 0, lib.smr_last_error_string()
+        h.check_status()
+        assert state.cpu().tolist() == [0] * words, call
+        assert np.array_equal(_t_bits(a_out), np.concatenate(shards))
+        _check(_t_bits(c_out), want)
+    bad = lib.smr_ag_matmul_fused
+    args = (a_shard.data_ptr(), a_out.data_ptr(), b.data_ptr(), c_out.data_ptr())
+    assert bad(*args, None, h.buffer_ptrs_dev, 2, M, N, K, rank, ws, M // ws, 0, -1, None, None) == -1
+    assert bad(*args, state.data_ptr(), None, 2, M, N, K, rank, ws, M // ws, 0, -1, None, None) == -1
+    assert bad(*args, state.data_ptr(), h.buffer_ptrs_dev, 4, M, N, K, rank, ws, M // ws, 0, -1, None, None) == -1
+    assert bad(*args, state.data_ptr(), h.buffer_ptrs_dev, 2, M, N, K, rank, ws, M // ws, -3, -1, None, None) == -1
+
+
+def test_fused_launch_needs_no_second_stream(cuda, lib):
+    """The fused call issues exactly one kernel on the current stream: run on a side stream
+    with nothing else in flight, with the copy-only workgroups taken away altogether (the
+    GEMM's workgroups then do all the copying themselves), it still completes and is right."""
+    from symm_mem_recipes import all_gather_matmul_tma_persistent
+    M, N, K, ws, rank = 8192, 1024, 512, 8, 2
+    a_shard, h, shards, b, b_bits, a_out, c_out = _setup(M, N, K, ws, rank, cuda)
+    want = O.ag_matmul_ref(shards, b_bits)
+    side = torch.cuda.Stream(cuda)
+    side.wait_stream(torch.cuda.current_stream(cuda))
+    with torch.cuda.stream(side):
+        a_out.zero_()
+        all_gather_matmul_tma_persistent(a_shard, b, a_out, c_out, None, fused=True, check=True)
+    side.synchronize()
+    _check(_t_bits(c_out), want)
+    assert np.array_equal(_t_bits(a_out), np.concatenate(shards))
+    # no copy-only workgroup at all: smr_ag_matmul_fused with a grid that leaves no room for them
+    try:
+        assert lib.smr_set_ag_matmul_grid_limit(0) == 0
+        words = lib.smr_ag_matmul_fused_state_words(ws, 1)
+        state = torch.zeros(words, dtype=torch.int32, device=cuda)
+        a_out.zero_()
+        c_out.fill_(float("nan"))
+        # 1 producer asked for, but pull_first off and one copy-only workgroup: the waiters do most of it
+        rc = lib.smr_ag_matmul_fused(a_shard.data_ptr(), a_out.data_ptr(), b.data_ptr(), c_out.data_ptr(),
+                                     state.data_ptr(), h.buffer_ptrs_dev, 2, M, N, K, rank, ws, M // ws, 1, 0,
+                                     h.status.data_ptr(), torch.cuda.current_stream(cuda).cuda_stream)
+        assert rc == 0
+        h.check_status()
+    finally:
+        lib.smr_set_ag_matmul_grid_limit(0)
+    _check(_t_bits(c_out), want)
+    assert np.array_equal(_t_bits(a_out), np.concatenate(shards))
+    assert state.cpu().tolist() == [0] * words
 
 
 @pytest.fixture(params=[0, 1], ids=["flag-only", "acquire"])
@@ -338,7 +355,7 @@ def test_fused_reads_fresh_rows_when_buffers_are_reused(cuda, either_form, acqui
     for bits, dev_bits in versions:
         for r in range(ws):
             h.get_buffer(r, (rows, K), torch.bfloat16).copy_(dev_bits[r])
-        all_gather_matmul_tma_persistent(a_shard, b, a_out, c_out, None)
+        all_gather_matmul_tma_persistent(a_shard, b, a_out, c_out, None, **either_form)
         outs.append((c_out.clone(), a_out.clone()))
     torch.cuda.synchronize()
     h.check_status()
@@ -371,7 +388,7 @@ def test_fused_parity_random_shapes(cuda, either_form, M, N, K, ws, rank, splits
     from symm_mem_recipes import all_gather_matmul_tma_persistent
     a_shard, h, shards, b, b_bits, a_out, c_out = _setup(M, N, K, ws, rank, cuda)
     a_out.zero_()
-    all_gather_matmul_tma_persistent(a_shard, b, a_out, c_out, None, splits_per_rank=splits)
+    all_gather_matmul_tma_persistent(a_shard, b, a_out, c_out, None, splits_per_rank=splits, **either_form)
     h.check_status()
     assert np.array_equal(_t_bits(a_out), np.concatenate(shards))
     _check(_t_bits(c_out), O.ag_matmul_ref(shards, b_bits))

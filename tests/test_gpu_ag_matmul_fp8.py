@@ -48,11 +48,10 @@ def _check(got, want):
 
 
 @pytest.fixture(params=[True, False], ids=["fused", "copy-then-multiply"])
-def either_form(request, monkeypatch):
-    """Small problems are planned as copy-then-multiply; both forms are tested."""
-    import importlib
-    monkeypatch.setattr(importlib.import_module("symm_mem_recipes.all_gather_matmul"), "FUSED", request.param)
-    return request.param
+def either_form(request):
+    """Small problems are planned as copy-then-multiply; both forms are tested (keyword
+    arguments for all_gather_matmul_tma_persistent)."""
+    return {"fused": request.param}
 
 
 @pytest.fixture(autouse=True)
@@ -76,7 +75,7 @@ def _release():
 def test_fp8_fused_parity(cuda, either_form, M, N, K, ws, rank):
     from symm_mem_recipes import all_gather_matmul_tma_persistent
     a_shard, h, shards, b, b_bits, a_out, c_out = _setup(M, N, K, ws, rank, cuda)
-    ret = all_gather_matmul_tma_persistent(a_shard, b, a_out, c_out, None)
+    ret = all_gather_matmul_tma_persistent(a_shard, b, a_out, c_out, None, **either_form)
     h.check_status()
     assert ret.data_ptr() == c_out.data_ptr()
     _check(_bits(c_out), O.ag_matmul_ref_fp8(shards, b_bits))
@@ -100,42 +99,39 @@ def _random_shapes(n, seed):
 def test_fp8_parity_random_shapes(cuda, either_form, M, N, K, ws, rank):
     from symm_mem_recipes import all_gather_matmul_tma_persistent
     a_shard, h, shards, b, b_bits, a_out, c_out = _setup(M, N, K, ws, rank, cuda)
-    all_gather_matmul_tma_persistent(a_shard, b, a_out, c_out, None)
+    all_gather_matmul_tma_persistent(a_shard, b, a_out, c_out, None, **either_form)
     h.check_status()
     assert np.array_equal(_bits(a_out), np.concatenate(shards))
     _check(_bits(c_out), O.ag_matmul_ref_fp8(shards, b_bits))
 
 
-def test_fp8_first_chunk_pulled_by_the_gemm(cuda, lib, monkeypatch):
-    """A launch wide enough that the grid copies the first remote chunk itself: same codes
-    as with every chunk left to the producer, gathered operand complete."""
-    import importlib
-    agm = importlib.import_module("symm_mem_recipes.all_gather_matmul")
-    monkeypatch.setattr(agm, "FUSED", True)
+def test_fp8_first_chunk_pulled_by_the_gemm(cuda, lib):
+    """A launch wide enough that every GEMM workgroup copies at the first remote chunk before
+    its first tile: same codes as without, gathered operand complete; and the fused entry
+    through the C ABI with e4m3fn operands leaves its state zeroed."""
+    from symm_mem_recipes import all_gather_matmul_tma_persistent
     M, N, K, ws, rank = 16384, 2048, 256, 8, 6
     a_shard, h, shards, b, b_bits, a_out, c_out = _setup(M, N, K, ws, rank, cuda)
     outs = []
     for pull in (False, True):
-        monkeypatch.setattr(agm, "PULL_FIRST", pull)
         a_out.view(torch.uint8).zero_()
         c = torch.full_like(c_out.view(torch.uint8), 0x7F).view(torch.float8_e4m3fn)
-        agm.all_gather_matmul_tma_persistent(a_shard, b, a_out, c, None)
+        all_gather_matmul_tma_persistent(a_shard, b, a_out, c, None, fused=True, pull_first=pull)
         h.check_status()
         assert np.array_equal(_bits(a_out), np.concatenate(shards))
         outs.append(_bits(c))
     _check(outs[0], O.ag_matmul_ref_fp8(shards, b_bits))
     assert np.array_equal(outs[0], outs[1])
-    state = torch.zeros(ws + 2, dtype=torch.int32, device=cuda)
-    state[:ws] = 1
-    state[(rank + 1) % ws] = 0
-    pulled = lib.smr_ag_matmul_pull_first(a_shard.data_ptr(), a_out.data_ptr(), b.data_ptr(), c_out.data_ptr(),
-                                          state.data_ptr(), state[ws:].data_ptr(), h.buffer_ptrs_dev, 1,
-                                          M, N, K, rank, ws, M // ws, h.status.data_ptr(),
-                                          torch.cuda.current_stream(cuda).cuda_stream)
-    torch.cuda.synchronize()
+    words = lib.smr_ag_matmul_fused_state_words(ws, 1)
+    state = torch.zeros(words, dtype=torch.int32, device=cuda)
+    a_out.view(torch.uint8).zero_()
+    rc = lib.smr_ag_matmul_fused(a_shard.data_ptr(), a_out.data_ptr(), b.data_ptr(), c_out.data_ptr(),
+                                 state.data_ptr(), h.buffer_ptrs_dev, 1, M, N, K, rank, ws, M // ws, 0, 1,
+                                 h.status.data_ptr(), torch.cuda.current_stream(cuda).cuda_stream)
+    assert rc == 0
     h.check_status()
-    final = state.cpu().tolist()
-    assert pulled > 0 and final[:ws] == [1] * ws and final[ws + 1] == -(-(M // ws) * K // 65536)
+    assert state.cpu().tolist() == [0] * words
+    assert np.array_equal(_bits(a_out), np.concatenate(shards))
     assert np.array_equal(_bits(c_out), outs[0])
 
 
@@ -156,7 +152,7 @@ def test_fp8_saturation_and_exact_small_integers(cuda, either_form):
     b_bits[0, :] = vals[-1]
     h.get_buffer(0, (M // ws, K), torch.uint8).copy_(torch.from_numpy(shards[0]))
     b = _t(b_bits).to(cuda)
-    all_gather_matmul_tma_persistent(a_shard, b, a_out, c_out, None)
+    all_gather_matmul_tma_persistent(a_shard, b, a_out, c_out, None, **either_form)
     h.check_status()
     want = O.ag_matmul_ref_fp8(shards, b_bits)
     got = _bits(c_out)

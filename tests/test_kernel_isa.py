@@ -28,21 +28,25 @@ def kernels(tmp_path_factory):
     subprocess.run(cmd, check=True, capture_output=True)
     text = out.read_text()
     bodies = {}
-    for m in re.finditer(r"^(_ZN3smr16ag_matmul_kernelILi(\d+)ELi(\d+)ELb([01])E\w*):[^\n]*\n(.*?)s_endpgm", text, re.S | re.M):
+    for m in re.finditer(r"^(_ZN3smr16ag_matmul_kernelILi(\d+)ELi(\d+)ELb([01])E\w*):[^\n]*\n(.*?)^\.Lfunc_end", text, re.S | re.M):
         bodies[(int(m.group(2)), int(m.group(3)), m.group(4) == "1")] = m.group(5).splitlines()
     return bodies
 
 
 def _k_loops(lines):
-    """Loops that contain the explicit wait for the tile loads: from the loop's label to
-    the backward branch."""
+    """Innermost loops with MFMAs in them: from a label to a conditional branch back to it,
+    with no other label in between."""
+    labels = {}
+    for i, ln in enumerate(lines):
+        m = re.match(r"^(\.LBB\d+_\d+):", ln)
+        if m:
+            labels[m.group(1)] = i
     loops = []
     for i, ln in enumerate(lines):
-        if re.search(r"s_waitcnt vmcnt\((8|4)\)", ln):
-            start = max(j for j in range(i) if re.match(r"^\.LBB\d+_\d+:", lines[j]))
-            end = next(j for j in range(i, len(lines)) if "s_cbranch" in lines[j])
-            body = lines[start:end + 1]
-            if any("v_mfma_" in x for x in body):           # (the copy loop of the pulled first chunk waits too)
+        m = re.search(r"s_cbranch_\w+ (\.LBB\d+_\d+)", ln)
+        if m and labels.get(m.group(1), i) < i:
+            body = lines[labels[m.group(1)]:i + 1]
+            if sum(bool(re.match(r"^\.LBB", x)) for x in body) == 1 and any("v_mfma_" in x for x in body):
                 loops.append(body)
     return loops
 
@@ -58,4 +62,6 @@ def test_k_loop_keeps_its_registers(kernels, key):
         assert mfma in (16, 32, 64, 128), mfma                   # one slab pair per trip (full or half-width tile)
         assert "scratch_" not in text, "spill inside the K loop"
         assert "v_accvgpr" not in text, "accumulators moved between register files inside the K loop"
+        assert "lane_b32" not in text, "scalar registers spilled inside the K loop"
+        assert re.search(r"s_waitcnt vmcnt\((8|4)\)", text), "the explicit wait for the tile loads is missing"
         assert len(re.findall(r"s_barrier", text)) == 1
