@@ -111,7 +111,9 @@ def bench_reduce(size_mib, steps, warmup, dev):
     dev_us = e0.elapsed_time(e1) * 1e3 / steps
     alg_bytes = (WS + 1) * nbytes
     # the same call behind the blockwise barrier, and the write-back-to-all variant
-    us_barrier = _time_events(lambda: one_shot_all_reduce(t, barrier=True), 20, 3)
+    # (the reference's call, triton_one_shot_all_reduce.py:70: timed the way the headline is,
+    # back-to-back launches between one event pair)
+    us_barrier = _time_batched(lambda: one_shot_all_reduce(t, barrier=True), max(steps // 2, 10), 3)
     us_write_all = _time_events(lambda: one_shot_all_reduce(t, barrier=False, write_all=True), 20, 3)
     # two-shot: every emulated rank reduces its eighth and writes it to all peers, two handshakes
     for r in range(WS):
@@ -125,7 +127,7 @@ def bench_reduce(size_mib, steps, warmup, dev):
                 us_write_all=us_write_all, write_all_bytes=2 * WS * nbytes, us_two_shot=us_two_shot)
 
 
-def bench_reduce_rotating(size_kib, dev, dtype_name="bf16", write_all=False, accumulate="fp32"):
+def bench_reduce_rotating(size_kib, dev, dtype_name="bf16", write_all=False, accumulate="fp32", barrier=False):
     """Messages below 64 MiB fit the 256 MB last-level cache; rotate over enough buffer
     sets (1 GiB in total, at most 64 sets) that every call reads from HBM."""
     import torch
@@ -144,14 +146,16 @@ def bench_reduce_rotating(size_kib, dev, dtype_name="bf16", write_all=False, acc
     idx = [0]
 
     def call():
-        one_shot_all_reduce(sets[idx[0] % nsets], barrier=False, write_all=write_all, accumulate=accumulate)
+        one_shot_all_reduce(sets[idx[0] % nsets], barrier=barrier, write_all=write_all, accumulate=accumulate)
         idx[0] += 1
     us = _time_batched(call, max(10 * nsets, 200), nsets)
     alg = (2 * WS if write_all else WS + 1) * nbytes
     res = dict(size_kib=size_kib, dtype=dtype_name, mode="write_all" if write_all else "single_output",
                accumulate=accumulate, us=us, gbs=alg / us / 1e3, frac=alg / us / 1e3 / HBM_PEAK_GBS,
                buffer_sets=nsets)
-    if nbytes <= (4 << 20) and not write_all:
+    if barrier:
+        res["mode"] += ", behind the blockwise barrier"
+    if nbytes <= (4 << 20) and not write_all and not barrier:
         # Below a few MiB the eager figure is the host's launch rate, not the kernel:
         # replay one pass over the buffer sets from a HIP graph (kernel nodes only) and
         # check every replay against the eager result.
@@ -326,7 +330,7 @@ def bench_barrier(dev):
     base = (base - (base >= 2 ** 31).to(torch.int64) * 2 ** 32).to(torch.int32)
     sums = torch.zeros(WS, blocks, dtype=torch.int32, device=dev)
     mism = torch.zeros(1, dtype=torch.int32, device=dev)
-    prounds = 1000
+    prounds = 10000                     # the configuration's 10,000 rounds, payload included
     stream = torch.cuda.current_stream().cuda_stream
 
     def payload():
@@ -334,7 +338,7 @@ def bench_barrier(dev):
                                   sums.data_ptr(), mism.data_ptr(), WS, blocks, chunk, prounds,
                                   h.status.data_ptr(), stream)
         assert rc == 0
-    us_payload = _time_events(payload, 3, 1) / prounds
+    us_payload = _time_events(payload, 1, 0) / prounds
     h.check_status()
     assert int(mism.item()) == 0, "signal-round checksum mismatch"
     SM.release()
@@ -344,6 +348,25 @@ def bench_barrier(dev):
                 rounds_payload=prounds, us_per_round_payload=us_payload,
                 payload_written_mib=written / 2 ** 20, payload_read_mib=WS * written / 2 ** 20,
                 payload_gbs=(written + WS * written) / us_payload / 1e3)
+
+
+def bench_reference_point(dev):
+    """The reference's own benchmark point (triton_one_shot_all_reduce.py:145-162): 8192 bf16
+    per rank, filled with ones, the call as the reference makes it (behind the blockwise
+    barrier), median device time of the kernel over 200 calls from the profiler."""
+    import torch
+    from symm_mem_recipes import EmulatedSymmetricMemory as SM, one_shot_all_reduce
+    from symm_mem_recipes.utils import benchmark_with_profiler
+    t = SM.empty_strided_p2p((8192,), (1,), torch.bfloat16, dev, world_size=WS, rank=0)
+    h = SM.rendezvous(t)
+    for r in range(WS):
+        h.get_buffer(r, (8192,), torch.bfloat16).fill_(1)
+    assert one_shot_all_reduce(t).eq(WS).all().item()
+    h.check_status()
+    us = benchmark_with_profiler(lambda: one_shot_all_reduce(t), r".*one_shot_all_reduce_kernel", benchmark_iters=200)
+    SM.release()
+    return {"workload": "8192 bf16 per rank behind the blockwise barrier, kernel time from the profiler, 200 calls",
+            "median_kernel_us": us}
 
 
 def calibration_copy(dev):
@@ -359,24 +382,44 @@ def calibration_copy(dev):
 
 
 def cpu_baseline(budget_s=10.0):
-    """The numpy oracle of the reduce on the reference's CPU-runnable case: 8 buffers
-    of 1,048,576 bf16, N(0,1) seeded per rank, fp32 accumulation in rank order."""
+    """The CPU oracle of the reduce on the reference's CPU-runnable case: 8 buffers of
+    1,048,576 bf16, N(0,1) seeded per rank, fp32 accumulation in rank order.  Three timings
+    of the same arithmetic: the torch restatement (`acc += buf.float()` per rank, cast) on all
+    host threads torch uses and on one, and the numpy oracle on one thread."""
+    import torch
     from oracle import oracle as O
+    from oracle import torch_reduce as T
     n = 1 << 20
-    bufs = [O.seeded_normal_bf16_bits(n, seed=r) for r in range(WS)]
-    O.reduce_ref(bufs, "bf16")
-    reps = 0
-    t0 = time.perf_counter()
-    while True:
-        O.reduce_ref(bufs, "bf16")
-        reps += 1
-        el = time.perf_counter() - t0
-        if el >= budget_s:
-            break
     nbytes = (WS + 1) * n * 2
-    out = {"value": nbytes * reps / el / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
-           "sample": f"{reps} repetitions of the 8 x 1,048,576 bf16 reduce (numpy oracle, one thread) in {el:.1f} s",
+
+    def timed(fn, seconds):
+        fn()
+        reps, t0 = 0, time.perf_counter()
+        while True:
+            fn()
+            reps += 1
+            el = time.perf_counter() - t0
+            if el >= seconds:
+                return reps, el
+
+    tens = [T.seeded_normal(n, r) for r in range(WS)]
+    all_threads = torch.get_num_threads()
+    reps, el = timed(lambda: T.reduce_ref_torch(tens), budget_s * 0.4)
+    out = {"value": nbytes * reps / el / 1e9, "unit": "GB/s", "cores": all_threads, "kind": "port",
+           "sample": f"{reps} repetitions of the 8 x 1,048,576 bf16 reduce (torch CPU restatement of the oracle, "
+                     f"{all_threads} threads) in {el:.1f} s",
            "host_cpus": os.cpu_count()}
+    torch.set_num_threads(1)
+    try:
+        reps, el = timed(lambda: T.reduce_ref_torch(tens), budget_s * 0.3)
+    finally:
+        torch.set_num_threads(all_threads)
+    out["one_thread"] = {"value": nbytes * reps / el / 1e9, "unit": "GB/s", "cores": 1,
+                         "sample": f"{reps} repetitions, torch CPU restatement, 1 thread, {el:.1f} s"}
+    bufs = [O.seeded_normal_bf16_bits(n, seed=r) for r in range(WS)]
+    reps, el = timed(lambda: O.reduce_ref(bufs, "bf16"), budget_s * 0.3)
+    out["numpy_one_thread"] = {"value": nbytes * reps / el / 1e9, "unit": "GB/s", "cores": 1,
+                               "sample": f"{reps} repetitions, numpy oracle, 1 thread, {el:.1f} s"}
     # the other two paths, once each on a bounded slice (numpy's BLAS uses the host's threads)
     M, N, K = 256, 3584, 8192
     shard = O.seeded_normal_bf16_bits(M * K, seed=0, std=0.02).reshape(M, K)
@@ -451,6 +494,7 @@ def main():
     extra = {
         "reduce_kernel_us": r["dev_us"],
         "reduce_behind_barrier_us": r["us_barrier"],
+        "reduce_behind_barrier_frac": r["alg_bytes"] / r["us_barrier"] / 1e3 / HBM_PEAK_GBS,
         "reduce_write_all_us": r["us_write_all"],
         "reduce_write_all_gbs": r["write_all_bytes"] / r["us_write_all"] / 1e3,
         "reduce_two_shot_us": r["us_two_shot"],
@@ -464,11 +508,16 @@ def main():
             [bench_reduce_rotating(k, dev, "bf16") for k in sweep] +
             [bench_reduce_rotating(k, dev, "fp32") for k in (1024, 8192, 16384)] +
             [bench_reduce_rotating(k, dev, "bf16", write_all=True) for k in (1024, 8192, 16384)] +
-            [bench_reduce_rotating(k, dev, "bf16", accumulate="bf16") for k in (8192,)])
+            [bench_reduce_rotating(k, dev, "bf16", accumulate="bf16") for k in (8192,)] +
+            [bench_reduce_rotating(k, dev, "bf16", barrier=True) for k in (8192, 16384)])
         extra["all_gather_matmul"] = bench_ag_matmul(dev)
         extra["all_gather_matmul_fp8"] = bench_ag_matmul_fp8(dev)
         extra["gemv_allreduce"] = bench_gemv(dev)
         extra["barrier"] = bench_barrier(dev)
+        try:
+            extra["reduce_reference_point"] = bench_reference_point(dev)
+        except Exception as exc:                    # the profiler is optional equipment
+            extra["reduce_reference_point"] = {"error": repr(exc)[:200]}
     line["extra"] = extra
     line["cpu_baseline"] = cpu_baseline(args.cpu_seconds) if args.cpu_seconds > 0 else None
     print(json.dumps(line))

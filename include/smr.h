@@ -266,7 +266,13 @@ int smr_ag_matmul_plan(int M, int N, int K, int world_size, int comm_block_m, in
  * literal reading of wait_signal + the loads that follow (triton_all_gather_matmul.py:72-95,
  * 170-174) asks for.  0 (default): flag poll past the caches and a workgroup barrier only;
  * the rows of a comm block cannot be in a cache before its flag is up, because nobody reads
- * them earlier inside the launch and a launch starts from invalidated caches. */
+ * them earlier inside the launch and a launch starts from invalidated caches.
+ * Preconditions of the default, which the caller owns: (1) nothing else on the GPU reads
+ * a_out while the launch runs (a concurrent reader on another stream could leave lines of
+ * a chunk in an L2 before its flag); (2) whoever writes a chunk writes it through to memory
+ * (agent-scope or system-scope stores, DMA) and raises the flag only after the writes are
+ * acknowledged - this library's producers do.  A caller that cannot promise both turns the
+ * fence on.  Process-wide. */
 int smr_set_ag_matmul_acquire(int on);
 
 /* Tuning knob of the gated schedule: the first `head` and the last `tail` comm blocks

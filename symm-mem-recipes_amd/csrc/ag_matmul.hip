@@ -29,6 +29,7 @@
 //     along instead of spinning;
 //   * the same kernel in e4m3fn (run_tile_fp8): the bytes move the same way, the
 //     tile is built from v_mfma_f32_32x32x64_f8f6f4.
+#include <atomic>
 #include <type_traits>
 
 #include "smr_device.hpp"
@@ -1000,16 +1001,17 @@ static int validate(int M, int N, int K, int rank, int world_size, int comm_bloc
 }
 
 static int cu_count() {
-  static int cached = 0;
-  if (cached == 0) {
-    int dev = 0, n = 0;
+  static std::atomic<int> cached{0};
+  int n = cached.load(std::memory_order_relaxed);
+  if (n == 0) {
+    int dev = 0;
     if (hipGetDevice(&dev) == hipSuccess &&
         hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0)
-      cached = n;
+      cached.store(n, std::memory_order_relaxed);
     else
       return 256;
   }
-  return cached;
+  return n;
 }
 
 // Persistent grid: the fewest workgroups (a multiple of 8, one per XCD slot) that
@@ -1058,9 +1060,11 @@ static FusedEstimate estimate_fused(const GemmSchedule& s, int cus, int grid, in
 
 // smr_set_ag_matmul_halves: ring positions cut into half tiles at either end of a
 // gated launch, or -1 to let make_schedule choose.
-static int g_force_head = -1, g_force_tail = -1;
-static int g_acquire_after_flag = 0;
-static int g_grid_limit = 0;            // smr_set_ag_matmul_grid_limit: 0 = none
+// Process-wide tuning knobs.  Each is one atomic word (head and tail share one), read once
+// per call by make_schedule, so a setter on another thread changes a whole launch or none of it.
+static std::atomic<uint32_t> g_force_halves{0xFFFFFFFFu};   // head in the low half, tail in the high half; 0xFFFF = let the library choose
+static std::atomic<int> g_acquire_after_flag{0};
+static std::atomic<int> g_grid_limit{0};                     // smr_set_ag_matmul_grid_limit: 0 = none
 
 static GemmSchedule make_schedule(int M, int N, int K, int rank, int world_size, int comm_block_m,
                                   int cus, bool gated, int elem_bytes = 2) {
@@ -1068,12 +1072,16 @@ static GemmSchedule make_schedule(int M, int N, int K, int rank, int world_size,
   s.M = M; s.N = N; s.K = K;
   s.rank = rank; s.world_size = world_size; s.comm_block_m = comm_block_m;
   s.head = s.tail = 0;
-  s.acquire = g_acquire_after_flag;
+  s.acquire = g_acquire_after_flag.load(std::memory_order_relaxed);
+  const int grid_limit = g_grid_limit.load(std::memory_order_relaxed);
+  const uint32_t halves = g_force_halves.load(std::memory_order_relaxed);
+  const int force_head = (halves & 0xFFFFu) == 0xFFFFu ? -1 : (int)(halves & 0xFFFFu);
+  const int force_tail = (halves >> 16) == 0xFFFFu ? -1 : (int)(halves >> 16);
   pick_tile(M, N, comm_block_m, s.BM, s.BN, cus);
   const int tn = (N + s.BN - 1) / s.BN;
   const int total = (M / s.BM) * tn;
   int max_grid = ((gated ? cus - kReservedCus : cus) / 8) * 8;
-  if (g_grid_limit > 0 && g_grid_limit < max_grid) max_grid = g_grid_limit / 8 * 8;
+  if (grid_limit > 0 && grid_limit < max_grid) max_grid = grid_limit / 8 * 8;
   if (max_grid < 8) max_grid = 8;
   const int passes = (total + max_grid - 1) / max_grid;
   const int need = ((total + passes - 1) / passes + 7) / 8 * 8;
@@ -1099,10 +1107,10 @@ static GemmSchedule make_schedule(int M, int N, int K, int rank, int world_size,
   // by their loads, and with a producer that delivers a chunk in less than a pass it
   // is cheaper to let the workgroups of the first remote comm block wait for it.
   const int n_comm = M / comm_block_m;
-  if (gated && elem_bytes == 2 && s.BN == 256 && g_force_head >= 0 && g_force_tail >= 0 &&
-      g_force_head + g_force_tail <= n_comm) {
-    s.head = g_force_head;
-    s.tail = g_force_tail;
+  if (gated && elem_bytes == 2 && s.BN == 256 && force_head >= 0 && force_tail >= 0 &&
+      force_head + force_tail <= n_comm) {
+    s.head = force_head;
+    s.tail = force_tail;
   }
   // Rows per group: the divisor of the comm block's row tiles for which an XCD's run of
   // a full pass touches the fewest slabs (rows of the patch + columns of the patch).
@@ -1292,7 +1300,7 @@ int smr_ag_matmul_fp8(const void* a_shard_dev, const void* a_out_dev, const void
 }
 
 int smr_set_ag_matmul_acquire(int on) {
-  smr::g_acquire_after_flag = on ? 1 : 0;
+  smr::g_acquire_after_flag.store(on ? 1 : 0, std::memory_order_relaxed);
   return 0;
 }
 
@@ -1307,14 +1315,14 @@ int smr_ag_matmul_plan_fp8(int M, int N, int K, int world_size, int comm_block_m
 
 int smr_set_ag_matmul_grid_limit(int workgroups) {
   if (workgroups < 0) return smr::fail(SMR_E_INVALID, "smr_set_ag_matmul_grid_limit: negative");
-  smr::g_grid_limit = workgroups;
+  smr::g_grid_limit.store(workgroups, std::memory_order_relaxed);
   return 0;
 }
 
 int smr_set_ag_matmul_halves(int head, int tail) {
   if ((head < 0) != (tail < 0)) return smr::fail(SMR_E_INVALID, "smr_set_ag_matmul_halves: both or neither negative");
-  smr::g_force_head = head;
-  smr::g_force_tail = tail;
+  if (head > 0xFFFE || tail > 0xFFFE) return smr::fail(SMR_E_INVALID, "smr_set_ag_matmul_halves: too large");
+  smr::g_force_halves.store(head < 0 ? 0xFFFFFFFFu : ((uint32_t)head | ((uint32_t)tail << 16)), std::memory_order_relaxed);
   return 0;
 }
 

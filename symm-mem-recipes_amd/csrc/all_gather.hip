@@ -17,6 +17,8 @@
 // 860 us with the write-backs, 760 us without).  The producer can be paced
 // (smr_set_gather_pacing: full width for the first chunks, fewer workgroups after);
 // with write-through stores that no longer gains anything and is off by default.
+#include <atomic>
+
 #include "smr_device.hpp"
 
 namespace smr {
@@ -28,8 +30,8 @@ constexpr int kGatherThreads = 1024;
 constexpr int kGatherDefaultWorkgroups = 8;
 // Pacing (smr_set_gather_pacing): chunks copied at full width, workgroups that stay
 // for the rest.
-static int g_gather_fast_chunks = 0;
-static int g_gather_slow_workgroups = 1024;
+// (one atomic word, fast chunks in the low half: a launch reads the pair once)
+static std::atomic<uint32_t> g_gather_pacing{1024u << 16};
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef __attribute__((address_space(1))) u32x4 GlobalVec;
@@ -103,18 +105,21 @@ __global__ __launch_bounds__(kGatherThreads) void all_gather_at_once_kernel(
   const int64_t stride = (int64_t)gridDim.x * kGatherThreads;
   for (int64_t i = (int64_t)blockIdx.x * kGatherThreads + threadIdx.x; i < chunk_vecs; i += stride) {
     for (int c0 = 0; c0 < chunks; c0 += 8) {
+      // (a group past the last chunk is skipped: the condition is the same for every lane)
       u32x4 v[8];
 #pragma unroll
       for (int u = 0; u < 8; ++u) {
-        const int idx = c0 + u < chunks ? c0 + u : chunks - 1;
-        const GlobalVec* src = (const GlobalVec*)(uintptr_t)buffer_ptrs[idx / splits_per_rank] +
-                               (int64_t)(idx % splits_per_rank) * chunk_vecs;
-        v[u] = __builtin_nontemporal_load(src + i);
+        const int idx = c0 + u;
+        if (idx < chunks) {
+          const GlobalVec* src = (const GlobalVec*)(uintptr_t)buffer_ptrs[idx / splits_per_rank] +
+                                 (int64_t)(idx % splits_per_rank) * chunk_vecs;
+          v[u] = __builtin_nontemporal_load(src + i);
+        }
       }
 #pragma unroll
       for (int u = 0; u < 8; ++u) {
-        const int idx = c0 + u < chunks ? c0 + u : chunks - 1;     // (the last chunk again: same bytes)
-        store_through((GlobalVec*)(uintptr_t)a_out + (int64_t)idx * chunk_vecs + i, v[u]);
+        const int idx = c0 + u;
+        if (idx < chunks) store_through((GlobalVec*)(uintptr_t)a_out + (int64_t)idx * chunk_vecs + i, v[u]);
       }
     }
   }
@@ -134,8 +139,9 @@ __global__ __launch_bounds__(kGatherThreads) void all_gather_at_once_kernel(
 extern "C" int smr_set_gather_pacing(int fast_chunks, int slow_workgroups) {
   if (fast_chunks < 0 || slow_workgroups < 0 || slow_workgroups > 1024)
     return smr::fail(SMR_E_INVALID, "smr_set_gather_pacing: negative or too large");
-  smr::g_gather_fast_chunks = fast_chunks;
-  smr::g_gather_slow_workgroups = slow_workgroups == 0 ? 1024 : slow_workgroups;
+  if (fast_chunks > 0xFFFF) return smr::fail(SMR_E_INVALID, "smr_set_gather_pacing: negative or too large");
+  smr::g_gather_pacing.store((uint32_t)fast_chunks | ((uint32_t)(slow_workgroups == 0 ? 1024 : slow_workgroups) << 16),
+                             std::memory_order_relaxed);
   return 0;
 }
 
@@ -163,11 +169,13 @@ static int launch_gather(const uint64_t* buffer_ptrs_dev, void* a_out_dev, uint3
                        chunk_bytes / 16, splits_per_rank);
     return check_hip(hipGetLastError(), "smr_all_gather launch");
   }
+  const uint32_t pacing = g_gather_pacing.load(std::memory_order_relaxed);
+  const int fast_chunks = (int)(pacing & 0xFFFFu), slow_wgs = (int)(pacing >> 16);
   hipLaunchKernelGGL(all_gather_kernel, dim3(nwg), dim3(kGatherThreads), 0,
                      reinterpret_cast<hipStream_t>(stream), buffer_ptrs_dev,
                      reinterpret_cast<uint8_t*>(a_out_dev), progress_dev, counters_dev, rank,
                      world_size, chunk_bytes / 16, splits_per_rank, trace_buffer(kTraceProducerWords),
-                     g_gather_fast_chunks, g_gather_slow_workgroups < nwg ? g_gather_slow_workgroups : nwg);
+                     fast_chunks, slow_wgs < nwg ? slow_wgs : nwg);
   return check_hip(hipGetLastError(), "smr_all_gather_with_progress launch");
 }
 

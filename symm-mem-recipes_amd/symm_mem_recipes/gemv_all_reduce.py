@@ -53,7 +53,11 @@ def gemv_all_reduce(x: torch.Tensor, w: torch.Tensor, world_size: int = 8,
     if workspace is None:
         workspace = GemvWorkspace(batch, N, world_size, x.device, K)
     assert (workspace.batch, workspace.N, workspace.world_size) == (batch, N, world_size)
-    assert workspace.senders >= _lib.load().smr_gemv_senders(N, K, world_size)
+    lib = _lib.load()
+    senders = lib.smr_gemv_senders(N, K, world_size)
+    # (the launch shape is a process-wide knob: a workspace made under another setting may be too small)
+    assert workspace.senders >= senders, "workspace was built for fewer partial producers"
+    assert workspace.flags.numel() >= lib.smr_gemv_flag_blocks(N) * senders, "workspace has too few flags"
     if out is None:
         out = torch.empty(batch, N, dtype=torch.bfloat16, device=x.device)
     rc = _lib.load().smr_gemv_allreduce(

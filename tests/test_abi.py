@@ -92,3 +92,53 @@ def test_missing_library_is_loud(monkeypatch, tmp_path):
     monkeypatch.setattr(_lib, "LIB_PATH", str(tmp_path / "nope.so"))
     with pytest.raises(_lib.SmrError):
         _lib.load()
+
+
+def test_knobs_set_from_two_threads_are_never_seen_half_updated(lib):
+    """The launch knobs that come in pairs are one atomic word each: while one thread flips a
+    pair between two settings, another thread's host-only queries see one setting or the
+    other, never a mix of the two."""
+    import threading
+    stop = threading.Event()
+
+    def flip():
+        i = 0
+        while not stop.is_set():
+            if i & 1:
+                lib.smr_set_reduce_launch(256, 512)
+                lib.smr_set_gemv_launch(16, 2)
+            else:
+                lib.smr_set_reduce_launch(512, 1024)
+                lib.smr_set_gemv_launch(64, 4)
+            i += 1
+
+    t = threading.Thread(target=flip)
+    t.start()
+    try:
+        numel = 8 * 512 * 300             # 153600 slots: (256, 512) -> 512 blocks, (512, 1024) -> 300; a torn pair gives 600
+        seen_reduce, seen_gemv = set(), set()
+        for _ in range(20000):
+            seen_reduce.add(lib.smr_reduce_num_blocks(numel, 0))
+            # (16, 2): 8 * 2 senders; (64, 4): 8 * 4; the column blocks follow the same word
+            seen_gemv.add((lib.smr_gemv_senders(4096, 8192, 8), ))
+        assert seen_reduce <= {512, 300, 256}, seen_reduce       # 256: the default, before the first flip lands
+        assert seen_gemv <= {(16,), (32,), (8,)}, seen_gemv
+    finally:
+        stop.set()
+        t.join()
+        lib.smr_set_reduce_launch(0, 0)
+        lib.smr_set_gemv_launch(0, 0)
+    assert lib.smr_reduce_num_blocks(1 << 25, 0) == 256
+
+
+def test_fused_entry_argument_errors(lib):
+    p = 0x1000
+    f = lib.smr_ag_matmul_fused
+    assert lib.smr_ag_matmul_fused_state_words(8, 2) == 49
+    assert lib.smr_ag_matmul_fused_state_words(9, 1) == 0
+    assert f(p, p, p, p, None, p, 2, 2048, 256, 256, 0, 8, 256, 0, -1, None, None) == -1     # no state
+    assert f(p, p, p, p, p, None, 2, 2048, 256, 256, 0, 8, 256, 0, -1, None, None) == -1     # no address table
+    assert f(p, p, p, p, p, p, 3, 2048, 256, 256, 0, 8, 256, 0, -1, None, None) == -1        # element size
+    assert f(p, p, p, p, p, p, 2, 2048, 256, 200, 0, 8, 256, 0, -1, None, None) == -2        # K % 64
+    assert f(p, p, p, p, p, p, 2, 2048, 256, 256, 0, 8, 256, 2000, -1, None, None) == -1     # producer count
+    assert f(p, p, p, p, p, p, 1, 2048, 256, 192, 0, 8, 256, 0, -1, None, None) == -2        # e4m3fn: K % 128

@@ -80,6 +80,35 @@ def test_all_gather_with_progress(cuda, rank, splits):
     assert progress.cpu().tolist() == prog.tolist()
 
 
+@pytest.mark.parametrize("rank,splits", [(0, 1), (5, 2), (7, 4)])
+def test_flags_go_up_in_the_reference_order(cuda, lib, rank, splits):
+    """The order in which the producer raises the progress flags
+    (triton_all_gather_matmul.py:43-44: sources rank+1, ..., rank+ws-1, rank; splits of a
+    source in order), read from the time stamps it leaves in the trace buffer.  (In the
+    fused launch only the walk of the copy-only workgroups is fixed: a GEMM workgroup that
+    finds its chunk missing copies at it, so a chunk can be complete out of turn.)"""
+    from symm_mem_recipes import all_gather_with_progress
+    ws, rows, K = 8, 2048, 1024                         # 4 MiB per rank: a chunk takes microseconds, the clock ticks every 10 ns
+    a_shard, h, shards, b, b_bits, a_out, c_out = _setup(ws * rows, 8, K, ws, rank, cuda)
+    words = 64 + 256 * 16 * 4
+    trace = torch.zeros(words, dtype=torch.int64, device=cuda)
+    chunks = ws * splits
+    try:
+        assert lib.smr_set_trace_buffer(trace.data_ptr(), words) == 0
+        progress = torch.zeros(chunks, dtype=torch.int32, device=cuda)
+        all_gather_with_progress(a_out, a_shard, progress, splits, num_workgroups=4)
+        torch.cuda.synchronize()
+        h.check_status()
+    finally:
+        lib.smr_set_trace_buffer(None, 0)
+    stamps = trace[:chunks].cpu().tolist()
+    assert all(t > 0 for t in stamps), stamps
+    order = sorted(range(chunks), key=lambda i: stamps[i])
+    assert order == list(O.all_gather_ref(shards, rank, splits)[2]), order
+    assert progress.cpu().tolist() == [1] * chunks
+    assert np.array_equal(_t_bits(a_out), np.concatenate(shards))
+
+
 @pytest.mark.parametrize("ws,rows,K,splits,wgs", [(8, 96, 200, 1, 3), (8, 96, 200, 2, 256), (3, 64, 72, 4, 1),
                                                  (8, 8, 8, 1, 256), (8, 512, 4096, 4, 256)])
 def test_all_gather_at_once(cuda, lib, ws, rows, K, splits, wgs):

@@ -429,3 +429,27 @@ def test_fp8_matmul_vs_torch_cpu():
     same = got[inr] == want[inr]
     assert same.mean() > 0.999
     assert np.all(got[~inr] & 0x7F == 126)
+
+
+def test_torch_restatement_of_the_reduce_matches_the_numpy_oracle():
+    """oracle/torch_reduce.py (what the benchmark times on the CPU) against reduce_ref, bit for
+    bit: N(0,1) data, random bit patterns with infinities and denormals, and fp32 buffers."""
+    import torch
+    from oracle import torch_reduce as T
+    rng = np.random.default_rng(7)
+    n = 4096
+    bits = [O.seeded_normal_bf16_bits(n, seed=r) for r in range(8)]
+    tens = [torch.from_numpy(b.view(np.int16).copy()).view(torch.bfloat16) for b in bits]
+    got = T.reduce_ref_torch(tens).view(torch.int16).numpy().view(np.uint16)
+    assert np.array_equal(got, O.reduce_ref(bits, "bf16"))
+    raw = [rng.integers(0, 1 << 16, size=n, dtype=np.uint16) for _ in range(8)]
+    tens = [torch.from_numpy(b.view(np.int16).copy()).view(torch.bfloat16) for b in raw]
+    got = T.reduce_ref_torch(tens).view(torch.int16).numpy().view(np.uint16)
+    want = O.reduce_ref(raw, "bf16")
+    nan = np.isnan(O.bf16_bits_to_f32(want))
+    assert np.array_equal(np.isnan(O.bf16_bits_to_f32(got)), nan) and np.array_equal(got[~nan], want[~nan])
+    f = [rng.standard_normal(n).astype(np.float32) for _ in range(8)]
+    got = T.reduce_ref_torch([torch.from_numpy(x.copy()) for x in f]).numpy()
+    assert np.array_equal(got.view(np.uint32), O.reduce_ref(f, "fp32").view(np.uint32))
+    # the per-rank generator of the benchmark's CPU leg is deterministic
+    assert torch.equal(T.seeded_normal(64, 3), T.seeded_normal(64, 3))
