@@ -206,6 +206,31 @@ def _time_interleaved(fns, iters, warm, pre=None):
     return [_median(t) for t in ts]
 
 
+def bench_mfma_only(dev):
+    """What the matrix cores sustain with every compute unit issuing bf16 MFMAs back to back on
+    N(0, 0.02) operands and nothing else (smr_probe_mfma_only): the part's power management
+    sets the clock, so this - not the published peak, which assumes the top clock - is what
+    the GEMM's MFMA share can be compared with."""
+    import torch
+    from symm_mem_recipes import _lib
+    lib = _lib.load()
+    cus = torch.cuda.get_device_properties(dev).multi_processor_count
+    vals = torch.empty(1 << 16, dtype=torch.bfloat16, device=dev).normal_(0, 0.02)
+    ticks = torch.zeros(2 * cus, dtype=torch.int64, device=dev)
+    sink = torch.zeros(256 * cus, dtype=torch.float32, device=dev)
+    iters = 20000                                  # about 10 ms per launch: time for the clock to settle
+    st = torch.cuda.current_stream(dev).cuda_stream
+    for _ in range(4):
+        rc = lib.smr_probe_mfma_only(vals.data_ptr(), vals.numel(), cus, iters, ticks.data_ptr(), sink.data_ptr(), st)
+        assert rc == 0
+    torch.cuda.synchronize()
+    t = ticks.view(cus, 2).double()
+    us = (t[:, 0] / 100.0).mean().item()
+    flops = cus * 4.0 * 64 * iters * 16384
+    return {"tflops": flops / us / 1e6, "shader_clock_mhz": (t[:, 1].mean() / us).item(),
+            "cycles_per_mfma": (t[:, 1].mean() / (64.0 * iters)).item(), "workgroups": cus}
+
+
 def bench_ag_matmul(dev, gated=True):
     import torch
     from symm_mem_recipes import EmulatedSymmetricMemory as SM, all_gather_matmul_tma_persistent
@@ -511,6 +536,7 @@ def main():
             [bench_reduce_rotating(k, dev, "bf16", accumulate="bf16") for k in (8192,)] +
             [bench_reduce_rotating(k, dev, "bf16", barrier=True) for k in (8192, 16384)])
         extra["all_gather_matmul"] = bench_ag_matmul(dev)
+        extra["all_gather_matmul"]["mfma_only"] = bench_mfma_only(dev)
         extra["all_gather_matmul_fp8"] = bench_ag_matmul_fp8(dev)
         extra["gemv_allreduce"] = bench_gemv(dev)
         extra["barrier"] = bench_barrier(dev)

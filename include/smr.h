@@ -292,21 +292,37 @@ int smr_set_ag_matmul_grid_limit(int workgroups);
  * engine and needs no compute units, triton_all_gather_matmul.py:46-49). */
 int smr_ag_matmul_grid(int M, int N, int K, int world_size, int comm_block_m, int gated);
 
+/* Measurement aid, no reference counterpart (its launch metadata publishes flops for a
+ * profiler, triton_all_gather_matmul.py:59-69): `workgroups` workgroups of 256 threads issue
+ * 64 * iters v_mfma_f32_16x16x32_bf16 per wave back to back on operands read once from
+ * values_dev (bf16 [nvalues]); nothing else runs in the loop.  What the matrix cores sustain
+ * at the clock the part's power management allows under that load is the ceiling to hold a
+ * GEMM against; the published peak assumes the top clock.
+ *   ticks_dev  uint64 [2 * workgroups]: per workgroup, elapsed ticks of the constant 100 MHz
+ *              clock and elapsed shader clock cycles
+ *   sink_dev   float [256 * workgroups]: keeps the arithmetic alive
+ * FLOPs issued: workgroups * 4 waves * 64 * iters * 16384. */
+int smr_probe_mfma_only(const void* values_dev, int nvalues, int workgroups, int iters,
+                        uint64_t* ticks_dev, float* sink_dev, void* stream);
+
 /* Split-K GEMV + rank-ordered combine through signal-pad flags.  No reference
  * code exists for it in symm_mem_recipes; it reuses the send/wait protocol of
  * triton_barrier.py:119-129 and triton_all_gather_matmul.py:72-95.
  *   x [batch,K] bf16, w [K,N] bf16 row-major, K split into ws rank shards, each
  *   cut further into sub-shards (one workgroup per column block and sub-shard);
  *   S = smr_gemv_senders(N, K, ws) partial producers per column block.
- *   partials fp32 [S, batch, N] scratch; flags uint32 [smr_gemv_flag_blocks(N) * S]
- *   zero on entry and zero again on exit; out [batch,N] bf16 = the fp32 sum of the
- *   S partials in sender order (rank-major), i.e.
+ *   partials fp32 [S, batch, N] scratch; flags uint32 [smr_gemv_flag_words(N, K, ws)]
+ *   (= smr_gemv_flag_blocks(N) * (S + 1): per column block one flag per producer and one
+ *   arrival word), zero on entry and zero again on exit.  Every producer raises its flag and
+ *   counts itself in; the one that arrives last consumes the flags and adds the partials:
+ *   out [batch,N] bf16 = the fp32 sum of the S partials in sender order (rank-major), i.e.
  *   bf16(((0 + p_0) + p_1) + ... + p_{ws-1}) when S == ws.  batch <= 8. */
 int smr_gemv_allreduce(const void* x_dev, const void* w_dev, float* partials_dev,
                        uint32_t* flags_dev, void* out_dev, int batch, int K, int N,
                        int world_size, uint32_t* status, void* stream);
 int smr_gemv_flag_blocks(int N);
 int smr_gemv_senders(int N, int K, int world_size);
+int smr_gemv_flag_words(int N, int K, int world_size);
 
 /* smr_gemv_allreduce for callers that cannot allocate device memory (code under HIP graph
  * capture, tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the

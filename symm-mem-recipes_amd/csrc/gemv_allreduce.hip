@@ -14,11 +14,13 @@
 //
 // Workgroup id -> (sender = rank * sub + sub-shard, column block), column block
 // fastest.  Every workgroup writes its fp32 partial, waits until the stores are
-// acknowledged, and raises flag[column block][sender] (CAS 0 -> 1).  The first
-// workgroup of a column block then consumes all flags (CAS 1 -> 0, so the flags
-// are zero again on exit) and adds the partials in sender order, i.e. rank by
-// rank.  The partials travel with agent-coherent stores and loads, so no cache
-// write-back or invalidate surrounds the flags.
+// acknowledged, raises flag[column block][sender] and counts itself in the column
+// block's arrival word.  The workgroup that arrives last knows that every partial is in
+// place: it consumes all flags (CAS 1 -> 0, so flags and arrival word are zero again on
+// exit) and adds the partials in sender order, i.e. rank by rank.  Nobody spins on a
+// flag that is not up yet, and the end of the kernel is two memory round trips behind the
+// last partial instead of four.  The partials travel with agent-coherent stores and
+// loads, so no cache write-back or invalidate surrounds the flags.
 #include <atomic>
 #include <cstdio>
 #include <mutex>
@@ -179,27 +181,36 @@ __global__ __launch_bounds__(kGemvThreads) void gemv_allreduce_kernel(
   }
 
   // publish the partial: it was written through, so once every thread's stores
-  // are acknowledged and the workgroup has met, one thread raises the flag
+  // are acknowledged and the workgroup has met, one thread raises the flag (nobody waits
+  // for that: the raise is a store-like atomic without a return value) and counts the
+  // workgroup in; the count comes back and tells whether it was the last
   wait_stores_acknowledged();
   __syncthreads();
-  uint32_t* my_flags = flags + (size_t)cblk * senders;
-  if (tid == 0 && !send_signal_relaxed(my_flags + sender, limit_ticks))
-    report(status, SMR_ST_SEND_TIMEOUT, sender, cblk, 0u);
-  if (sender != 0) return;
-
-  // first workgroup of the column block: consume all flags, then add the partials
-  // in rank order (sub-shards of a rank in order inside it)
-  int bad = 0;
-  if (tid < senders && !wait_signal_reset(my_flags + tid, limit_ticks)) {
-    report(status, SMR_ST_WAIT_TIMEOUT, tid, cblk, 0u);
-    bad = 1;
+  uint32_t* my_flags = flags + (size_t)cblk * (senders + 1);
+  __shared__ uint32_t arrived;
+  if (tid == 0) {
+    __hip_atomic_fetch_or(my_flags + sender, 1u, __ATOMIC_RELAXED, kScope);
+    arrived = __hip_atomic_fetch_add(my_flags + senders, 1u, __ATOMIC_RELAXED, kScope);
   }
-  bad = __syncthreads_or(bad);
-  if (bad) return;
+  __syncthreads();
+  if (arrived + 1u != (uint32_t)senders) return;
+
+  // Last arrival of the column block.  The last wave consumes the flags (all raised by now,
+  // or a moment from landing: the wait is the protocol's bounded CAS 1 -> 0) and clears the
+  // arrival word, while the other waves already add the partials in rank order (sub-shards
+  // of a rank in order inside it).
+  constexpr int kCombiners = kGemvThreads - 64;
+  if (tid >= kCombiners) {
+    const int lane = tid - kCombiners;
+    for (int f = lane; f < senders; f += 64)
+      if (!wait_signal_reset(my_flags + f, limit_ticks)) report(status, SMR_ST_WAIT_TIMEOUT, f, cblk, 0u);
+    if (lane == 0) __hip_atomic_store(my_flags + senders, 0u, __ATOMIC_RELAXED, kScope);
+    return;
+  }
   // 16 partials are fetched at a time (independent loads), then added strictly in
   // sender order; the +0 terms that pad the last group cannot change a sum that
   // starts from +0.
-  for (int idx = tid; idx < batch * kCols; idx += kGemvThreads) {
+  for (int idx = tid; idx < batch * kCols; idx += kCombiners) {
     const int b = idx / kCols, c = idx % kCols;
     const int col = cblk * kCols + c;
     if (col >= N) continue;
@@ -289,7 +300,8 @@ static int launch_gemv(const char* who, const void* x_dev, const void* w_dev, fl
   const int64_t grid64 = (int64_t)cblocks * world_size * sub;
   if (grid64 > 4096) return bad(SMR_E_UNSUPPORTED, "more than 4096 workgroups cannot be co-resident");
   const unsigned grid = (unsigned)grid64;
-  if (flag_capacity >= 0 && grid64 > flag_capacity) return bad(SMR_E_UNSUPPORTED, "too many workgroups for the flag array");
+  const int64_t flag_words = (int64_t)cblocks * (world_size * sub + 1);
+  if (flag_capacity >= 0 && flag_words > flag_capacity) return bad(SMR_E_UNSUPPORTED, "too many flags for the flag array");
   if (partial_capacity >= 0 && (int64_t)world_size * sub * batch * N * 4 > partial_capacity)
     return bad(SMR_E_UNSUPPORTED, "partial sums exceed the scratch array (senders * batch * N * 4 bytes)");
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
@@ -298,7 +310,8 @@ static int launch_gemv(const char* who, const void* x_dev, const void* w_dev, fl
   uint16_t* out = reinterpret_cast<uint16_t*>(out_dev);
   const uint64_t lim = spin_limit_ticks();
   if (clear_flags) {
-    hipLaunchKernelGGL(gemv_clear_words_kernel, dim3((grid + 255) / 256), dim3(256), 0, st, flags_dev, (int)grid);
+    hipLaunchKernelGGL(gemv_clear_words_kernel, dim3(((unsigned)flag_words + 255) / 256), dim3(256), 0, st, flags_dev,
+                       (int)flag_words);
     if (int rc = check_hip(hipGetLastError(), who)) return rc;
   }
 #define SMR_GEMV_LAUNCH(BP, TPR)                                                                   \
@@ -336,6 +349,13 @@ int smr_set_gemv_launch(int threads_per_row, int sub_shards) {
 int smr_gemv_flag_blocks(int N) {
   const int cols = smr::gemv_launch_knobs().tpr * 8;
   return N <= 0 ? 0 : (N + cols - 1) / cols;
+}
+
+int smr_gemv_flag_words(int N, int K, int world_size) {
+  if (N <= 0 || K <= 0 || world_size < 1 || world_size > SMR_MAX_WORLD_SIZE) return 0;
+  const smr::GemvLaunch knobs = smr::gemv_launch_knobs();
+  const int cols = knobs.tpr * 8;
+  return ((N + cols - 1) / cols) * (world_size * smr::gemv_sub_for(knobs, N, K, world_size) + 1);
 }
 
 int smr_gemv_senders(int N, int K, int world_size) {

@@ -61,11 +61,13 @@ SIGNATURES = {
     "smr_ag_matmul_plan": (_i, [_i, _i, _i, _i, _i, _p]),
     "smr_ag_matmul_fp8": (_i, [_p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _p, _p]),
     "smr_ag_matmul_plan_fp8": (_i, [_i, _i, _i, _i, _i, _p]),
+    "smr_probe_mfma_only": (_i, [_p, _i, _i, _i, _p, _p, _p]),
     "smr_gemv_allreduce": (_i, [_p, _p, _p, _p, _p, _i, _i, _i, _i, _p, _p]),
     "smr_gemv_allreduce_static": (_i, [_p, _p, _p, _i, _i, _i, _i, _p, _p]),
     "smr_gemv_static_scratch_bytes": (_i64, []),
     "smr_gemv_flag_blocks": (_i, [_i]),
     "smr_gemv_senders": (_i, [_i, _i, _i]),
+    "smr_gemv_flag_words": (_i, [_i, _i, _i]),
     "smr_set_gemv_launch": (_i, [_i, _i]),
 }
 

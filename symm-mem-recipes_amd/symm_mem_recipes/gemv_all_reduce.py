@@ -28,7 +28,8 @@ class GemvWorkspace:
         # partial producers per column block: the ranks, each possibly cut into K sub-shards
         self.senders = lib.smr_gemv_senders(N, K, world_size) if K else 8 * world_size
         self.partials = torch.empty(self.senders, batch, N, dtype=torch.float32, device=device)
-        self.flags = torch.zeros(lib.smr_gemv_flag_blocks(N) * self.senders, dtype=torch.int32, device=device)
+        # per column block one flag per producer and one arrival word
+        self.flags = torch.zeros(lib.smr_gemv_flag_blocks(N) * (self.senders + 1), dtype=torch.int32, device=device)
         self.status = torch.zeros(_lib.STATUS_WORDS, dtype=torch.int32, device=device)
 
     def check_status(self) -> None:
@@ -57,7 +58,7 @@ def gemv_all_reduce(x: torch.Tensor, w: torch.Tensor, world_size: int = 8,
     senders = lib.smr_gemv_senders(N, K, world_size)
     # (the launch shape is a process-wide knob: a workspace made under another setting may be too small)
     assert workspace.senders >= senders, "workspace was built for fewer partial producers"
-    assert workspace.flags.numel() >= lib.smr_gemv_flag_blocks(N) * senders, "workspace has too few flags"
+    assert workspace.flags.numel() >= lib.smr_gemv_flag_words(N, K, world_size), "workspace has too few flags"
     if out is None:
         out = torch.empty(batch, N, dtype=torch.bfloat16, device=x.device)
     rc = _lib.load().smr_gemv_allreduce(

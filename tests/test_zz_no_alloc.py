@@ -22,7 +22,7 @@ def _case(lib, cuda, batch, K, N, ws, seed):
     w = _bits_t(O.seeded_normal_bf16_bits(K * N, seed=seed + 1, std=0.02).reshape(K, N)).to(cuda)
     senders = lib.smr_gemv_senders(N, K, ws)
     partials = torch.empty(senders, batch, N, dtype=torch.float32, device=cuda)
-    flags = torch.zeros(lib.smr_gemv_flag_blocks(N) * senders, dtype=torch.int32, device=cuda)
+    flags = torch.zeros(lib.smr_gemv_flag_words(N, K, ws), dtype=torch.int32, device=cuda)
     want = torch.empty(batch, N, dtype=torch.bfloat16, device=cuda)
     got = torch.full((batch, N), float("nan"), dtype=torch.bfloat16, device=cuda)
     status = torch.zeros(4, dtype=torch.int32, device=cuda)
