@@ -341,6 +341,12 @@ int64_t smr_gemv_static_scratch_bytes(void);
 /* Tuning knob: threads per contiguous row segment (16 or 64; 0 = default 16) and
  * sub-shards per rank (1..8; 0 = chosen so that at least 256 workgroups run). */
 int smr_set_gemv_launch(int threads_per_row, int sub_shards);
+/* Tuning knob: 1 (default) runs batches of 3..8 rows on the matrix cores (W tiles turned
+ * through LDS with transposing reads, v_mfma_f32_16x16x32_bf16 with x padded to 16 rows);
+ * 0 keeps every batch on the vector ALUs (v_dot2c_f32_bf16), as batches of 1 and 2 always
+ * are.  The two kernels add a rank's K rows in different orders: their fp32 partials agree
+ * to rounding, not bit for bit.  Process-wide. */
+int smr_set_gemv_matrix_cores(int on);
 
 #ifdef __cplusplus
 }

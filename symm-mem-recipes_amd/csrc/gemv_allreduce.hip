@@ -43,15 +43,96 @@ constexpr int kGemvKChunk = 1024;            // K rows of x staged in LDS at a t
 static std::atomic<uint32_t> g_gemv_launch{16u};   // sub-shards 0 = pick so that >= 256 workgroups run
 struct GemvLaunch {
   int tpr, sub;
+  bool mfma;      // batches above 2 on the matrix cores (bit 15 of the low half set = off)
 };
 static GemvLaunch gemv_launch_knobs() {
   const uint32_t v = g_gemv_launch.load(std::memory_order_relaxed);
-  return {(int)(v & 0xFFFFu), (int)(v >> 16)};
+  return {(int)(v & 0x7FFFu), (int)(v >> 16), (v & 0x8000u) == 0};
 }
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef __attribute__((address_space(1))) u32x4 GlobalVec;
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+
+// What follows the multiplication, shared by both kernels.  `red` holds the four waves'
+// partial sums as fp32 [wave][BR][kCols]; the workgroup adds them (wave order), writes its
+// partial, raises its flag and counts itself in, and the workgroup that arrives last at the
+// column block combines the partials of all senders in sender order.
+template <int BR, int kCols>
+__device__ __forceinline__ void publish_and_combine(const float* red, float* __restrict__ partials,
+                                                    uint32_t* __restrict__ flags, uint16_t* __restrict__ out,
+                                                    int batch, int N, int cblk, int sender, int senders,
+                                                    uint64_t limit_ticks, uint32_t* status) {
+  const int tid = threadIdx.x;
+  auto red_at = [&](int w, int b, int c) { return red[((size_t)w * BR + b) * kCols + c]; };
+  for (int c = tid; c < kCols; c += kGemvThreads) {
+    const int col = cblk * kCols + c;
+    if (col < N) {
+      for (int b = 0; b < batch; ++b) {
+        const float p = ((red_at(0, b, c) + red_at(1, b, c)) + red_at(2, b, c)) + red_at(3, b, c);
+        store_coherent(&partials[((int64_t)sender * batch + b) * N + col], p);
+      }
+    }
+  }
+
+  // publish the partial: it was written through, so once every thread's stores
+  // are acknowledged and the workgroup has met, one thread raises the flag (nobody waits
+  // for that: the raise is a store-like atomic without a return value) and counts the
+  // workgroup in; the count comes back and tells whether it was the last
+  wait_stores_acknowledged();
+  __syncthreads();
+  uint32_t* my_flags = flags + (size_t)cblk * (senders + 1);
+  __shared__ uint32_t arrived;
+  if (tid == 0) {
+    __hip_atomic_fetch_or(my_flags + sender, 1u, __ATOMIC_RELAXED, kScope);
+    arrived = __hip_atomic_fetch_add(my_flags + senders, 1u, __ATOMIC_RELAXED, kScope);
+  }
+  __syncthreads();
+  if (arrived + 1u != (uint32_t)senders) return;
+
+  // Last arrival of the column block.  The last wave consumes the flags (all raised by now,
+  // or a moment from landing: the wait is the protocol's bounded CAS 1 -> 0) and clears the
+  // arrival word, while the other waves already add the partials in rank order (sub-shards
+  // of a rank in order inside it).
+  constexpr int kCombiners = kGemvThreads - 64;
+  if (tid >= kCombiners) {
+    const int lane = tid - kCombiners;
+    for (int f = lane; f < senders; f += 64)
+      if (!wait_signal_reset(my_flags + f, limit_ticks)) report(status, SMR_ST_WAIT_TIMEOUT, f, cblk, 0u);
+    if (lane == 0) __hip_atomic_store(my_flags + senders, 0u, __ATOMIC_RELAXED, kScope);
+    return;
+  }
+  // All of a thread's outputs at once: their partials are fetched eight senders at a time
+  // (independent loads, a few dozen in flight per thread - one output after the other would
+  // be one memory round trip after the other), then added strictly in sender order; the +0
+  // terms that pad the last group cannot change a sum that starts from +0.
+  constexpr int kOutputs = (8 * kCols + kCombiners - 1) / kCombiners;    // per thread at batch 8
+  const int64_t plane = (int64_t)batch * N;
+  const float* p[kOutputs];
+  float a[kOutputs];
+#pragma unroll
+  for (int e = 0; e < kOutputs; ++e) {
+    const int idx = tid + e * kCombiners;
+    const int b = idx / kCols, col = cblk * kCols + idx % kCols;
+    p[e] = (idx < batch * kCols && col < N) ? partials + (int64_t)b * N + col : nullptr;
+    a[e] = 0.0f;
+  }
+  for (int r0 = 0; r0 < senders; r0 += 8) {
+    float v[kOutputs][8];
+#pragma unroll
+    for (int e = 0; e < kOutputs; ++e)
+#pragma unroll
+      for (int u = 0; u < 8; ++u)
+        v[e][u] = (p[e] != nullptr && r0 + u < senders) ? load_coherent(p[e] + (int64_t)(r0 + u) * plane) : 0.0f;
+#pragma unroll
+    for (int e = 0; e < kOutputs; ++e)
+#pragma unroll
+      for (int u = 0; u < 8; ++u) a[e] += v[e][u];
+  }
+#pragma unroll
+  for (int e = 0; e < kOutputs; ++e)
+    if (p[e] != nullptr) out[p[e] - partials] = (uint16_t)f32_to_bf16_bits(a[e]);
+}
 
 template <int B, int TPR>
 __global__ __launch_bounds__(kGemvThreads) void gemv_allreduce_kernel(
@@ -170,62 +251,131 @@ __global__ __launch_bounds__(kGemvThreads) void gemv_allreduce_kernel(
   }
   __syncthreads();
   static_assert(kKGroupsPerWave * (kGemvThreads / 64) == kKGroups, "row groups = per wave x waves");
-  for (int c = tid; c < kCols; c += kGemvThreads) {
-    const int col = cblk * kCols + c;
-    if (col < N) {
-      for (int b = 0; b < batch; ++b) {
-        const float p = ((red[0][b][c] + red[1][b][c]) + red[2][b][c]) + red[3][b][c];
-        store_coherent(&partials[((int64_t)sender * batch + b) * N + col], p);
-      }
+  publish_and_combine<B, kCols>(&red[0][0][0], partials, flags, out, batch, N, cblk, sender, senders, limit_ticks, status);
+}
+
+// ---------------------------------------------------------------------------
+// The same job on the matrix cores, for batches whose multiply-adds would otherwise bind
+// the kernel (8 rows of x: 33 us on the vector ALUs against 26 us for one row).
+//
+// v_mfma_f32_16x16x32_bf16 wants both operands with K running inside a lane; W has N
+// running inside a row.  A wave therefore puts each 32 x 128 tile of W (32 K rows of its
+// column block) into its own 8 KiB of LDS as it comes - row r at r * 256 bytes, the eight
+// 32-byte column blocks of a row rotated by r so that the reads below spread over the
+// banks - and reads it back transposed with ds_read_b64_tr_b16: within 16 lanes, lane i
+// supplies the address of a 4-element chunk, and receives element i & 3 of the chunks of
+// lanes i >> 2, 4 + (i >> 2), 8 + (i >> 2), 12 + (i >> 2).  With lane i pointing at row
+// 4 * G + (i >> 2) (G = lane / 16), column 4 * (i & 3), that is column i of rows 4 * G .. + 3:
+// half an operand.  The MFMA's K index is ours to assign, as long as x uses the same
+// assignment: position jj of lane group G stands for tile row 16 * (jj >> 2) + 4 * G + (jj & 3).
+// x (padded to 16 rows, the MFMA's M) is the other operand, straight from its LDS copy; the
+// result fragment D[b][n] has the batch row in (lane / 16) * 4 + register and the column in
+// lane % 16, so only the lanes below 32 carry real rows.
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(3))) bf16x4 LdsBf16x4;
+typedef __attribute__((address_space(3))) u32x4 LdsVec;
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef __attribute__((address_space(3))) u32x2 LdsVec2;
+
+constexpr int kMfmaCols = 128;                 // columns per workgroup: 8 blocks of 16
+constexpr int kMfmaTileRows = 32;              // K rows per MFMA
+
+// Needs whole tiles and 8-byte aligned pieces of x: the K rows of a workgroup a multiple of 32.
+__global__ __launch_bounds__(kGemvThreads) void gemv_allreduce_mfma_kernel(
+    const uint16_t* __restrict__ x, const uint8_t* __restrict__ w, float* __restrict__ partials,
+    uint32_t* __restrict__ flags, uint16_t* __restrict__ out, int batch, int K, int N,
+    int world_size, int sub, uint64_t limit_ticks, uint32_t* status) {
+  constexpr int kTileBytes = kMfmaTileRows * kMfmaCols * 2;      // 8 KiB, also one wave's [16][128] fp32 sums
+  __shared__ __attribute__((aligned(16))) uint8_t smem[4 * kTileBytes];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const uint32_t lds_tile = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) void*)smem + wave * kTileBytes;
+
+  const int senders = world_size * sub;
+  const int cblocks = gridDim.x / senders;
+  const int cblk = blockIdx.x % cblocks;
+  const int sender = blockIdx.x / cblocks;
+  const int rank = sender / sub;
+  const int ks = K / world_size;
+  const int kss = ks / sub;                      // (a multiple of 32: the host checks)
+  const int k_begin = rank * ks + (sender % sub) * kss;
+  const int64_t row_bytes = (int64_t)N * 2;
+
+  // this lane's 16 bytes of a tile row: columns 8c .. 8c+7 of the column block (clamped into
+  // the matrix: the columns past N feed results that are never stored)
+  const int c = lane & 15, rsub = lane >> 4;
+  int col = cblk * kMfmaCols + c * 8;
+  if (col > N - 8) col = N - 8;
+  const int G = lane >> 4, i = lane & 15;
+  const __attribute__((address_space(1))) uint8_t* wp =
+      (const __attribute__((address_space(1))) uint8_t*)(uintptr_t)(w + (int64_t)k_begin * row_bytes + (int64_t)col * 2);
+  // x: batch row i (zero beyond the batch), K positions 4G .. 4G+3 and 16 + 4G .. 16 + 4G+3 of a tile
+  typedef __attribute__((address_space(1))) u32x2 GlobalVec2;
+  const GlobalVec2* xp = (const GlobalVec2*)(uintptr_t)(x + (int64_t)(i < batch ? i : 0) * K + k_begin + 4 * G);
+  const bool x_row = i < batch;
+
+  f32x4 acc[8];
+#pragma unroll
+  for (int nb = 0; nb < 8; ++nb) acc[nb] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+
+  struct Tile {
+    u32x4 v[8];
+    u32x2 xlo, xhi;
+  };
+  const int ntiles = kss / kMfmaTileRows;
+  auto load_tile = [&](Tile& tl, int t) {
+#pragma unroll
+    for (int u = 0; u < 8; ++u)
+      tl.v[u] = __builtin_nontemporal_load((const GlobalVec*)(wp + (int64_t)(t * kMfmaTileRows + 4 * u + rsub) * row_bytes));
+    tl.xlo = u32x2{0u, 0u};
+    tl.xhi = u32x2{0u, 0u};
+    if (x_row) {
+      tl.xlo = xp[t * (kMfmaTileRows / 4)];
+      tl.xhi = xp[t * (kMfmaTileRows / 4) + 4];
     }
+  };
+  auto multiply_tile = [&](const Tile& tl) {
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const int r = 4 * u + rsub;
+      *reinterpret_cast<LdsVec*>((uintptr_t)(lds_tile + r * 256 + ((((c >> 1) + r) & 7) << 5) + ((c & 1) << 4))) = tl.v[u];
+    }
+    const u32x4 xw = {tl.xlo.x, tl.xlo.y, tl.xhi.x, tl.xhi.y};
+    const bf16x8 xf = __builtin_bit_cast(bf16x8, xw);
+#pragma unroll
+    for (int nb = 0; nb < 8; ++nb) {
+      const int r0 = 4 * G + (i >> 2), r1 = 16 + r0;
+      const bf16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(
+          reinterpret_cast<LdsBf16x4*>((uintptr_t)(lds_tile + r0 * 256 + (((nb + r0) & 7) << 5) + ((i & 3) << 3))));
+      const bf16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(
+          reinterpret_cast<LdsBf16x4*>((uintptr_t)(lds_tile + r1 * 256 + (((nb + r1) & 7) << 5) + ((i & 3) << 3))));
+      const bf16x8 wf = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+      acc[nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xf, wf, acc[nb], 0, 0, 0);
+    }
+  };
+  // two tiles in turn: the next tile's loads are in flight while this one is multiplied
+  Tile ta, tb;
+  int t = wave;
+  if (t < ntiles) load_tile(ta, t);
+  while (t < ntiles) {
+    const int t1 = t + 4;
+    if (t1 < ntiles) load_tile(tb, t1);
+    multiply_tile(ta);
+    if (t1 >= ntiles) break;
+    t = t1 + 4;
+    if (t < ntiles) load_tile(ta, t);
+    multiply_tile(tb);
   }
 
-  // publish the partial: it was written through, so once every thread's stores
-  // are acknowledged and the workgroup has met, one thread raises the flag (nobody waits
-  // for that: the raise is a store-like atomic without a return value) and counts the
-  // workgroup in; the count comes back and tells whether it was the last
-  wait_stores_acknowledged();
-  __syncthreads();
-  uint32_t* my_flags = flags + (size_t)cblk * (senders + 1);
-  __shared__ uint32_t arrived;
-  if (tid == 0) {
-    __hip_atomic_fetch_or(my_flags + sender, 1u, __ATOMIC_RELAXED, kScope);
-    arrived = __hip_atomic_fetch_add(my_flags + senders, 1u, __ATOMIC_RELAXED, kScope);
-  }
-  __syncthreads();
-  if (arrived + 1u != (uint32_t)senders) return;
-
-  // Last arrival of the column block.  The last wave consumes the flags (all raised by now,
-  // or a moment from landing: the wait is the protocol's bounded CAS 1 -> 0) and clears the
-  // arrival word, while the other waves already add the partials in rank order (sub-shards
-  // of a rank in order inside it).
-  constexpr int kCombiners = kGemvThreads - 64;
-  if (tid >= kCombiners) {
-    const int lane = tid - kCombiners;
-    for (int f = lane; f < senders; f += 64)
-      if (!wait_signal_reset(my_flags + f, limit_ticks)) report(status, SMR_ST_WAIT_TIMEOUT, f, cblk, 0u);
-    if (lane == 0) __hip_atomic_store(my_flags + senders, 0u, __ATOMIC_RELAXED, kScope);
-    return;
-  }
-  // 16 partials are fetched at a time (independent loads), then added strictly in
-  // sender order; the +0 terms that pad the last group cannot change a sum that
-  // starts from +0.
-  for (int idx = tid; idx < batch * kCols; idx += kCombiners) {
-    const int b = idx / kCols, c = idx % kCols;
-    const int col = cblk * kCols + c;
-    if (col >= N) continue;
-    const float* p = partials + (int64_t)b * N + col;
-    const int64_t plane = (int64_t)batch * N;
-    float a = 0.0f;
-    for (int r0 = 0; r0 < senders; r0 += 16) {
-      float v[16];
+  // the wave's sums, [16 rows][128 columns] fp32, into its own tile buffer (nobody else's)
+  float* red = reinterpret_cast<float*>(smem);
 #pragma unroll
-      for (int u = 0; u < 16; ++u) v[u] = r0 + u < senders ? load_coherent(p + (int64_t)(r0 + u) * plane) : 0.0f;
+  for (int nb = 0; nb < 8; ++nb)
 #pragma unroll
-      for (int u = 0; u < 16; ++u) a += v[u];
-    }
-    out[(int64_t)b * N + col] = (uint16_t)f32_to_bf16_bits(a);
-  }
+    for (int e = 0; e < 4; ++e) red[((size_t)wave * 16 + 4 * G + e) * kMfmaCols + nb * 16 + i] = acc[nb][e];
+  __syncthreads();
+  publish_and_combine<16, kMfmaCols>(red, partials, flags, out, batch, N, cblk, sender, senders, limit_ticks, status);
 }
 
 static int gemv_sub_for(const GemvLaunch& knobs, int N, int K, int world_size) {
@@ -324,7 +474,13 @@ static int launch_gemv(const char* who, const void* x_dev, const void* w_dev, fl
     else if (batch <= 4) SMR_GEMV_LAUNCH(4, TPR);                                                  \
     else SMR_GEMV_LAUNCH(8, TPR);                                                                  \
   } while (0)
-  if (knobs.tpr == 16) SMR_GEMV_BATCH(16);
+  // (the matrix-core kernel works in whole 32-row tiles and reads x in 8-byte pieces)
+  const bool whole_tiles = (K / world_size) % sub == 0 && ((K / world_size) / sub) % 32 == 0 &&
+                           (reinterpret_cast<uintptr_t>(x_dev) & 7u) == 0;
+  if (knobs.tpr == 16 && batch > 2 && knobs.mfma && whole_tiles)
+    hipLaunchKernelGGL(gemv_allreduce_mfma_kernel, dim3(grid), dim3(kGemvThreads), 0, st, x, w, partials_dev,
+                       flags_dev, out, batch, K, N, world_size, sub, lim, status);
+  else if (knobs.tpr == 16) SMR_GEMV_BATCH(16);
   else SMR_GEMV_BATCH(64);
 #undef SMR_GEMV_BATCH
 #undef SMR_GEMV_LAUNCH
@@ -342,7 +498,20 @@ int smr_set_gemv_launch(int threads_per_row, int sub_shards) {
     return fail(SMR_E_INVALID, "smr_set_gemv_launch: threads_per_row must be 16 or 64");
   if (sub_shards < 0 || sub_shards > 8)
     return fail(SMR_E_INVALID, "smr_set_gemv_launch: sub_shards must be 0..8");
-  g_gemv_launch.store((uint32_t)threads_per_row | ((uint32_t)sub_shards << 16), std::memory_order_relaxed);
+  // (the matrix-core switch shares the word: keep it)
+  uint32_t old = g_gemv_launch.load(std::memory_order_relaxed), want;
+  do {
+    want = (uint32_t)threads_per_row | (old & 0x8000u) | ((uint32_t)sub_shards << 16);
+  } while (!g_gemv_launch.compare_exchange_weak(old, want, std::memory_order_relaxed));
+  return 0;
+}
+
+int smr_set_gemv_matrix_cores(int on) {
+  using namespace smr;
+  uint32_t old = g_gemv_launch.load(std::memory_order_relaxed), want;
+  do {
+    want = on ? (old & ~0x8000u) : (old | 0x8000u);
+  } while (!g_gemv_launch.compare_exchange_weak(old, want, std::memory_order_relaxed));
   return 0;
 }
 

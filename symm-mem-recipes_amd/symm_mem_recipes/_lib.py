@@ -69,6 +69,7 @@ SIGNATURES = {
     "smr_gemv_senders": (_i, [_i, _i, _i]),
     "smr_gemv_flag_words": (_i, [_i, _i, _i]),
     "smr_set_gemv_launch": (_i, [_i, _i]),
+    "smr_set_gemv_matrix_cores": (_i, [_i]),
 }
 
 _lib: Optional[C.CDLL] = None

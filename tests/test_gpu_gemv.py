@@ -35,12 +35,18 @@ def _within_one_ulp(got, ref, term_sum):
     return np.all(np.abs(got - ref) <= tol)
 
 
-@pytest.fixture(params=[(0, 0), (64, 0), (64, 3)], ids=["default", "wide", "wide-3sub"])
+@pytest.fixture(params=[(0, 0, 1), (0, 0, 0), (0, 2, 1), (64, 0, 1), (64, 3, 1)],
+                ids=["default", "vector-only", "2sub", "wide", "wide-3sub"])
 def launch_shape(request, lib):
-    tpr, sub = request.param
+    """Launch shapes: the default (batches above 2 on the matrix cores where the K rows of a
+    workgroup are whole 32-row tiles), every batch on the vector ALUs, K sub-shards, and the
+    64-thread row segments."""
+    tpr, sub, matrix = request.param
     assert lib.smr_set_gemv_launch(tpr, sub) == 0
+    assert lib.smr_set_gemv_matrix_cores(matrix) == 0
     yield request.param
     lib.smr_set_gemv_launch(0, 0)
+    lib.smr_set_gemv_matrix_cores(1)
 
 
 @pytest.mark.parametrize("batch,K,N,ws", [(1, 512, 128, 8), (4, 1024, 256, 8), (8, 2048, 1000, 8),
