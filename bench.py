@@ -24,18 +24,23 @@ for _p in (ROOT, os.path.join(ROOT, "symm-mem-recipes_amd")):
         sys.path.insert(0, _p)
 
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
-# HBM bytes per launch of the reduce kernel from rocprofv3 FETCH_SIZE / WRITE_SIZE,
+# Memory bytes per launch of the reduce kernel from rocprofv3 FETCH_SIZE / WRITE_SIZE,
 # each scaled by what the counter reads for this script's 512 MiB calibration copy
 # (profiles/one_shot_all_reduce_64MiB_bf16_traffic.md); keyed by MiB per buffer.
-MEASURED_REDUCE_TRAFFIC_BYTES = {64: 604405370}
+MEASURED_REDUCE_TRAFFIC_BYTES = {64: 604043000}
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
 MFMA_FP8_PEAK_TFLOPS = 5000.0   # MI355X dense fp8, published
-# Fabric bytes per launch of the ungated GEMM at M=16384 N=3584 K=8192 (FETCH_SIZE scaled
-# as above plus WRITE_SIZE; profiles/ag_matmul_M16384_N3584_K8192_counters.md).  A counter
-# run cannot hold the gated launch (it serialises kernels); the gated GEMM reads and writes
-# the same tiles in the same order.
-MEASURED_GEMM_TRAFFIC_BYTES = 1618400051
-MEASURED_GEMM_FP8_TRAFFIC_BYTES = 799597261   # the same two counter runs of `bench.py --gemm-only --fp8`
+# Counter figures of the GEMM at M=16384 N=3584 K=8192 from `bench.py --gemm-only` under
+# rocprofv3 --pmc (profiles/ag_matmul_M16384_N3584_K8192_counters.md).  "traffic" is what
+# passes between the XCDs' L2s and the fabric (FETCH_SIZE scaled as above plus WRITE_SIZE):
+# the 256 MiB last-level cache serves part of it, so it is not HBM traffic.  "mfma_busy" is
+# SQ_VALU_MFMA_BUSY_CYCLES per SIMD over the launch's elapsed shader cycles (GRBM_GUI_ACTIVE).
+MEASURED_GEMM_COUNTERS = {
+    "fused": {"traffic": 2240936000, "mfma_busy": 0.712},
+    "ungated": {"traffic": 1620303800, "mfma_busy": 0.744},
+    "hipblaslt": {"traffic": 1596000000, "mfma_busy": 0.790},
+}
+MEASURED_GEMM_FP8_TRAFFIC_BYTES = 799597261   # ungated e4m3fn launch, the same two counter runs with --fp8
 WS = 8
 
 
@@ -261,7 +266,10 @@ def bench_ag_matmul(dev, gated=True):
                 gating_overhead=us_gated / us_ungated - 1.0,
                 roofline={"bound": "mfma", "achieved": flops / us_gated / 1e6, "peak": MFMA_BF16_PEAK_TFLOPS,
                           "unit": "TFLOP/s", "frac": flops / us_gated / 1e6 / MFMA_BF16_PEAK_TFLOPS,
-                          "traffic": MEASURED_GEMM_TRAFFIC_BYTES},
+                          "traffic": MEASURED_GEMM_COUNTERS["fused"]["traffic"],
+                          "traffic_kind": "L2 <-> fabric bytes per launch (last-level cache or HBM behind it)",
+                          "mfma_busy": MEASURED_GEMM_COUNTERS["fused"]["mfma_busy"]},
+                counters_ungated=MEASURED_GEMM_COUNTERS["ungated"], counters_hipblaslt=MEASURED_GEMM_COUNTERS["hipblaslt"],
                 torch_matmul_us=us_lib, torch_matmul_tflops=flops / us_lib / 1e6)
 
 

@@ -65,3 +65,23 @@ def test_trace_of_a_launch(cuda):
         if mode.startswith("fused"):
             assert r["producer_start_us"] is not None and len(r["flags_us"]) >= 6
             assert all(v > r["producer_start_us"] for v in r["flags_us"].values())
+
+
+def test_mfma_only_probe(cuda, lib):
+    """The measurement aid behind the bench's "mfma_only" figure: it runs, every workgroup
+    reports its two clocks, and back-to-back MFMAs issue at 16 cycles apiece (a little more
+    with the loop's branch), which is what the figure's FLOP count assumes."""
+    wgs, iters = 16, 2000
+    vals = torch.empty(4096, dtype=torch.bfloat16, device=cuda).normal_(0, 0.02)
+    ticks = torch.zeros(2 * wgs, dtype=torch.int64, device=cuda)
+    sink = torch.zeros(256 * wgs, dtype=torch.float32, device=cuda)
+    st = torch.cuda.current_stream(cuda).cuda_stream
+    assert lib.smr_probe_mfma_only(vals.data_ptr(), vals.numel(), wgs, iters, ticks.data_ptr(), sink.data_ptr(), st) == 0
+    torch.cuda.synchronize()
+    t = ticks.view(wgs, 2).cpu()
+    assert bool((t > 0).all())
+    per_mfma = t[:, 1].double() / (64.0 * iters)
+    assert 15.9 <= per_mfma.min().item() and per_mfma.max().item() <= 20.0, per_mfma.tolist()
+    assert torch.isfinite(sink).all()
+    assert lib.smr_probe_mfma_only(None, 1, 1, 1, ticks.data_ptr(), sink.data_ptr(), st) == -1
+    assert lib.smr_probe_mfma_only(vals.data_ptr(), 0, 1, 1, ticks.data_ptr(), sink.data_ptr(), st) == -1
