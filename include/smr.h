@@ -223,8 +223,9 @@ int smr_ag_matmul_schedule(int M, int N, int K, int rank, int world_size, int co
  *     too instead of spinning, so the launch finishes whichever of its workgroups are
  *     resident, and needs no second stream and no kernel running beside it;
  *   - pull_first 1: every GEMM workgroup starts by copying at the first remote chunk (as many
- *     workgroups begin on that comm block as on the local one); 0: never; -1: when at least
- *     48 workgroups would otherwise start with a wait.
+ *     workgroups begin on that comm block as on the local one); 0 or negative: only the
+ *     workgroups that wait copy.  Measured slower than 0 at every shape tried; kept for
+ *     measurements.
  *   elem_bytes 2 = smr_ag_matmul's arithmetic (bf16), 1 = smr_ag_matmul_fp8's (e4m3fn).
  *   state_dev  uint32 [smr_ag_matmul_fused_state_words(ws, splits)]: flags, tickets and
  *              counters.  Zero before the first launch; the last workgroup to finish zeroes

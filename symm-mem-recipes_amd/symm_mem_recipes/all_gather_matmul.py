@@ -93,8 +93,8 @@ def all_gather_matmul_tma_persistent(a_shard: torch.Tensor, b: torch.Tensor, a_o
     Keyword arguments beyond the reference's signature (triton_all_gather_matmul.py:219-221):
     ``fused``      None: the library's plan decides between the fused launch and, for a GEMM too
                    short to hide the copy behind, copy-then-multiply; True / False force one.
-    ``pull_first`` None: the GEMM's workgroups copy the first remote chunk themselves when enough
-                   of them would otherwise start with a wait; True / False force it.
+    ``pull_first`` True: every GEMM workgroup copies at the first remote chunk before its first
+                   tile; None / False: only the workgroups that wait for a chunk copy at it.
     ``producer_workgroups`` copy-only workgroups of the fused launch; None = the plan's.
     ``check``      synchronise and raise if a bounded wait inside the kernel expired (the result
                    is then not valid); without it the caller looks at ``check_status()`` later.

@@ -274,9 +274,9 @@ def test_fused_launch_replays_from_a_graph(cuda, either_form, M, N, K):
 
 @pytest.mark.parametrize("M,N,K,rank,splits", [(16384, 2048, 256, 0, 1), (16384, 2048, 192, 5, 1), (16384, 3072, 128, 7, 2)])
 def test_first_chunk_pulled_by_the_gemm(cuda, lib, M, N, K, rank, splits):
-    """Enough workgroups would wait for the first remote chunk that every GEMM workgroup copies
-    at it before its first tile: same product, bit for bit, as with the copying left to the
-    copy-only workgroups and the waiters; gathered operand complete; state zero again."""
+    """On request every GEMM workgroup copies at the first remote chunk before its first tile:
+    same product, bit for bit, as with the copying left to the copy-only workgroups and the
+    waiters (the default); gathered operand complete; state zero again."""
     from symm_mem_recipes import all_gather_matmul_tma_persistent
     ws = 8
     a_shard, h, shards, b, b_bits, a_out, c_out = _setup(M, N, K, ws, rank, cuda)

@@ -56,7 +56,7 @@ def test_trace_of_a_launch(cuda):
     """The kernels' own time stamps: every workgroup's tiles in order, the producer's flags
     behind its start, and the fused launch's first wait no longer than the whole launch."""
     from symm_mem_recipes import trace
-    for mode in ("ungated", "fused", "fused-no-pull", "sequential"):
+    for mode in ("ungated", "fused", "fused-pull", "sequential"):
         r = trace.trace_launch(16384, 2048, 256, mode, warm=2)
         assert r["end_us"] > 0 and r["steps"], mode
         assert sum(s["workgroups"] for s in r["steps"]) == (16384 // 256) * (2048 // 256), mode
