@@ -188,17 +188,22 @@ def bench_reduce_rotating(size_kib, dev, dtype_name="bf16", write_all=False, acc
 
 
 def _time_interleaved(fns, iters, warm, pre=None):
-    """Median device time in microseconds of each fn in `fns`, the calls taken in turn
-    (a, b, c, a, b, c, ...): variants measured one block after another see different
-    clocks, because the part's power management reacts to the last milliseconds of load."""
+    """Median device time in microseconds of each fn in `fns`, one call of each per round in
+    an order drawn afresh for every round (seeded): variants measured one block after another
+    see different clocks, because the part's power management reacts to the last milliseconds
+    of load, and in a fixed order every variant would always run behind the same other one."""
+    import random
     import torch
     for _ in range(warm):
         for fn in fns:
             fn()
     torch.cuda.synchronize()
     ts = [[] for _ in fns]
+    rng = random.Random(0)
     for _ in range(iters):
-        for k, fn in enumerate(fns):
+        order = list(enumerate(fns))
+        rng.shuffle(order)
+        for k, fn in order:
             if pre is not None:
                 pre()
             a = torch.cuda.Event(enable_timing=True)
