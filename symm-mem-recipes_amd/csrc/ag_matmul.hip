@@ -831,6 +831,9 @@ __device__ __forceinline__ void copy_pieces(const CopyJob& job, int c, uint32_t 
 // A workgroup is through: the last one puts the launch's state back to zero.
 __device__ __forceinline__ void leave(const CopyJob& job) {
   if (threadIdx.x != 0) return;
+  // this thread's own last flag store has landed before the workgroup counts as gone: the
+  // zeroing below must not be overtaken by it
+  wait_stores_acknowledged();
   const uint32_t prev = __hip_atomic_fetch_add(job.exits, 1u, __ATOMIC_RELAXED, kScope);
   if (prev + 1u != gridDim.x) return;
   // every other workgroup's last access to these words lies before its count above
