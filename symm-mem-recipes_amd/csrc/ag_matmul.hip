@@ -1033,32 +1033,58 @@ static int total_steps(const GemmSchedule& s) {
          ceil_div(s.tail * half, s.grid);
 }
 
-// Coarse model of a fused launch, for splitting the compute units between the GEMM
-// and the producer.  Rates measured on MI355X with both kernels running: a GEMM
-// workgroup sustains about 6 TFLOP/s, a producer workgroup moves about 35 GB/s
-// (bytes read plus bytes written) and spends about 2.5 us per chunk on publishing it.
+// Coarse model of a fused launch, for splitting the compute units between the GEMM and the
+// copy and for choosing between the fused launch and copy-then-multiply.  Its constants are
+// fitted to launches timed on MI355X (ten shapes from M=2048 to M=32768, bf16 and e4m3fn,
+// both forms of each): a GEMM workgroup sustains 6.5 TFLOP/s on 256x256 tiles next to the copy
+// (6.6 without it, half of that on narrower tiles, twice that in e4m3fn) plus 6 us per tile;
+// a copy-only workgroup moves 25 GB/s (bytes read plus bytes written) while the GEMM runs;
+// while workgroups wait for a chunk everybody copies at 10 GB/s apiece, and four fifths of such
+// a wait show in the launch's duration.
 struct FusedEstimate {
   double gemm_us, copy_us, total_us;
   int producer_wgs;
 };
 constexpr int kMaxProducerWgs = 128;
-// copy-then-multiply is chosen when its estimate is below this multiple of the fused one
-constexpr double kSequentialBias = 1.0;
-// every chunk ends with a wait for the stores, a workgroup barrier and an arrival count
-static double copy_us(double bytes, int chunks, int wgs) { return bytes / (wgs * 35.0e3) + 2.5 * chunks; }
+constexpr double kCopyOnlyBytesPerUs = 25.0e3, kWaiterBytesPerUs = 10.0e3, kWaitShows = 0.8;
+static double model_tile_us(int BM, int BN, int K, int elem_bytes, bool beside_copy) {
+  double rate = BM == 256 && BN == 256 ? (beside_copy ? 6.5e6 : 6.6e6) : 3.2e6;      // FLOP per us
+  if (elem_bytes == 1) rate *= 2.0;
+  return 2.0 * BM * BN * K / rate + 6.0;
+}
 static FusedEstimate estimate_fused(const GemmSchedule& s, int cus, int grid, int elem_bytes = 2) {
-  // (e4m3fn: twice the MFMA rate per workgroup, half the bytes to copy)
-  const double tile_us = 2.0 * s.BM * s.BN * s.K / (elem_bytes == 1 ? 12.0e6 : 6.0e6) + 8.0;
+  const double tile_us = model_tile_us(s.BM, s.BN, s.K, elem_bytes, true);
   const int tiles = (s.M / s.BM) * ceil_div(s.N, s.BN);
   const int tiles_per_cb = (s.comm_block_m / s.BM) * ceil_div(s.N, s.BN);
+  const int n_comm = s.M / s.comm_block_m, per_rank = n_comm / s.world_size;
   FusedEstimate e;
   e.producer_wgs = cus - grid < kMaxProducerWgs ? cus - grid : kMaxProducerWgs;
   if (e.producer_wgs < 1) e.producer_wgs = 1;
-  const double remote_bytes = 2.0 * elem_bytes * s.M * s.K * (s.world_size - 1) / s.world_size;
-  e.gemm_us = ceil_div(tiles, grid) * tile_us;
-  e.copy_us = copy_us(remote_bytes, s.M / s.comm_block_m, e.producer_wgs);
-  const double tail_us = e.copy_us + ceil_div(tiles_per_cb, grid) * tile_us;
-  e.total_us = e.gemm_us > tail_us ? e.gemm_us : tail_us;
+  const double chunk_bytes = 2.0 * elem_bytes * s.comm_block_m * s.K;         // read and written
+  const double remote_bytes = chunk_bytes * (n_comm - per_rank);
+  const int passes = ceil_div(tiles, grid);
+  // Pass by pass, tiles in ring order: a pass starts when the chunks it touches are in place;
+  // what is missing then is copied by the copy-only workgroups and the workgroups that wait.
+  double now = 0.0, copied = 0.0;
+  for (int pass = 0; pass < passes; ++pass) {
+    const int first = pass * grid;
+    const int last = (tiles < first + grid ? tiles : first + grid) - 1;
+    double need = (last / tiles_per_cb + 1 - per_rank) * chunk_bytes;
+    if (need > remote_bytes) need = remote_bytes;
+    if (copied < need) {
+      const int first_missing = (per_rank + (int)(copied / chunk_bytes)) * tiles_per_cb;
+      const int waiting = last + 1 - (first > first_missing ? first : first_missing);
+      // (with that many at it at once the copy-only workgroups move no more than the others)
+      now += kWaitShows * (need - copied) / ((e.producer_wgs + (waiting > 0 ? waiting : 0)) * kWaiterBytesPerUs);
+      copied = need;
+    }
+    now += tile_us;
+    copied += e.producer_wgs * kCopyOnlyBytesPerUs * tile_us;
+    if (copied > remote_bytes) copied = remote_bytes;
+  }
+  e.gemm_us = passes * tile_us;
+  e.copy_us = remote_bytes / (e.producer_wgs * kCopyOnlyBytesPerUs);
+  e.total_us = now;
   return e;
 }
 
@@ -1322,19 +1348,18 @@ static void fill_plan(int M, int N, int K, int world_size, int comm_block_m, int
   // The alternative for a problem too small to hide the copy behind: copy with the
   // whole GPU, then multiply with the whole GPU.
   const GemmSchedule u = make_schedule(M, N, K, 0, world_size, comm_block_m, cus, false, elem_bytes);
-  // (with no copy next to it a GEMM workgroup sustains a little more: 6.4 TFLOP/s)
-  const double tile_us = 2.0 * u.BM * u.BN * K / (elem_bytes == 1 ? 12.8e6 : 6.4e6) + 8.0;
+  const double tile_us = model_tile_us(u.BM, u.BN, K, elem_bytes, false);
   const int tiles = (M / u.BM) * ceil_div(N, u.BN);
   // the ungated schedule ends on a pass of half tiles when that is shorter: count passes in halves
   const double passes = ceil_div(2 * tiles, u.grid) * 0.5;
   // (all chunks at once, the own shard included: read + write at what a copy reaches on the part)
-  const double gather_us = 2.0 * elem_bytes * M * K / 5.0e6 + 4.0;
+  const double gather_us = 2.0 * elem_bytes * M * K / 5.4e6 + 4.0;
   const double seq_us = gather_us + passes * tile_us + 5.0;
   out5[0] = s.grid;
   out5[1] = e.producer_wgs;
   out5[2] = (int32_t)(e.total_us + 0.5);
   out5[3] = (int32_t)(seq_us + 0.5);
-  out5[4] = seq_us < kSequentialBias * e.total_us ? 1 : 0;
+  out5[4] = seq_us < e.total_us ? 1 : 0;
 }
 
 int smr_ag_matmul_plan(int M, int N, int K, int world_size, int comm_block_m, int32_t* out5) {

@@ -214,12 +214,12 @@ def test_fused_back_to_back_calls_are_identical(cuda, either_form):
 
 def test_copy_then_multiply_matches_fused(cuda, lib):
     """A GEMM too short to hide the copy behind is planned as copy-then-multiply
-    (M=4096 N=1792 K=4096 is); the planned form and both forced forms give the oracle's
+    (M=2048 N=4096 K=2048 is); the planned form and both forced forms give the oracle's
     product and one another's bits, with the gathered operand complete in each."""
     import ctypes
     import importlib
     agm = importlib.import_module("symm_mem_recipes.all_gather_matmul")
-    M, N, K, ws, rank = 4096, 1792, 4096, 8, 3
+    M, N, K, ws, rank = 2048, 4096, 2048, 8, 3
     plan = (ctypes.c_int32 * 5)()
     assert lib.smr_ag_matmul_plan(M, N, K, ws, M // ws, plan) == 0 and plan[4] == 1
     a_shard, h, shards, b, b_bits, a_out, c_out = _setup(M, N, K, ws, rank, cuda)
