@@ -815,6 +815,12 @@ __device__ __forceinline__ void copy_pieces(const CopyJob& job, int c, uint32_t 
       if (t0 < pieces) load(v0, t0);
     }
   }
+  // A wait the compiler can see (the builtin, not assembly text): its own count of loads in
+  // flight is per register and joins all paths, so behind the loop above it takes the piece
+  // registers for possibly still being loaded - and would put its wait for them where they are
+  // next written, which is in the middle of a K loop (every direct-to-LDS load drained once per
+  // trip: the 256x128 and 128x128 kernels ran 30 % slower that way).
+  __builtin_amdgcn_s_waitcnt(0x0F70);      // vmcnt(0), the other counters left alone
   if (mine == 0) return;
   // written through: once acknowledged the pieces are where every XCD reads them
   wait_stores_acknowledged();

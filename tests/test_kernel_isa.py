@@ -51,7 +51,8 @@ def _k_loops(lines):
     return loops
 
 
-@pytest.mark.parametrize("key", [(256, 256, False), (256, 256, True)])
+@pytest.mark.parametrize("key", [(256, 256, False), (256, 256, True), (256, 128, False), (128, 128, False),
+                                 (256, 128, True), (128, 128, True)])
 def test_k_loop_keeps_its_registers(kernels, key):
     assert key in kernels, sorted(kernels)
     loops = _k_loops(kernels[key])
@@ -59,9 +60,16 @@ def test_k_loop_keeps_its_registers(kernels, key):
     for body in loops:
         text = "\n".join(body)
         mfma = len(re.findall(r"v_mfma_", text))
-        assert mfma in (16, 32, 64, 128), mfma                   # one slab pair per trip (full or half-width tile)
+        assert mfma in (4, 8, 16, 32, 64, 128), mfma             # one slab pair per trip (full or half-width tile)
         assert "scratch_" not in text, "spill inside the K loop"
         assert "v_accvgpr" not in text, "accumulators moved between register files inside the K loop"
         assert "lane_b32" not in text, "scalar registers spilled inside the K loop"
         assert re.search(r"s_waitcnt vmcnt\((8|4)\)", text), "the explicit wait for the tile loads is missing"
         assert len(re.findall(r"s_barrier", text)) == 1
+        # The tile loads are assembly and waited for by hand, once per trip.  A wait of the
+        # compiler's own inside the loop (it once took the copy code's piece registers for still
+        # being loaded and waited where the loop first wrote one of them) drains all of them
+        # every trip: the narrower kernels ran 30 % slower, every parity test green.
+        waits = [i for i, x in enumerate(body) if re.search(r"s_waitcnt.*vmcnt", x)]
+        by_hand = [i for i in waits if "ASMSTART" in body[i - 1]]
+        assert len(by_hand) == 1 and waits == by_hand, [body[i].strip() for i in waits]
