@@ -1041,20 +1041,21 @@ static int total_steps(const GemmSchedule& s) {
 
 // Coarse model of a fused launch, for splitting the compute units between the GEMM and the
 // copy and for choosing between the fused launch and copy-then-multiply.  Its constants are
-// fitted to launches timed on MI355X (ten shapes from M=2048 to M=32768, bf16 and e4m3fn,
-// both forms of each): a GEMM workgroup sustains 6.5 TFLOP/s on 256x256 tiles next to the copy
-// (6.6 without it, half of that on narrower tiles, twice that in e4m3fn) plus 6 us per tile;
-// a copy-only workgroup moves 25 GB/s (bytes read plus bytes written) while the GEMM runs;
-// while workgroups wait for a chunk everybody copies at 10 GB/s apiece, and four fifths of such
-// a wait show in the launch's duration.
+// fitted to launches timed on MI355X (24 problems from M=1024 to M=32768, bf16 and e4m3fn, both
+// forms of each): a GEMM workgroup sustains 6.5 TFLOP/s on 256x256 tiles next to the copy (6.6
+// without it, 4.6 on narrower tiles, twice that in e4m3fn) plus 6 us per tile; a copy-only
+// workgroup moves 25 GB/s (bytes read plus bytes written) while the GEMM runs; while workgroups
+// wait for a chunk everybody copies at 12 GB/s apiece, and three fifths of such a wait show in
+// the launch's duration; a fused launch costs 18 us on top (the first pieces' way through
+// tickets, loads, write-through stores and flags), copy-then-multiply 10 us for its two launches.
 struct FusedEstimate {
   double gemm_us, copy_us, total_us;
   int producer_wgs;
 };
 constexpr int kMaxProducerWgs = 128;
-constexpr double kCopyOnlyBytesPerUs = 25.0e3, kWaiterBytesPerUs = 10.0e3, kWaitShows = 0.8;
+constexpr double kCopyOnlyBytesPerUs = 25.0e3, kWaiterBytesPerUs = 12.0e3, kWaitShows = 0.6, kFusedFixedUs = 18.0;
 static double model_tile_us(int BM, int BN, int K, int elem_bytes, bool beside_copy) {
-  double rate = BM == 256 && BN == 256 ? (beside_copy ? 6.5e6 : 6.6e6) : 3.2e6;      // FLOP per us
+  double rate = BM == 256 && BN == 256 ? (beside_copy ? 6.5e6 : 6.6e6) : 4.6e6;      // FLOP per us
   if (elem_bytes == 1) rate *= 2.0;
   return 2.0 * BM * BN * K / rate + 6.0;
 }
@@ -1071,7 +1072,7 @@ static FusedEstimate estimate_fused(const GemmSchedule& s, int cus, int grid, in
   const int passes = ceil_div(tiles, grid);
   // Pass by pass, tiles in ring order: a pass starts when the chunks it touches are in place;
   // what is missing then is copied by the copy-only workgroups and the workgroups that wait.
-  double now = 0.0, copied = 0.0;
+  double now = kFusedFixedUs, copied = 0.0;
   for (int pass = 0; pass < passes; ++pass) {
     const int first = pass * grid;
     const int last = (tiles < first + grid ? tiles : first + grid) - 1;
@@ -1360,7 +1361,7 @@ static void fill_plan(int M, int N, int K, int world_size, int comm_block_m, int
   const double passes = ceil_div(2 * tiles, u.grid) * 0.5;
   // (all chunks at once, the own shard included: read + write at what a copy reaches on the part)
   const double gather_us = 2.0 * elem_bytes * M * K / 5.4e6 + 4.0;
-  const double seq_us = gather_us + passes * tile_us + 5.0;
+  const double seq_us = gather_us + passes * tile_us + 10.0;
   out5[0] = s.grid;
   out5[1] = e.producer_wgs;
   out5[2] = (int32_t)(e.total_us + 0.5);

@@ -1,6 +1,7 @@
 """The fused launch's copy protocol (tickets, piece counts, flags, self-zeroing state) run on the
 CPU: the copy functions are cut out of ag_matmul.hip as they are, their four device-only
-statements (address-space typedefs, the LDS slot, the write-through store, the streaming load)
+statements (address-space typedefs, the LDS slot, the write-through store, the streaming load,
+the wait for the memory counter)
 replaced by host stand-ins, and compiled with AddressSanitizer next to a harness that runs one
 host thread per GPU thread (tests/cpu/copy_protocol_harness.cpp)."""
 import os
@@ -22,6 +23,7 @@ STAND_INS = [
      "store_checked(dst + i, v[u]);"),
     ("__builtin_nontemporal_load(src + (i < job.chunk_vecs ? i : job.chunk_vecs - 1))",
      "load_checked(src + (i < job.chunk_vecs ? i : job.chunk_vecs - 1))"),
+    ("__builtin_amdgcn_s_waitcnt(0x0F70);", ";"),
 ]
 
 
