@@ -504,15 +504,28 @@ __device__ __forceinline__ void run_tile(const TileContext& cx, const TileRef& t
 // The same tile with e4m3fn operands and result (the reference's FP8_OUTPUT switch,
 // triton_all_gather_matmul.py:115,123,188).  A row of a slab is still 128 bytes, now
 // 128 K values; everything that moves bytes (the ring, the loads, the swizzle, the
-// waits) is the bf16 tile's.  The MFMA is v_mfma_f32_32x32x64_f8f6f4: an operand
-// fragment is 32 rows x 64 K, lane l holds row l & 31 and the 32 bytes number l >> 5
-// of the two, i.e. chunks 4*kk + 2*(l >> 5) and the one after it in K step kk
-// (0 or 1).  Both operands use the same lane -> K mapping, which is all the sum
-// over K needs.  The 8 lanes x 2 that an LDS read serves together are 8 consecutive
-// rows at two chunks that differ by 2: the case row_swizzle is built for.
-// A wave of a 256x256 tile holds 4 x 4 accumulators of 16 registers.
+// waits) is the bf16 tile's.  The MFMA is v_mfma_f32_16x16x128_f8f6f4 (without scales:
+// both operands e4m3fn as they are): it computes what the 32x32x64 form computes in as
+// many cycles and draws less power, as with bf16 - a loop of nothing but MFMAs on
+// N(0, 0.5) operands runs 7 to 9 % faster with it, and this kernel's clock is
+// power-limited too.  An operand fragment is 16 rows x 128 K, one whole slab row per
+// fragment row: lane l holds row l & 15 and the 32 bytes number l >> 4 of the four
+// (chunks 2 * (l >> 4) and the one after it).  Both operands use the same lane -> K
+// mapping, which is all the sum over K needs.  The 8 lanes x 2 that an LDS read serves
+// together are 8 consecutive rows at two chunks that differ by 4; row_swizzle separates
+// those as well (four distinct values in bits 0,1 over the rows of one parity, bit 2
+// left to the chunk).
+//
+// One K step is a whole slab pair, and a fragment is 8 registers, so the fragments cannot
+// all be double-buffered: the A fragments are (two sets, taken in turn by trip parity),
+// the B fragments are one set whose halves are refilled while the other half is in use.
+// A trip's MFMAs go B row by B row; the workgroup barrier stands in the middle:
+//   first half   MFMAs with B fragments 0 .. FN/2-1; B fragments FN/2 .. FN-1 of this
+//                slab pair are read; loads of A slab kt+2 are issued
+//   barrier      slab pair kt is read by everyone, pair kt+1 has landed
+//   second half  MFMAs with B fragments FN/2 .. FN-1; the other set of A fragments and
+//                B fragments 0 .. FN/2-1 are read from pair kt+1; loads of B slab kt+2
 typedef int i32x8 __attribute__((ext_vector_type(8)));
-typedef float f32x16 __attribute__((ext_vector_type(16)));
 
 __device__ __forceinline__ uint32_t pack_fp8x4(float a, float b, float c, float d) {
   // saturate to the largest finite e4m3fn value, keep NaN (cvt.rn.satfinite semantics)
@@ -522,6 +535,17 @@ __device__ __forceinline__ uint32_t pack_fp8x4(float a, float b, float c, float 
   return (uint32_t)w;
 }
 
+// D += A x B on a 16x16x128 e4m3fn fragment pair; the accumulator named as an accumulation
+// register for the reason given at mfma_bf16.
+__device__ __forceinline__ void mfma_fp8(f32x4& acc, const i32x8& first, const i32x8& second) {
+  asm volatile("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, %0" : "+a"(acc) : "v"(first), "v"(second));
+}
+
+template <int P>
+struct Parity {
+  static constexpr int value = P;
+};
+
 template <int BM, int BN, typename Between>
 __device__ __forceinline__ void run_tile_fp8(const TileContext& cx, const TileRef& tile,
                                              const uint8_t* a_rows, const uint8_t* b_rows,
@@ -529,8 +553,7 @@ __device__ __forceinline__ void run_tile_fp8(const TileContext& cx, const TileRe
   using T = GemmTile<BM, BN>;
   const uint8_t* a_base = uniform_ptr(a_rows);
   const uint8_t* b_base = uniform_ptr(b_rows);
-  constexpr int WM = T::WM, WN = T::WN, GA = T::GA, GB = T::GB;
-  constexpr int FM = WM / 32, FN = WN / 32;          // 32x32 fragments per wave tile
+  constexpr int WM = T::WM, WN = T::WN, FM = T::FM, FN = T::FN, GA = T::GA, GB = T::GB;
   constexpr uint32_t kSlot = T::kSlotBytes;
   const int lane = cx.lane, wave = cx.wave;
   const int wm = wave >> 1, wn = wave & 1;
@@ -543,16 +566,14 @@ __device__ __forceinline__ void run_tile_fp8(const TileContext& cx, const TileRe
 
   int ln = lane;
   asm volatile("" : "+v"(ln));
-  // fragment read addresses: [K step][first or second chunk of the lane's 32 bytes]
-  uint32_t a_fr[2][2], b_fr[2][2];
+  // fragment read addresses: first and second chunk of the lane's 32 bytes
+  uint32_t a_fr[2], b_fr[2];
 #pragma unroll
-  for (int kk = 0; kk < 2; ++kk)
-#pragma unroll
-    for (int q = 0; q < 2; ++q) {
-      const int pos = (4 * kk + 2 * (ln >> 5) + q) ^ row_swizzle(ln & 15);
-      a_fr[kk][q] = lds0 + (uint32_t)((wm * WM + (ln & 31)) * kRowBytes + (pos << 4));
-      b_fr[kk][q] = lds0 + kSlot + (uint32_t)((wn * WN + (ln & 31)) * kRowBytes + (pos << 4));
-    }
+  for (int q = 0; q < 2; ++q) {
+    const int pos = (2 * (ln >> 4) + q) ^ row_swizzle(ln & 15);
+    a_fr[q] = lds0 + (uint32_t)((wm * WM + (ln & 15)) * kRowBytes + (pos << 4));
+    b_fr[q] = lds0 + kSlot + (uint32_t)((wn * WN + (ln & 15)) * kRowBytes + (pos << 4));
+  }
   uint32_t a_at = 0, b_at = kSlot;
 
   const int u = (ln & 7) ^ row_swizzle(ln >> 3);
@@ -572,20 +593,17 @@ __device__ __forceinline__ void run_tile_fp8(const TileContext& cx, const TileRe
     b_off[j] = (uint32_t)r * row_stride + (uint32_t)((u ^ ((q & 1) << 2)) << 4);
   }
 
-  f32x16 acc[FN][FM];
+  f32x4 acc[FN][FM];
 #pragma unroll
   for (int ni = 0; ni < FN; ++ni)
 #pragma unroll
     for (int mi = 0; mi < FM; ++mi)
 #pragma unroll
-      for (int e = 0; e < 16; ++e) acc[ni][mi][e] = 0.0f;
+      for (int e = 0; e < 4; ++e) acc[ni][mi][e] = 0.0f;
 
-  // one 128-bit read = half a fragment: reads 0 .. 2*FM-1 fill A, the rest B
-  auto read_half = [&](i32x8 (&af)[FM], i32x8 (&bf)[FN], int kk, int r) {
-    const bool is_a = r < 2 * FM;
-    const int f = (is_a ? r : r - 2 * FM) >> 1, q = r & 1;
-    const u32x4 v = lds_read_b128((is_a ? a_fr[kk][q] : b_fr[kk][q]) + f * (32 * kRowBytes));
-    i32x8& dst = is_a ? af[f] : bf[f];
+  // one 128-bit read = half a fragment (q = 0 or 1) of fragment row f
+  auto read_half = [&](i32x8& dst, uint32_t (&fr)[2], int f, int q) __attribute__((always_inline)) {
+    const u32x4 v = lds_read_b128(fr[q] + f * (16 * kRowBytes));
     dst[4 * q + 0] = (int)v.x;
     dst[4 * q + 1] = (int)v.y;
     dst[4 * q + 2] = (int)v.z;
@@ -596,102 +614,123 @@ __device__ __forceinline__ void run_tile_fp8(const TileContext& cx, const TileRe
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
 
-  i32x8 af0[FM], bf0[FN], af1[FM], bf1[FN];
-  constexpr int kMfma = FM * FN, kReads = 2 * (FM + FN);
+  constexpr int HN = FN / 2;                      // B fragments per half of a trip
+  constexpr int kHalf = FM * HN;                  // MFMAs per half
+  i32x8 af[2][FM], bf[FN];
 #pragma unroll
-  for (int r = 0; r < kReads; ++r) read_half(af0, bf0, 0, r);
+  for (int f = 0; f < FM; ++f)
+#pragma unroll
+    for (int q = 0; q < 2; ++q) read_half(af[0][f], a_fr, f, q);
+#pragma unroll
+  for (int f = 0; f < HN; ++f)
+#pragma unroll
+    for (int q = 0; q < 2; ++q) read_half(bf[f], b_fr, f, q);
 
-  // the reads of the next K step go under the first three quarters of the MFMAs
-  constexpr int kReadSpan = kMfma * 3 / 4;
-  auto mfma = [&](const i32x8& bfrag, const i32x8& afrag, f32x16& d) {
-    // scale exponents 127 = 2^0 on both operands
-    d = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(bfrag, afrag, d, 0, 0, 0, 0x7F7F7F7F, 0, 0x7F7F7F7F);
-  };
-  auto first_step = [&](const uint8_t* ak, uint32_t la) {
-#pragma unroll
-    for (int ni = 0; ni < FN; ++ni) {
-#pragma unroll
-      for (int mi = 0; mi < FM; ++mi) {
-        const int slot = ni * FM + mi;
-        mfma(bf0[ni], af0[mi], acc[ni][mi]);
-#pragma unroll
-        for (int r = 0; r < kReads; ++r)
-          if (r * kReadSpan / kReads == slot) read_half(af1, bf1, 1, r);
-#pragma unroll
-        for (int g = 0; g < GA; ++g)
-          if (g * kMfma / GA == slot) load_group(ak, a_off[g], la + g * 1024);
-        __builtin_amdgcn_sched_barrier(0);
-      }
-    }
-  };
-  auto second_step = [&](int kt) {
-    const int kb = kt + 2 < nk ? kt + 2 : nk - 1;
-    const uint8_t* bk = b_base + (int64_t)kb * kRowBytes;
-    const uint32_t lb = lds0 + a_at + wave * (GB * 1024);
-    const uint32_t a_to = a_at + 2 * kSlot < kRingSlots * kSlot ? a_at + 2 * kSlot : a_at + 2 * kSlot - kRingSlots * kSlot;
-    const uint32_t b_to = b_at + 2 * kSlot < kRingSlots * kSlot ? b_at + 2 * kSlot : b_at + 2 * kSlot - kRingSlots * kSlot;
-#pragma unroll
-    for (int kk = 0; kk < 2; ++kk)
-#pragma unroll
-      for (int q = 0; q < 2; ++q) {
-        a_fr[kk][q] += a_to - a_at;
-        b_fr[kk][q] += b_to - b_at;
-      }
-    a_at = a_to;
-    b_at = b_to;
-#pragma unroll
-    for (int ni = 0; ni < FN; ++ni) {
-#pragma unroll
-      for (int mi = 0; mi < FM; ++mi) {
-        const int slot = ni * FM + mi;
-        mfma(bf1[ni], af1[mi], acc[ni][mi]);
-#pragma unroll
-        for (int g = 0; g < GB; ++g)
-          if (g * (kMfma / 2) / GB == slot) load_group(bk, b_off[g], lb + g * 1024);
-#pragma unroll
-        for (int r = 0; r < kReads; ++r)
-          if (r * kReadSpan / kReads == slot) read_half(af0, bf0, 0, r);
-        __builtin_amdgcn_sched_barrier(0);
-      }
-    }
-  };
-  for (int kt = 0; kt < nk; ++kt) {
+  // Reads under the MFMAs, in the order they are needed.  First half: the FN reads of B
+  // fragments HN .. FN-1, under the first three quarters.  Second half: B fragment 0 and
+  // the A fragments of the next trip's first row first, then the other B fragments; the
+  // last read is issued an eighth of a half before its end.
+  constexpr int kReads1 = 2 * HN, kSpan1 = kHalf * 3 / 4;
+  constexpr int kReads2 = 2 * (FM + HN), kSpan2 = kHalf * 7 / 8;
+  auto trip = [&](auto parity, int kt) __attribute__((always_inline)) {
+    constexpr int P = decltype(parity)::value;
     const int ka = kt + 2 < nk ? kt + 2 : nk - 1;
     const uint8_t* ak = a_base + (int64_t)ka * kRowBytes;
+    // four slots on from A slab kt = one slot back = where B slab kt-1 was
     const uint32_t a_dst = a_at >= kSlot ? a_at - kSlot : a_at + (kRingSlots - 1) * kSlot;
-    first_step(ak, lds0 + a_dst + wave * (GA * 1024));
+    const uint32_t la = lds0 + a_dst + wave * (GA * 1024);
+#pragma unroll
+    for (int ni = 0; ni < HN; ++ni) {
+#pragma unroll
+      for (int mi = 0; mi < FM; ++mi) {
+        const int slot = ni * FM + mi;
+        mfma_fp8(acc[ni][mi], bf[ni], af[P][mi]);
+#pragma unroll
+        for (int r = 0; r < kReads1; ++r)
+          if (r * kSpan1 / kReads1 == slot) read_half(bf[HN + (r >> 1)], b_fr, HN + (r >> 1), r & 1);
+#pragma unroll
+        for (int g = 0; g < GA; ++g)
+          if (g * kHalf / GA == slot) load_group(ak, a_off[g], la + g * 1024);
+        __builtin_amdgcn_sched_barrier(0);     // keep this interleaving
+      }
+    }
+    // Wait for this wave's own loads of B slab kt+1 (and everything older) before the
+    // barrier; the GA loads of A slab kt+2, issued last, may stay in flight.
     static_assert(GA == 8 || GA == 4, "explicit vmcnt below");
     if constexpr (GA == 8) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
     else asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
-    __syncthreads();
-    second_step(kt);
+    __syncthreads();     // slab pair kt fully read by everyone; pair kt+1 has landed
+
+    const int kb = kt + 2 < nk ? kt + 2 : nk - 1;
+    const uint8_t* bk = b_base + (int64_t)kb * kRowBytes;
+    const uint32_t lb = lds0 + a_at + wave * (GB * 1024);
+    // the next slab pair sits two slots further round the ring
+    const uint32_t a_to = a_at + 2 * kSlot < kRingSlots * kSlot ? a_at + 2 * kSlot : a_at + 2 * kSlot - kRingSlots * kSlot;
+    const uint32_t b_to = b_at + 2 * kSlot < kRingSlots * kSlot ? b_at + 2 * kSlot : b_at + 2 * kSlot - kRingSlots * kSlot;
+#pragma unroll
+    for (int q = 0; q < 2; ++q) {
+      a_fr[q] += a_to - a_at;
+      b_fr[q] += b_to - b_at;
+    }
+    a_at = a_to;
+    b_at = b_to;
+#pragma unroll
+    for (int ni = 0; ni < HN; ++ni) {
+#pragma unroll
+      for (int mi = 0; mi < FM; ++mi) {
+        const int slot = ni * FM + mi;
+        mfma_fp8(acc[HN + ni][mi], bf[HN + ni], af[P][mi]);
+#pragma unroll
+        for (int g = 0; g < GB; ++g)
+          if (g * (kHalf / 2) / GB == slot) load_group(bk, b_off[g], lb + g * 1024);
+#pragma unroll
+        for (int r = 0; r < kReads2; ++r)
+          if (r * kSpan2 / kReads2 == slot) {
+            // order: B fragment 0, all A fragments, B fragments 1 .. HN-1
+            if (r < 2) read_half(bf[0], b_fr, 0, r & 1);
+            else if (r < 2 + 2 * FM) read_half(af[1 - P][(r - 2) >> 1], a_fr, (r - 2) >> 1, r & 1);
+            else read_half(bf[(r - 2 * FM) >> 1], b_fr, (r - 2 * FM) >> 1, r & 1);
+          }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+  };
+  // Two trips per turn of the loop, one for each set of A fragments; an odd last trip
+  // stands behind the loop (an exit in the middle of the loop would leave the compiler with
+  // two places the accumulators can come from, and it then keeps two copies of them).
+  int kt = 0;
+  for (; kt + 1 < nk; kt += 2) {
+    trip(Parity<0>{}, kt);
+    trip(Parity<1>{}, kt + 1);
   }
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  if (kt < nk) trip(Parity<0>{}, kt);
+  // The repeated loads of the last K steps must not land on top of the next tile's first
+  // slabs, and the last MFMAs (assembly the compiler does not time) must be through before
+  // their results are read.
+  asm volatile("s_waitcnt vmcnt(0)\n\ts_nop 15\n\ts_nop 15" ::: "memory");
   __syncthreads();
   if (tr != nullptr) tr[2] = wall_clock64();
   between();
 
-  // Epilogue.  D[n][m]: a lane holds row m = lane & 31 of a 32x32 fragment and, per
-  // group g of 4 registers, the 4 consecutive columns g*8 + (lane >> 5)*4 .. +3: one
-  // 32-bit word of e4m3fn.  32 rows at a time go through the wave's quarter of ring
-  // slot 4 (WN bytes per row, chunk c of row r at position c ^ (r >> 1), modulo the
-  // chunks of a row) and leave as whole rows, 16 bytes per lane.
+  // Epilogue.  D[n][m]: a lane holds row m = lane & 15 of a 16x16 fragment and the 4
+  // consecutive columns (lane >> 4)*4 .. +3: one 32-bit word of e4m3fn.  32 rows at a
+  // time go through the wave's quarter of ring slot 4 (WN bytes per row, chunk c of row
+  // r at position c ^ (r >> 1), modulo the chunks of a row) and leave as whole rows, 16
+  // bytes per lane.
   constexpr int kChunks = WN / 16;                // 16-byte chunks per wave-tile row
   constexpr int kRowsPerStore = 64 / kChunks;
   const uint32_t turn = lds0 + (kRingSlots - 1) * kSlot + wave * (32 * WN);
-  const int half = ln >> 5, wr_row = ln & 31;
   const int rd_row = ln / kChunks, rd_chunk = ln % kChunks;
 #pragma unroll
-  for (int mi = 0; mi < FM; ++mi) {
+  for (int band = 0; band < FM / 2; ++band) {
 #pragma unroll
-    for (int ni = 0; ni < FN; ++ni) {
+    for (int sub = 0; sub < 2; ++sub) {
+      const int wr_row = sub * 16 + (ln & 15);
 #pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        const f32x16& d = acc[ni][mi];
-        const uint32_t w = pack_fp8x4(d[g * 4 + 0], d[g * 4 + 1], d[g * 4 + 2], d[g * 4 + 3]);
-        const int chunk = ni * 2 + (g >> 1);
-        const uint32_t addr = turn + wr_row * WN + (((chunk ^ (wr_row >> 1)) & (kChunks - 1)) << 4) +
-                              ((g & 1) * 2 + half) * 4;
+      for (int ni = 0; ni < FN; ++ni) {
+        const f32x4 d = acc[ni][band * 2 + sub];
+        const uint32_t w = pack_fp8x4(d[0], d[1], d[2], d[3]);
+        const uint32_t addr = turn + wr_row * WN + (((ni ^ (wr_row >> 1)) & (kChunks - 1)) << 4) + (ln >> 4) * 4;
         *reinterpret_cast<__attribute__((address_space(3))) uint32_t*>((uintptr_t)addr) = w;
       }
     }
@@ -699,7 +738,7 @@ __device__ __forceinline__ void run_tile_fp8(const TileContext& cx, const TileRe
     for (int i = 0; i < 32 / kRowsPerStore; ++i) {
       const int r = i * kRowsPerStore + rd_row;
       const u32x4 v = lds_read_b128(turn + r * WN + (((rd_chunk ^ (r >> 1)) & (kChunks - 1)) << 4));
-      const int m = tile.row0 + wm * WM + mi * 32 + r;
+      const int m = tile.row0 + wm * WM + band * 32 + r;
       const int n = tile.col0 + wn * WN + rd_chunk * 16;
       if (n < s.N) *reinterpret_cast<u32x4*>(c + (int64_t)m * s.N + n) = v;
     }
@@ -784,8 +823,11 @@ __device__ __forceinline__ void copy_pieces(const CopyJob& job, int c, uint32_t 
 #pragma unroll
     for (int u = 0; u < kPullInFlight; ++u) {
       const int64_t i = i0 + u * kGemmThreads;
+      // (the idle slots: the hardware reads a 128-bit store's data for two cycles after issue, a
+      // vector instruction that writes one of these registers right behind the store changes what
+      // is stored, and the compiler, which spaces its own stores, does not look into assembly)
       if (i < job.chunk_vecs)
-        asm volatile("global_store_dwordx4 %0, %1, off sc1" : : "v"(dst + i), "v"(v[u]) : "memory");
+        asm volatile("global_store_dwordx4 %0, %1, off sc1\n\ts_nop 1" : : "v"(dst + i), "v"(v[u]) : "memory");
     }
   };
   uint32_t mine = 0;

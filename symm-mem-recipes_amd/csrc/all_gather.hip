@@ -36,9 +36,12 @@ static std::atomic<uint32_t> g_gather_pacing{1024u << 16};
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef __attribute__((address_space(1))) u32x4 GlobalVec;
 
-// 128-bit store at agent scope: written through the XCD's L2.
+// 128-bit store at agent scope: written through the XCD's L2.  The idle slots behind it: the
+// hardware reads a 128-bit store's data for two cycles after issue, and a vector instruction
+// that writes one of the data registers in that time changes what is stored; the compiler
+// spaces its own stores but does not look into assembly.
 __device__ __forceinline__ void store_through(GlobalVec* p, u32x4 v) {
-  asm volatile("global_store_dwordx4 %0, %1, off sc1" : : "v"(p), "v"(v) : "memory");
+  asm volatile("global_store_dwordx4 %0, %1, off sc1\n\ts_nop 1" : : "v"(p), "v"(v) : "memory");
 }
 
 __global__ __launch_bounds__(kGatherThreads) void all_gather_kernel(

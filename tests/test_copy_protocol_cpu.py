@@ -19,7 +19,7 @@ STAND_INS = [
     ("typedef __attribute__((address_space(1))) u32x4 GlobalVec;", "typedef u32x4 GlobalVec;"),
     ("typedef __attribute__((address_space(3))) uint32_t LdsWord;", "typedef uint32_t LdsWord;"),
     ("reinterpret_cast<LdsWord*>((uintptr_t)lds0)", "lds_ptr(lds0)"),
-    ('asm volatile("global_store_dwordx4 %0, %1, off sc1" : : "v"(dst + i), "v"(v[u]) : "memory");',
+    ('asm volatile("global_store_dwordx4 %0, %1, off sc1\\n\\ts_nop 1" : : "v"(dst + i), "v"(v[u]) : "memory");',
      "store_checked(dst + i, v[u]);"),
     ("__builtin_nontemporal_load(src + (i < job.chunk_vecs ? i : job.chunk_vecs - 1))",
      "load_checked(src + (i < job.chunk_vecs ? i : job.chunk_vecs - 1))"),
