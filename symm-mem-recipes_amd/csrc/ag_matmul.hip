@@ -1098,7 +1098,7 @@ constexpr int kMaxProducerWgs = 128;
 constexpr double kCopyOnlyBytesPerUs = 25.0e3, kWaiterBytesPerUs = 12.0e3, kWaitShows = 0.6, kFusedFixedUs = 18.0;
 static double model_tile_us(int BM, int BN, int K, int elem_bytes, bool beside_copy) {
   double rate = BM == 256 && BN == 256 ? (beside_copy ? 6.5e6 : 6.6e6) : 4.6e6;      // FLOP per us
-  if (elem_bytes == 1) rate *= 2.0;
+  if (elem_bytes == 1) rate = BM == 256 && BN == 256 ? (beside_copy ? 14.2e6 : 14.0e6) : 9.2e6;
   return 2.0 * BM * BN * K / rate + 6.0;
 }
 static FusedEstimate estimate_fused(const GemmSchedule& s, int cus, int grid, int elem_bytes = 2) {
