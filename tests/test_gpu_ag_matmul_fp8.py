@@ -71,6 +71,9 @@ def _release():
     (2048, 128, 1024, 8, 6),      # 128x128 tiles, eight K slabs
     (4096, 1280, 256, 8, 4),      # 256x128 tiles
     (8192, 1280, 128, 8, 1),      # 256x256 tiles, many of them
+    (8192, 1280, 384, 8, 2),      # 256x256 tiles, three K slabs: the odd trip behind the K loop
+    (4096, 1280, 640, 8, 7),      # 256x128 tiles, five K slabs
+    (2048, 128, 896, 8, 3),       # 128x128 tiles, seven K slabs
 ])
 def test_fp8_fused_parity(cuda, either_form, M, N, K, ws, rank):
     from symm_mem_recipes import all_gather_matmul_tma_persistent
@@ -192,3 +195,26 @@ def test_fp8_full_size_linearity(cuda):
     # every entry is off by at most half an e4m3fn ulp (2^-4 relative); random walk over N entries
     tol = 8 * (N ** 0.5) * 2.0 ** -4 * float(c.pow(2).mean().sqrt()) + 1e-3
     assert torch.all((c.sum(dim=1) - rowsum).abs() <= tol)
+
+
+@pytest.mark.parametrize("M,N,K", [(16384, 1792, 4096), (8192, 3584, 8192)])
+def test_fp8_fused_launch_at_full_size_gathers_every_row(cuda, M, N, K):
+    """The fused launch at sizes where its workgroups copy between two tiles with every register
+    taken: the gathered operand equals the shards and the product equals the ungated launch's
+    bit for bit.  (A register the compiler reloaded right behind one of the copy's assembly
+    stores once changed what was stored: one row in sixteen of the last chunks, at the first of
+    these shapes only.)"""
+    from symm_mem_recipes import all_gather_matmul_tma_persistent
+    ws = 8
+    a_shard, h, shards, b, b_bits, a_out, c_out = _setup(M, N, K, ws, 0, cuda)
+    want_a = np.concatenate(shards)
+    for _ in range(3):
+        a_out.view(torch.uint8).fill_(0x11)
+        all_gather_matmul_tma_persistent(a_shard, b, a_out, c_out, None, fused=True)
+        h.check_status()
+        assert np.array_equal(_bits(a_out), want_a)
+        fused_bits = _bits(c_out)
+        c_out.view(torch.uint8).fill_(0x7F)
+        all_gather_matmul_tma_persistent(a_shard, b, a_out, c_out, None, mm_only=True)
+        h.check_status()
+        assert np.array_equal(fused_bits, _bits(c_out))
