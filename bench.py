@@ -36,9 +36,9 @@ MFMA_FP8_PEAK_TFLOPS = 5000.0   # MI355X dense fp8, published
 # the 256 MiB last-level cache serves part of it, so it is not HBM traffic.  "mfma_busy" is
 # SQ_VALU_MFMA_BUSY_CYCLES per SIMD over the launch's elapsed shader cycles (GRBM_GUI_ACTIVE).
 MEASURED_GEMM_COUNTERS = {
-    "fused": {"traffic": 2255402900, "mfma_busy": 0.702},
-    "ungated": {"traffic": 1616701600, "mfma_busy": 0.733},
-    "hipblaslt": {"traffic": 1595657300, "mfma_busy": 0.774},
+    "fused": {"traffic": 2255402900, "mfma_busy": 0.737},
+    "ungated": {"traffic": 1616701600, "mfma_busy": 0.756},
+    "hipblaslt": {"traffic": 1595657300, "mfma_busy": 0.790},
 }
 MEASURED_GEMM_FP8_TRAFFIC_BYTES = 799597261   # ungated e4m3fn launch, the same two counter runs with --fp8
 WS = 8
