@@ -552,12 +552,22 @@ __device__ __forceinline__ void run_tile(const TileContext& cx, const TileRef& t
 //                B fragments 0 .. FN/2-1 are read from pair kt+1; loads of B slab kt+2
 typedef int i32x8 __attribute__((ext_vector_type(8)));
 
+// Four fp32 values to e4m3fn, round to nearest even, finite values beyond the range to the
+// largest finite one (+-448), NaN kept: cvt.rn.satfinite.  The conversion instruction does all
+// of that by itself once the wave's overflow mode bit is set (set_fp8_saturation, at kernel
+// entry); without the bit a finite value beyond 464 becomes NaN, and clamping by hand with NaN
+// passed through was nine vector instructions per pair instead of one - 2 us of a tile's epilogue.
+// (An infinite input would still give NaN; an fp32 sum of products of e4m3fn values cannot get
+// there: 448 * 448 * K stays finite for any K an int can hold.)
 __device__ __forceinline__ uint32_t pack_fp8x4(float a, float b, float c, float d) {
-  // saturate to the largest finite e4m3fn value, keep NaN (cvt.rn.satfinite semantics)
-  auto sat = [](float x) { return x != x ? x : __builtin_fminf(__builtin_fmaxf(x, -448.0f), 448.0f); };
-  int w = __builtin_amdgcn_cvt_pk_fp8_f32(sat(a), sat(b), 0, false);
-  w = __builtin_amdgcn_cvt_pk_fp8_f32(sat(c), sat(d), w, true);
+  int w = __builtin_amdgcn_cvt_pk_fp8_f32(a, b, 0, false);
+  w = __builtin_amdgcn_cvt_pk_fp8_f32(c, d, w, true);
   return (uint32_t)w;
+}
+// MODE.FP16_OVFL (bit 23 of hardware register 1) = 1 for the rest of the wave's life.  Nothing
+// else in this kernel converts to a 16-bit or 8-bit float type.
+__device__ __forceinline__ void set_fp8_saturation() {
+  __builtin_amdgcn_s_setreg((0 << 11) | (23 << 6) | 1, 1);
 }
 
 // D += A x B on a 16x16x128 e4m3fn fragment pair; the accumulator named as an accumulation
@@ -942,6 +952,7 @@ __global__ __launch_bounds__(kGemmThreads, 1) void ag_matmul_kernel(
     return;
   }
 
+  if constexpr (FP8) set_fp8_saturation();
   TileContext cx;
   cx.lane = threadIdx.x & 63;
   cx.wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
