@@ -152,6 +152,8 @@ def test_fp8_saturation_and_exact_small_integers(cuda, either_form):
     b_bits = rng.choice(vals, size=(N, K)).astype(np.uint8)
     b = _t(b_bits).to(cuda)
     shards[0][0, :] = vals[-1]                     # 4 * 4 * 256 = 4096 -> saturates to 448
+    shards[0][1, :] = vals[0]                      # -4 * 4 * 256 -> saturates to -448
+    shards[0][2, 5] = 0x7F                         # one NaN in a row of A: the whole row of C is NaN
     b_bits[0, :] = vals[-1]
     h.get_buffer(0, (M // ws, K), torch.uint8).copy_(torch.from_numpy(shards[0]))
     b = _t(b_bits).to(cuda)
@@ -160,7 +162,10 @@ def test_fp8_saturation_and_exact_small_integers(cuda, either_form):
     want = O.ag_matmul_ref_fp8(shards, b_bits)
     got = _bits(c_out)
     assert got[0, 0] == 126 and want[0, 0] == 126
-    assert np.array_equal(got, want)
+    assert got[1, 0] == 254 and want[1, 0] == 254
+    assert np.all((got[2] & 0x7F) == 0x7F) and np.all((want[2] & 0x7F) == 0x7F)
+    keep = np.arange(M) != 2                       # (a NaN's sign is not part of the contract)
+    assert np.array_equal(got[keep], want[keep])
 
 
 def test_fp8_mm_only_and_validation(cuda):
