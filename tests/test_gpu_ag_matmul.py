@@ -494,6 +494,31 @@ def test_full_size_config5(cuda):
     assert torch.all((got - rowsum).abs() <= tol), float((got - rowsum).abs().max())
 
 
+@pytest.mark.parametrize("M,N,K", [(16384, 1792, 4096), (8192, 3584, 8192), (32768, 1792, 2048)])
+def test_fused_launch_at_full_size_gathers_every_row(cuda, M, N, K):
+    """The fused launch at sizes where its workgroups copy between two tiles with every register
+    taken: the gathered operand equals the shards and the product equals that of the
+    copy-then-multiply form bit for bit.  (In the e4m3fn kernel a register the compiler reloaded
+    right behind one of the copy's assembly stores once changed what was stored, at the first of
+    these shapes only.)"""
+    from symm_mem_recipes import all_gather_matmul_tma_persistent
+    ws = 8
+    a_shard, h, shards, b, b_bits, a_out, c_out = _setup(M, N, K, ws, 3, cuda)
+    want_a = np.concatenate(shards)
+    for _ in range(3):
+        a_out.fill_(float("nan"))
+        all_gather_matmul_tma_persistent(a_shard, b, a_out, c_out, None, fused=True)
+        h.check_status()
+        assert np.array_equal(_t_bits(a_out), want_a)
+        fused_bits = _t_bits(c_out)
+        c_out.fill_(float("nan"))
+        a_out.fill_(float("nan"))
+        all_gather_matmul_tma_persistent(a_shard, b, a_out, c_out, None, fused=False)
+        h.check_status()
+        assert np.array_equal(_t_bits(a_out), want_a)
+        assert np.array_equal(fused_bits, _t_bits(c_out))
+
+
 def test_golden_vectors(cuda):
     """tests/golden/ag_matmul.npz: 4 shards of [128, 64], B [72, 64]."""
     import os
