@@ -167,3 +167,51 @@ def test_schedule_rejects_bad_shapes():
         gemm_schedule(1024, 252, 256, 0, 8, 128)        # N not a multiple of 8
     with pytest.raises(AssertionError):
         gemm_schedule(1024, 256, 256, 8, 8, 128)        # rank out of range
+
+
+def _row_swizzle_from_source():
+    """The kernel's row_swizzle, taken from the source text (the expression is valid Python)."""
+    import os
+    import re
+    src = open(os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))),
+                            "symm-mem-recipes_amd", "csrc", "ag_matmul.hip")).read()
+    m = re.search(r"inline int row_swizzle\(int r\) \{\s*return (.*?);\s*\}", src, re.S)
+    assert m, "row_swizzle not found"
+    expr = m.group(1)
+    return lambda r: eval(expr, {"r": r})
+
+
+def _lds_columns(accesses):
+    """16-byte columns of the 256-byte bank row that a set of (row, position) accesses to a slab
+    touches: a slab row is 128 bytes, so even rows lie in columns 0-7 and odd rows in 8-15."""
+    return [(row & 1) * 8 + pos for row, pos in accesses]
+
+
+def test_fragment_reads_are_free_of_bank_conflicts():
+    """A 128-bit LDS read is served 16 lanes at a time (lanes 8g..8g+7 with 32+8g..32+8g+7), and
+    those 16 must fall into 16 different 16-byte columns.  Checked for the bf16 fragments
+    (lane l: row l & 15, chunk 4 * kk + (l >> 4)), the e4m3fn fragments (row l & 15, chunks
+    2 * (l >> 4) + q) and for every 16-row fragment of a slab, with the swizzle the kernel uses."""
+    sw = _row_swizzle_from_source()
+    groups = [[8 * g + i for i in range(8)] + [32 + 8 * g + i for i in range(8)] for g in range(4)]
+    for frag_row0 in range(0, 256, 16):
+        for lanes in groups:
+            for kk in range(2):                    # bf16: K step kk of a slab
+                acc = [(frag_row0 + (l & 15), (4 * kk + (l >> 4)) ^ sw((frag_row0 + (l & 15)) & 15)) for l in lanes]
+                assert len(set(_lds_columns(acc))) == 16, ("bf16", frag_row0, lanes, kk)
+            for q in range(2):                     # e4m3fn: first and second half of the lane's 32 bytes
+                acc = [(frag_row0 + (l & 15), (2 * (l >> 4) + q) ^ sw((frag_row0 + (l & 15)) & 15)) for l in lanes]
+                assert len(set(_lds_columns(acc))) == 16, ("e4m3fn", frag_row0, lanes, q)
+
+
+def test_tile_loads_fill_every_chunk_of_a_slab_once():
+    """A direct-to-LDS load lands lane l of load group q at byte q * 1024 + l * 16, i.e. row
+    q * 8 + (l >> 3), position l & 7; the lane fetches chunk (l & 7) ^ swizzle(l >> 3) ^ ((q & 1) << 2)
+    of that row.  Position p of row r must hold chunk p ^ row_swizzle(r): every chunk of every row
+    exactly once."""
+    sw = _row_swizzle_from_source()
+    for q in range(32):
+        for l in range(64):
+            row, pos = q * 8 + (l >> 3), l & 7
+            chunk = ((l & 7) ^ sw(l >> 3)) ^ ((q & 1) << 2)
+            assert chunk == pos ^ sw(row & 15), (q, l)
