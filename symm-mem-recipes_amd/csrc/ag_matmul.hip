@@ -28,7 +28,7 @@
 //     same grid only copy, and a GEMM workgroup that finds its tile's chunk missing copies
 //     along instead of spinning;
 //   * the same kernel in e4m3fn (run_tile_fp8): the bytes move the same way, the
-//     tile is built from v_mfma_f32_32x32x64_f8f6f4.
+//     tile is built from v_mfma_f32_16x16x128_f8f6f4.
 #include <atomic>
 #include <type_traits>
 
