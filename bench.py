@@ -24,24 +24,25 @@ for _p in (ROOT, os.path.join(ROOT, "symm-mem-recipes_amd")):
         sys.path.insert(0, _p)
 
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
-# Memory bytes per launch of the reduce kernel from rocprofv3 FETCH_SIZE / WRITE_SIZE,
-# each scaled by what the counter reads for this script's 512 MiB calibration copy
-# (profiles/one_shot_all_reduce_64MiB_bf16_traffic.md); keyed by MiB per buffer.
-MEASURED_REDUCE_TRAFFIC_BYTES = {64: 604043000}
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
 MFMA_FP8_PEAK_TFLOPS = 5000.0   # MI355X dense fp8, published
-# Counter figures of the GEMM at M=16384 N=3584 K=8192 from `bench.py --gemm-only` under
-# rocprofv3 --pmc (profiles/ag_matmul_M16384_N3584_K8192_counters.md).  "traffic" is what
-# passes between the XCDs' L2s and the fabric (FETCH_SIZE scaled as above plus WRITE_SIZE):
-# the 256 MiB last-level cache serves part of it, so it is not HBM traffic.  "mfma_busy" is
-# SQ_VALU_MFMA_BUSY_CYCLES per SIMD over the launch's elapsed shader cycles (GRBM_GUI_ACTIVE).
-MEASURED_GEMM_COUNTERS = {
-    "fused": {"traffic": 2255402900, "mfma_busy": 0.737},
-    "ungated": {"traffic": 1616701600, "mfma_busy": 0.756},
-    "hipblaslt": {"traffic": 1595657300, "mfma_busy": 0.790},
-}
-MEASURED_GEMM_FP8_TRAFFIC_BYTES = 799597261   # ungated e4m3fn launch, the same two counter runs with --fp8
 WS = 8
+
+
+def _counters():
+    """Hardware-counter figures that a timing run cannot take itself, from the file written next
+    to the rocprofv3 summaries they come from (profiles/counters.json; every entry names its
+    summary).  reduce_traffic_bytes: memory bytes per launch of the reduce kernel (FETCH_SIZE /
+    WRITE_SIZE, each scaled by what the counter reads for this script's 512 MiB calibration
+    copy), keyed by MiB per buffer.  gemm / gemm_fp8: per launch at M=16384 N=3584 K=8192,
+    "traffic" = bytes between the XCDs' L2s and the fabric (the 256 MiB last-level cache serves
+    part of it, so it is not HBM traffic), "mfma_busy" = SQ_VALU_MFMA_BUSY_CYCLES per SIMD over
+    the launch's elapsed shader cycles.  A missing file or entry gives null in the output."""
+    try:
+        with open(os.path.join(ROOT, "profiles", "counters.json")) as f:
+            return json.load(f)
+    except (OSError, ValueError):
+        return {}
 
 
 def _median(xs):
@@ -99,26 +100,27 @@ def bench_reduce(size_mib, steps, warmup, dev):
     for r in range(WS):
         g.manual_seed(r)
         h.get_buffer(r, (numel,), torch.bfloat16).normal_(generator=g)
+    # The headline is the reference's call as the drop-in ships it: the blockwise barrier, then
+    # the reduce (triton_one_shot_all_reduce.py:70-93).
     out = None
     for _ in range(warmup):
-        out = one_shot_all_reduce(t, barrier=False)
+        out = one_shot_all_reduce(t)
     torch.cuda.synchronize()
     e0 = torch.cuda.Event(enable_timing=True)
     e1 = torch.cuda.Event(enable_timing=True)
     t0 = time.perf_counter()
     e0.record()
     for _ in range(steps):
-        out = one_shot_all_reduce(t, barrier=False)
+        out = one_shot_all_reduce(t)
     e1.record()
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
     h.check_status()
     dev_us = e0.elapsed_time(e1) * 1e3 / steps
     alg_bytes = (WS + 1) * nbytes
-    # the same call behind the blockwise barrier, and the write-back-to-all variant
-    # (the reference's call, triton_one_shot_all_reduce.py:70: timed the way the headline is,
-    # back-to-back launches between one event pair)
-    us_barrier = _time_batched(lambda: one_shot_all_reduce(t, barrier=True), max(steps // 2, 10), 3)
+    # the same reduce without the handshake (peers' data already stream-ordered), timed the way
+    # the headline is (back-to-back launches between one event pair), and the write-back-to-all variant
+    us_no_barrier = _time_batched(lambda: one_shot_all_reduce(t, barrier=False), max(steps // 2, 10), 3)
     us_write_all = _time_events(lambda: one_shot_all_reduce(t, barrier=False, write_all=True), 20, 3)
     # two-shot: every emulated rank reduces its eighth and writes it to all peers, two handshakes
     for r in range(WS):
@@ -128,7 +130,7 @@ def bench_reduce(size_mib, steps, warmup, dev):
     h.check_status()
     SM.release()
     del out
-    return dict(wall_s=wall, dev_us=dev_us, alg_bytes=alg_bytes, us_barrier=us_barrier,
+    return dict(wall_s=wall, dev_us=dev_us, alg_bytes=alg_bytes, us_no_barrier=us_no_barrier,
                 us_write_all=us_write_all, write_all_bytes=2 * WS * nbytes, us_two_shot=us_two_shot)
 
 
@@ -223,7 +225,7 @@ def bench_mfma_only(dev):
     the GEMM's MFMA share can be compared with."""
     import torch
     from symm_mem_recipes import _lib
-    lib = _lib.load()
+    lib = _lib.load_probe()
     cus = torch.cuda.get_device_properties(dev).multi_processor_count
     vals = torch.empty(1 << 16, dtype=torch.bfloat16, device=dev).normal_(0, 0.02)
     ticks = torch.zeros(2 * cus, dtype=torch.int64, device=dev)
@@ -243,6 +245,7 @@ def bench_mfma_only(dev):
 
 def bench_ag_matmul(dev, gated=True):
     import torch
+    counters = _counters().get("gemm", {})
     from symm_mem_recipes import EmulatedSymmetricMemory as SM, all_gather_matmul_tma_persistent
     M, N, K = 16384, 3584, 8192
     a_shard = SM.empty_strided_p2p((M // WS, K), (K, 1), torch.bfloat16, dev, world_size=WS, rank=0)
@@ -271,10 +274,11 @@ def bench_ag_matmul(dev, gated=True):
                 gating_overhead=us_gated / us_ungated - 1.0,
                 roofline={"bound": "mfma", "achieved": flops / us_gated / 1e6, "peak": MFMA_BF16_PEAK_TFLOPS,
                           "unit": "TFLOP/s", "frac": flops / us_gated / 1e6 / MFMA_BF16_PEAK_TFLOPS,
-                          "traffic": MEASURED_GEMM_COUNTERS["fused"]["traffic"],
+                          "traffic": counters.get("fused", {}).get("traffic"),
                           "traffic_kind": "L2 <-> fabric bytes per launch (last-level cache or HBM behind it)",
-                          "mfma_busy": MEASURED_GEMM_COUNTERS["fused"]["mfma_busy"]},
-                counters_ungated=MEASURED_GEMM_COUNTERS["ungated"], counters_hipblaslt=MEASURED_GEMM_COUNTERS["hipblaslt"],
+                          "mfma_busy": counters.get("fused", {}).get("mfma_busy")},
+                counters_ungated=counters.get("ungated"), counters_hipblaslt=counters.get("hipblaslt"),
+                counters_source=counters.get("source"),
                 torch_matmul_us=us_lib, torch_matmul_tflops=flops / us_lib / 1e6)
 
 
@@ -309,7 +313,7 @@ def bench_ag_matmul_fp8(dev, gated=True):
                gating_overhead=us_gated / us_ungated - 1.0,
                roofline={"bound": "mfma", "achieved": flops / us_gated / 1e6, "peak": MFMA_FP8_PEAK_TFLOPS,
                          "unit": "TFLOP/s", "frac": flops / us_gated / 1e6 / MFMA_FP8_PEAK_TFLOPS,
-                         "traffic": MEASURED_GEMM_FP8_TRAFFIC_BYTES})
+                         "traffic": _counters().get("gemm_fp8", {}).get("ungated", {}).get("traffic")})
     try:                                            # the library's fp8 GEMM of the same operands (bf16 result)
         one = torch.ones((), device=dev)
         us_lib = _time_events(lambda: torch._scaled_mm(a_out, b.T, scale_a=one, scale_b=one,
@@ -510,7 +514,8 @@ def main():
     value = r["alg_bytes"] * args.steps / r["wall_s"] / 1e9
     achieved = r["alg_bytes"] / r["dev_us"] / 1e3
     line = {
-        "metric": "one-shot all-reduce GB/s, 8 x bf16 peer buffers (algorithmic bytes 9*S per call)",
+        "metric": "one-shot all-reduce GB/s, 8 x bf16 peer buffers (algorithmic bytes 9*S per call), "
+                  "behind the blockwise barrier as the reference calls it",
         "value": value,
         "unit": "GB/s",
         "n_gpus": 1,
@@ -523,16 +528,17 @@ def main():
         "dtype": "bf16",
         "data": "synthetic",
         "config": {"workload": f"one-shot all-reduce, 8 emulated peer buffers of {args.size_mib} MiB bf16 "
-                               "N(0,1) seeded per rank, resident in HBM, single output, fp32 accumulation "
-                               "in rank order", "world_size": WS, "bytes_per_buffer": args.size_mib << 20},
+                               "N(0,1) seeded per rank, resident in HBM, blockwise barrier then single output, "
+                               "fp32 accumulation in rank order", "world_size": WS,
+                    "bytes_per_buffer": args.size_mib << 20},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBS,
-                     "traffic": MEASURED_REDUCE_TRAFFIC_BYTES.get(args.size_mib)},
+                     "traffic": _counters().get("reduce_traffic_bytes", {}).get(str(args.size_mib))},
     }
     extra = {
         "reduce_kernel_us": r["dev_us"],
-        "reduce_behind_barrier_us": r["us_barrier"],
-        "reduce_behind_barrier_frac": r["alg_bytes"] / r["us_barrier"] / 1e3 / HBM_PEAK_GBS,
+        "reduce_without_barrier_us": r["us_no_barrier"],
+        "reduce_without_barrier_frac": r["alg_bytes"] / r["us_no_barrier"] / 1e3 / HBM_PEAK_GBS,
         "reduce_write_all_us": r["us_write_all"],
         "reduce_write_all_gbs": r["write_all_bytes"] / r["us_write_all"] / 1e3,
         "reduce_two_shot_us": r["us_two_shot"],
@@ -547,7 +553,8 @@ def main():
             [bench_reduce_rotating(k, dev, "fp32") for k in (1024, 8192, 16384)] +
             [bench_reduce_rotating(k, dev, "bf16", write_all=True) for k in (1024, 8192, 16384)] +
             [bench_reduce_rotating(k, dev, "bf16", accumulate="bf16") for k in (8192,)] +
-            [bench_reduce_rotating(k, dev, "bf16", barrier=True) for k in (8192, 16384)])
+            [bench_reduce_rotating(k, dev, "bf16", barrier=True) for k in (16, 1024, 8192, 16384, 32768)] +
+            [bench_reduce_rotating(k, dev, "fp32", barrier=True) for k in (8192, 16384)])
         extra["all_gather_matmul"] = bench_ag_matmul(dev)
         extra["all_gather_matmul"]["mfma_only"] = bench_mfma_only(dev)
         extra["all_gather_matmul_fp8"] = bench_ag_matmul_fp8(dev)

@@ -22,6 +22,10 @@
  *     per rank), exactly what the reference hands to its kernels
  *     (symm_mem_recipes/triton_one_shot_all_reduce.py:115-116,
  *     symm_mem_recipes/triton_barrier.py:167).
+ *
+ * The device functions of the flag protocol (blockwise_barrier, send_signal, wait_signal,
+ * wait_signal_reset), which the reference's kernels import from one another, are in
+ * smr_device.h for HIP kernels of other libraries; this header is the host side.
  */
 #ifndef SMR_H_
 #define SMR_H_
@@ -32,7 +36,7 @@
 extern "C" {
 #endif
 
-#define SMR_VERSION 100
+#define SMR_VERSION 110
 
 #define SMR_DTYPE_BF16 0
 #define SMR_DTYPE_FP32 1
@@ -185,12 +189,6 @@ int smr_all_gather_at_once(const uint64_t* buffer_ptrs_dev, void* a_out_dev,
                            int world_size, int64_t shard_bytes, int splits_per_rank,
                            int num_workgroups, void* stream);
 
-/* Pacing of the producer: the first `fast_chunks` chunks are copied by all
- * workgroups, the remaining ones by `slow_workgroups` of them (0 = all, i.e. no
- * pacing).  Default 0 and 0.  No reference counterpart (copy engines pace
- * themselves by link speed). */
-int smr_set_gather_pacing(int fast_chunks, int slow_workgroups);
-
 /* Flag-gated bf16 GEMM.  Replaces matmul_kernel_tma_persistent and its launch
  * (symm_mem_recipes/triton_all_gather_matmul.py:98-193, :287-315).
  *   C[M,N] = A[M,K] * B[N,K]^T, fp32 accumulate, bf16 output, all row-major.
@@ -216,16 +214,12 @@ int smr_ag_matmul_schedule(int M, int N, int K, int rank, int world_size, int co
  * fresh flags, producer on a second stream, persistent GEMM, stream join).  The reference's
  * producer is a copy engine and costs no SMs; on one GPU the copy runs on compute units, and
  * here it runs inside the GEMM's own grid:
- *   - `producer_workgroups` extra workgroups (0 = the plan's, see smr_ag_matmul_plan) only
- *     copy: the peers' shards from buffer_ptrs_dev into a_out in the reference's order
+ *   - `producer_workgroups` extra workgroups (0 = the plan's, see smr_ag_matmul_plan; never
+ *     fewer than one: the local shard reaches a_out through them) only copy: the peers' shards from buffer_ptrs_dev into a_out in the reference's order
  *     (sources rank+1, ..., rank+ws-1, rank; :43-44), in 64 KiB pieces taken by ticket;
  *   - a GEMM workgroup whose next tile's chunk is not in place takes pieces of that chunk
  *     too instead of spinning, so the launch finishes whichever of its workgroups are
  *     resident, and needs no second stream and no kernel running beside it;
- *   - pull_first 1: every GEMM workgroup starts by copying at the first remote chunk (as many
- *     workgroups begin on that comm block as on the local one); 0 or negative: only the
- *     workgroups that wait copy.  Measured slower than 0 at every shape tried; kept for
- *     measurements.
  *   elem_bytes 2 = smr_ag_matmul's arithmetic (bf16), 1 = smr_ag_matmul_fp8's (e4m3fn).
  *   state_dev  uint32 [smr_ag_matmul_fused_state_words(ws, splits)]: flags, tickets and
  *              counters.  Zero before the first launch; the last workgroup to finish zeroes
@@ -237,7 +231,7 @@ int smr_ag_matmul_schedule(int M, int N, int K, int rank, int world_size, int co
 int smr_ag_matmul_fused(const void* a_shard_dev, void* a_out_dev, const void* b_nk_dev, void* c_dev,
                         uint32_t* state_dev, const uint64_t* buffer_ptrs_dev, int elem_bytes, int M,
                         int N, int K, int rank, int world_size, int comm_block_m,
-                        int producer_workgroups, int pull_first, uint32_t* status, void* stream);
+                        int producer_workgroups, uint32_t* status, void* stream);
 int smr_ag_matmul_fused_state_words(int world_size, int splits_per_rank);
 
 /* The same GEMM with e4m3fn (OCP FP8) operands and result, fp32 accumulation: the
@@ -276,11 +270,6 @@ int smr_ag_matmul_plan(int M, int N, int K, int world_size, int comm_block_m, in
  * fence on.  Process-wide. */
 int smr_set_ag_matmul_acquire(int on);
 
-/* Tuning knob of the gated schedule: the first `head` and the last `tail` comm blocks
- * of the ring order are computed in tiles of half the width.  Both -1 (the default)
- * means none.  No reference counterpart. */
-int smr_set_ag_matmul_halves(int head, int tail);
-
 /* Tuning knob: cap on the workgroups of the GEMM's persistent grid (rounded down to a multiple
  * of 8; 0 = none), for measuring how the kernel scales with the compute units it is given.
  * Process-wide.  No reference counterpart (its grid is NUM_SMS, triton_all_gather_matmul.py:287-294). */
@@ -293,19 +282,6 @@ int smr_set_ag_matmul_grid_limit(int workgroups);
  * engine and needs no compute units, triton_all_gather_matmul.py:46-49). */
 int smr_ag_matmul_grid(int M, int N, int K, int world_size, int comm_block_m, int gated);
 
-/* Measurement aid, no reference counterpart (its launch metadata publishes flops for a
- * profiler, triton_all_gather_matmul.py:59-69): `workgroups` workgroups of 256 threads issue
- * 64 * iters v_mfma_f32_16x16x32_bf16 per wave back to back on operands read once from
- * values_dev (bf16 [nvalues]); nothing else runs in the loop.  What the matrix cores sustain
- * at the clock the part's power management allows under that load is the ceiling to hold a
- * GEMM against; the published peak assumes the top clock.
- *   ticks_dev  uint64 [2 * workgroups]: per workgroup, elapsed ticks of the constant 100 MHz
- *              clock and elapsed shader clock cycles
- *   sink_dev   float [256 * workgroups]: keeps the arithmetic alive
- * FLOPs issued: workgroups * 4 waves * 64 * iters * 16384. */
-int smr_probe_mfma_only(const void* values_dev, int nvalues, int workgroups, int iters,
-                        uint64_t* ticks_dev, float* sink_dev, void* stream);
-
 /* Split-K GEMV + rank-ordered combine through signal-pad flags.  No reference
  * code exists for it in symm_mem_recipes; it reuses the send/wait protocol of
  * triton_barrier.py:119-129 and triton_all_gather_matmul.py:72-95.
@@ -317,9 +293,13 @@ int smr_probe_mfma_only(const void* values_dev, int nvalues, int workgroups, int
  *   arrival word), zero on entry and zero again on exit.  Every producer raises its flag and
  *   counts itself in; the one that arrives last consumes the flags and adds the partials:
  *   out [batch,N] bf16 = the fp32 sum of the S partials in sender order (rank-major), i.e.
- *   bf16(((0 + p_0) + p_1) + ... + p_{ws-1}) when S == ws.  batch <= 8. */
-int smr_gemv_allreduce(const void* x_dev, const void* w_dev, float* partials_dev,
-                       uint32_t* flags_dev, void* out_dev, int batch, int K, int N,
+ *   bf16(((0 + p_0) + p_1) + ... + p_{ws-1}) when S == ws.  batch <= 8.
+ *   partials_bytes, flag_words: what the caller allocated for the two scratch arrays.  The
+ *   layout of both follows the process-wide launch knobs (smr_set_gemv_launch), so a caller
+ *   that sized them under another setting is told (SMR_E_INVALID) instead of having the
+ *   kernel write past the end. */
+int smr_gemv_allreduce(const void* x_dev, const void* w_dev, float* partials_dev, int64_t partials_bytes,
+                       uint32_t* flags_dev, int64_t flag_words, void* out_dev, int batch, int K, int N,
                        int world_size, uint32_t* status, void* stream);
 int smr_gemv_flag_blocks(int N);
 int smr_gemv_senders(int N, int K, int world_size);
@@ -331,8 +311,8 @@ int smr_gemv_flag_words(int N, int K, int world_size);
  * a fixed array inside the library (one copy per GPU, 4 MiB + 16 KiB, held until the process
  * ends) instead of caller-provided scratch, and the call allocates nothing.
  *   Limits: smr_gemv_senders(N, K, ws) * batch * N * 4 <= smr_gemv_static_scratch_bytes()
- *   (4 MiB; K = N = 8192, batch 8, ws 8 needs 2 MiB) and at most 4096 workgroups; beyond
- *   them SMR_E_UNSUPPORTED.
+ *   (4 MiB; K = N = 8192, batch 8, ws 8 needs 2 MiB) and smr_gemv_flag_words(N, K, ws) <= 4096
+ *   (one word per workgroup and one per column block); beyond them SMR_E_UNSUPPORTED.
  *   Every call on a GPU uses that GPU's one array: calls that overlap on one GPU (two
  *   streams, two threads) race and must be serialised by the caller.  The flags are cleared
  *   by a small kernel ahead of the launch, so a call that timed out leaves nothing behind. */

@@ -1,49 +1,35 @@
-// Device-side building blocks shared by every kernel of libsmr_gfx950:
-// bf16 packing, the bounded-spin flag protocol (send / wait / blockwise barrier)
-// and the host-side error plumbing.  gfx950 only.
-#pragma once
+/*
+ * smr_device.h - the device side of the flag protocol, for HIP kernels of other libraries
+ * (gfx950).  Header-only, device-only: nothing here touches the host, and nothing of
+ * libsmr_gfx950.so needs to be linked.
+ *
+ * The reference's barrier and flag waits are device functions that other kernels import
+ * (symm_mem_recipes/triton_one_shot_all_reduce.py:9 imports blockwise_barrier,
+ * symm_mem_recipes/triton_all_gather_matmul.py:17 imports get_flat_tid); these are their
+ * counterparts:
+ *   smr::blockwise_barrier   symm_mem_recipes/triton_barrier.py:50-153
+ *   smr::send_signal         the send half, triton_barrier.py:119-122
+ *   smr::wait_signal_reset   the wait half, triton_barrier.py:124-129
+ *   smr::wait_signal         symm_mem_recipes/triton_all_gather_matmul.py:72-95
+ * (get_tid / get_flat_tid, triton_barrier.py:11-47, are threadIdx.x of a one-dimensional
+ * workgroup.)  Differences from the reference, all in the caller's favour: every spin is
+ * bounded by `limit_ticks` (ticks of the GPU's constant 100 MHz clock, 0 = unbounded as in the
+ * reference) and a spin that expires writes a SMR_ST_* code into `status` (nullable; layout in
+ * smr.h) and returns false instead of hanging; waiting lanes back off with s_sleep.
+ *
+ * Signal pads are zero-initialised uint32 arrays, one per rank; `signal_pad_ptrs` is a device
+ * array of world_size uint64 addresses; the slot of (block, peer) is pad[block * world_size +
+ * peer], as in triton_barrier.py:100-110.
+ */
+#ifndef SMR_DEVICE_H_
+#define SMR_DEVICE_H_
 
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
-#include "../../include/smr.h"
+#include "smr.h"
 
 namespace smr {
-
-// ---------------------------------------------------------------- host side
-void set_last_error(const char* msg);
-int fail(int code, const char* msg);            // records msg, returns code
-int check_hip(hipError_t e, const char* what);  // 0 or the hip error (recorded)
-uint64_t spin_limit_ticks();                    // current timeout in wall_clock64 ticks (0 = none)
-uint64_t* trace_buffer(int64_t min_words);      // the registered trace buffer if it is large enough
-
-// Layout of the optional trace buffer (uint64 words of the 100 MHz device clock):
-//   [0 .. 63]                       producer: word i = time flag i was raised, word 63 = start
-//   [64 + (wg*kTraceSteps + step)*4 + k]   GEMM workgroup wg, its step-th tile:
-//        k = 0 tile picked, 1 flag wait over, 2 K loop done, 3 tile stored
-constexpr int kTraceProducerWords = 64;
-constexpr int kTraceSteps = 16;
-constexpr int kTraceGemmWords = 256 * kTraceSteps * 4;
-
-// ---------------------------------------------------------------- bf16
-__device__ __forceinline__ float bf16_lo(uint32_t w) { return __uint_as_float(w << 16); }
-__device__ __forceinline__ float bf16_hi(uint32_t w) { return __uint_as_float(w & 0xFFFF0000u); }
-
-// fp32 -> bf16, round-to-nearest-even, NaN quieted; bit pattern in the low half.
-__device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {
-  uint32_t u = __float_as_uint(f);
-  uint32_t r = (u + 0x7FFFu + ((u >> 16) & 1u)) >> 16;
-  uint32_t q = (u >> 16) | 0x40u;
-  return ((u & 0x7FFFFFFFu) > 0x7F800000u) ? q : r;
-}
-// Two at once through the hardware conversion (v_cvt_pk_bf16_f32: round-to-nearest-even,
-// NaN quieted): one instruction instead of a dozen integer operations per pair.
-typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
-typedef float f32x2_t __attribute__((ext_vector_type(2)));
-__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
-  const f32x2_t v = {lo, hi};
-  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));
-}
 
 // ---------------------------------------------------------------- status
 __device__ __forceinline__ void report(uint32_t* status, uint32_t code, uint32_t a, uint32_t b,
@@ -259,3 +245,5 @@ __device__ __forceinline__ bool blockwise_barrier(const uint64_t* signal_pad_ptr
 }
 
 }  // namespace smr
+
+#endif /* SMR_DEVICE_H_ */

@@ -32,7 +32,7 @@
 #include <atomic>
 #include <type_traits>
 
-#include "smr_device.hpp"
+#include "smr_internal.hpp"
 
 namespace smr {
 
@@ -49,20 +49,13 @@ struct GemmSchedule {
   int rank, world_size, comm_block_m;
   int BM, BN;
   int grid;                      // persistent workgroups, a multiple of 8
-  // The comm blocks are visited in ring order starting at the local one.  The
-  // first `head` and the last `tail` ring positions can be cut into tiles of half
-  // the width (smr_set_ag_matmul_halves; 0 and 0 by default): a pass over half
-  // tiles takes half as long, so with the local comm block in halves every
-  // workgroup starts on rows that need no flag.
-  int head, tail;
-  int steps;                     // trips of the busiest workgroup (passes over all phases)
+  int steps;                     // trips of the busiest workgroup (passes over the tile order)
   int group_m;                   // row tiles per group of the tile order; divides the comm block's
   int acquire;                   // invalidate the caches behind every flag wait (smr_set_ag_matmul_acquire)
 };
 
 struct TileRef {
   int row0, col0;                // output tile origin
-  int cols;                      // tile width: BN or BN / 2
   int comm_block;                // progress flag index
   int local;                     // rows come from the local shard, no wait
   int a_row;                     // first row inside the source (shard-relative when local)
@@ -71,10 +64,9 @@ struct TileRef {
 __host__ __device__ inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
 
 // Tile visited by workgroup `wg` in trip `step` of the grid; false when it has none in that trip.
-// Three phases: `head` ring positions in half tiles, the middle in full tiles, `tail`
-// in half tiles.  A phase is walked in passes of `grid` tiles; within a pass XCD x
-// (workgroups with id % 8 == x) takes a contiguous run of the tile order.  The tile
-// order inside a phase is comm block (ring order), then group of row tiles, then column
+// The comm blocks are visited in ring order starting at the local one, in passes of `grid`
+// tiles; within a pass XCD x (workgroups with id % 8 == x) takes a contiguous run of the tile
+// order.  The tile order is comm block (ring order), then group of row tiles, then column
 // tile, then row tile: an XCD's run is then a patch about as wide as it is high, and
 // the workgroups that share an L2 load the fewest distinct A and B slabs.
 __host__ __device__ inline bool tile_for(const GemmSchedule& s, int wg, int step, TileRef& t) {
@@ -82,49 +74,37 @@ __host__ __device__ inline bool tile_for(const GemmSchedule& s, int wg, int step
   const int n_comm = s.M / s.comm_block_m;
   const int per_rank = n_comm / s.world_size;
   const int first_local = s.rank * per_rank;
-  int ring0 = 0;                                   // first ring position of the phase
-  for (int phase = 0; phase < 3; ++phase) {
-    const int positions = phase == 0 ? s.head : (phase == 1 ? n_comm - s.head - s.tail : s.tail);
-    const int bn = phase == 1 ? s.BN : s.BN / 2;
-    const int tn = ceil_div(s.N, bn);
-    const int tiles_per_cb = cb_tiles_m * tn;
-    const int total = positions * tiles_per_cb;
-    const int passes = ceil_div(total, s.grid);
-    if (step < passes) {
-      const int start = step * s.grid;
-      const int cnt = (total - start) < s.grid ? (total - start) : s.grid;
-      const int per_xcd = (cnt + 7) >> 3;
-      const int slot = wg >> 3;
-      if (slot >= per_xcd) return false;
-      const int in_pass = (wg & 7) * per_xcd + slot;
-      if (in_pass >= cnt) return false;
-      const int lin = start + in_pass;
-      const int pos = lin / tiles_per_cb;
-      const int rem = lin - pos * tiles_per_cb;
-      // inside a comm block: groups of group_m row tiles, column by column inside a group
-      const int per_group = s.group_m * tn;
-      const int group = rem / per_group;
-      const int in_group = rem - group * per_group;
-      const int tile_n = in_group / s.group_m;
-      const int tile_m = group * s.group_m + (in_group - tile_n * s.group_m);
-      const int cb = (first_local + ring0 + pos) % n_comm;
-      t.comm_block = cb;
-      t.row0 = cb * s.comm_block_m + tile_m * s.BM;
-      t.col0 = tile_n * bn;
-      t.cols = bn;
-      t.local = (cb / per_rank) == s.rank;
-      t.a_row = t.local ? t.row0 - first_local * s.comm_block_m : t.row0;
-      return true;
-    }
-    step -= passes;
-    ring0 += positions;
-  }
-  return false;
+  const int tn = ceil_div(s.N, s.BN);
+  const int tiles_per_cb = cb_tiles_m * tn;
+  const int total = n_comm * tiles_per_cb;
+  const int start = step * s.grid;
+  if (start >= total) return false;
+  const int cnt = (total - start) < s.grid ? (total - start) : s.grid;
+  const int per_xcd = (cnt + 7) >> 3;
+  const int slot = wg >> 3;
+  if (slot >= per_xcd) return false;
+  const int in_pass = (wg & 7) * per_xcd + slot;
+  if (in_pass >= cnt) return false;
+  const int lin = start + in_pass;
+  const int pos = lin / tiles_per_cb;
+  const int rem = lin - pos * tiles_per_cb;
+  // inside a comm block: groups of group_m row tiles, column by column inside a group
+  const int per_group = s.group_m * tn;
+  const int group = rem / per_group;
+  const int in_group = rem - group * per_group;
+  const int tile_n = in_group / s.group_m;
+  const int tile_m = group * s.group_m + (in_group - tile_n * s.group_m);
+  const int cb = (first_local + pos) % n_comm;
+  t.comm_block = cb;
+  t.row0 = cb * s.comm_block_m + tile_m * s.BM;
+  t.col0 = tile_n * s.BN;
+  t.local = (cb / per_rank) == s.rank;
+  t.a_row = t.local ? t.row0 - first_local * s.comm_block_m : t.row0;
+  return true;
 }
 
-// First tile of workgroup `wg` at or after trip `step` (a workgroup can sit out the
-// ragged last pass of a phase and still have work in the next phase); advances `step`
-// to that trip.  False when the workgroup is done.
+// First tile of workgroup `wg` at or after trip `step`; advances `step` to that trip.
+// False when the workgroup is done.
 __host__ __device__ inline bool next_tile(const GemmSchedule& s, int wg, int& step, TileRef& t) {
   for (; step < s.steps; ++step)
     if (tile_for(s, wg, step, t)) return true;
@@ -228,8 +208,7 @@ struct GemmTile {
   static constexpr int WM = BM / 2, WN = BN / 2;        // wave tile (2 x 2 waves)
   static constexpr int FM = WM / 16, FN = WN / 16;      // 16x16 fragments per wave tile
   static constexpr int GA = BM / 32, GB = BN / 32;      // 8-row load groups per wave and slab
-  // BN <= BM in every configuration; a slot takes the larger slab, which also lets a
-  // half-width tile share the ring (and the next tile's early loads) with a full one.
+  // BN <= BM in every configuration; a slot takes the larger slab.
   static constexpr int kSlotBytes = BM * kRowBytes;
   static constexpr int kLdsBytes = kRingSlots * kSlotBytes;
   static_assert(BN <= BM, "slot size is the A slab");
@@ -799,12 +778,6 @@ __device__ __forceinline__ void run_tile_fp8(const TileContext& cx, const TileRe
 // ever runs the GEMM's workgroups copy everything themselves, only later.  Pieces are written
 // through to memory; whoever completes a chunk's count raises its flag.
 //
-// On request (pull_first) every GEMM workgroup copies at the first remote chunk before its
-// first tile, so that the workgroups that begin on that comm block and those that begin on the
-// local one start their K loops together.  Off by default: with launches interleaved in
-// rotating order the launch that leaves the copying to those who wait ends earlier (bf16
-// M=16384 N=3584 K=8192: 3.3 against 4.3 % over the ungated GEMM; e4m3fn 0.3 against 1.6 %).
-//
 // State (uint32 words, zero before the first launch): flags[chunks], tickets[chunks],
 // finished[chunks], exits[1].  The last workgroup to leave zeroes all of it, so the next
 // launch - or the next replay of a captured graph - starts from zero again with no fill.
@@ -819,7 +792,6 @@ struct CopyJob {
   int pieces;                    // per chunk
   int chunks, splits, rank, world_size;
   int gemm_grid;                 // workgroups from here on only copy
-  int pull_chunk;                // chunk every GEMM workgroup copies at before its first tile, or -1
 };
 
 typedef __attribute__((address_space(1))) u32x4 GlobalVec;
@@ -1003,7 +975,6 @@ __global__ __launch_bounds__(kGemmThreads, 1) void ag_matmul_kernel(
   bool have = next_tile(s, blockIdx.x, step, tile);
   const uint8_t* a_base = nullptr;
   const uint8_t* b_base = nullptr;
-  if (job.buffer_ptrs != nullptr && job.pull_chunk >= 0) copy_pieces<1>(job, job.pull_chunk, lds0, trace);
   if (have) {
     a_base = a_rows_of(tile);
     b_base = b_nk + (int64_t)tile.col0 * cx.row_stride;
@@ -1014,7 +985,7 @@ __global__ __launch_bounds__(kGemmThreads, 1) void ag_matmul_kernel(
     if (trace != nullptr && trip < kTraceSteps && blockIdx.x < 256 && threadIdx.x == 0) {
       cx.tr = trace + kTraceProducerWords + ((size_t)blockIdx.x * kTraceSteps + trip) * 4;
       cx.tr[0] = cx.tr[1] = wall_clock64();
-      if (trip == 0) cx.tr[0] = t_entry;     // the first tile's wait includes the pull of the first chunk
+      if (trip == 0) cx.tr[0] = t_entry;
     }
     TileRef next;
     bool have_next = false;
@@ -1028,25 +999,10 @@ __global__ __launch_bounds__(kGemmThreads, 1) void ag_matmul_kernel(
       if (!have_next) return;
       a_next = a_rows_of(next);
       b_next = b_nk + (int64_t)next.col0 * cx.row_stride;
-      const int b_last = s.N - 1 - next.col0;
-      if constexpr (BN == 256) {
-        if (next.cols != BN) issue_prologue<BM, BN / 2>(cx, a_next, b_next, b_last);
-        else issue_prologue<BM, BN>(cx, a_next, b_next, b_last);
-      } else {
-        issue_prologue<BM, BN>(cx, a_next, b_next, b_last);
-      }
+      issue_prologue<BM, BN>(cx, a_next, b_next, s.N - 1 - next.col0);
     };
-    if constexpr (FP8 && BN == 256) {
-      if (tile.cols != BN) run_tile_fp8<BM, BN / 2>(cx, tile, a_base, b_base, preloaded, between);
-      else run_tile_fp8<BM, BN>(cx, tile, a_base, b_base, preloaded, between);
-    } else if constexpr (FP8) {
-      run_tile_fp8<BM, BN>(cx, tile, a_base, b_base, preloaded, between);
-    } else if constexpr (BN == 256) {
-      if (tile.cols != BN) run_tile<BM, BN / 2>(cx, tile, a_base, b_base, preloaded, between);
-      else run_tile<BM, BN>(cx, tile, a_base, b_base, preloaded, between);
-    } else {
-      run_tile<BM, BN>(cx, tile, a_base, b_base, preloaded, between);
-    }
+    if constexpr (FP8) run_tile_fp8<BM, BN>(cx, tile, a_base, b_base, preloaded, between);
+    else run_tile<BM, BN>(cx, tile, a_base, b_base, preloaded, between);
     if (cx.tr != nullptr) cx.tr[3] = wall_clock64();
     have = have_next;
     tile = next;
@@ -1093,16 +1049,16 @@ static int validate(int M, int N, int K, int rank, int world_size, int comm_bloc
   return 0;
 }
 
+// Compute units of the current device (cached per device: a process may drive several parts).
 static int cu_count() {
-  static std::atomic<int> cached{0};
-  int n = cached.load(std::memory_order_relaxed);
+  constexpr int kMaxDevices = 64;
+  static std::atomic<int> cached[kMaxDevices];
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return 256;
+  int n = cached[dev].load(std::memory_order_relaxed);
   if (n == 0) {
-    int dev = 0;
-    if (hipGetDevice(&dev) == hipSuccess &&
-        hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0)
-      cached.store(n, std::memory_order_relaxed);
-    else
-      return 256;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) return 256;
+    cached[dev].store(n, std::memory_order_relaxed);
   }
   return n;
 }
@@ -1115,11 +1071,7 @@ static int cu_count() {
 constexpr int kReservedCus = 8;
 
 static int total_steps(const GemmSchedule& s) {
-  const int cb_tiles_m = s.comm_block_m / s.BM;
-  const int n_comm = s.M / s.comm_block_m;
-  const int full = cb_tiles_m * ceil_div(s.N, s.BN), half = cb_tiles_m * ceil_div(s.N, s.BN / 2);
-  return ceil_div(s.head * half, s.grid) + ceil_div((n_comm - s.head - s.tail) * full, s.grid) +
-         ceil_div(s.tail * half, s.grid);
+  return ceil_div((s.M / s.BM) * ceil_div(s.N, s.BN), s.grid);
 }
 
 // Coarse model of a fused launch, for splitting the compute units between the GEMM and the
@@ -1178,11 +1130,8 @@ static FusedEstimate estimate_fused(const GemmSchedule& s, int cus, int grid, in
   return e;
 }
 
-// smr_set_ag_matmul_halves: ring positions cut into half tiles at either end of a
-// gated launch, or -1 to let make_schedule choose.
-// Process-wide tuning knobs.  Each is one atomic word (head and tail share one), read once
-// per call by make_schedule, so a setter on another thread changes a whole launch or none of it.
-static std::atomic<uint32_t> g_force_halves{0xFFFFFFFFu};   // head in the low half, tail in the high half; 0xFFFF = let the library choose
+// Process-wide tuning knobs.  Each is one atomic word, read once per call by make_schedule,
+// so a setter on another thread changes a whole launch or none of it.
 static std::atomic<int> g_acquire_after_flag{0};
 static std::atomic<int> g_grid_limit{0};                     // smr_set_ag_matmul_grid_limit: 0 = none
 
@@ -1191,12 +1140,8 @@ static GemmSchedule make_schedule(int M, int N, int K, int rank, int world_size,
   GemmSchedule s;
   s.M = M; s.N = N; s.K = K;
   s.rank = rank; s.world_size = world_size; s.comm_block_m = comm_block_m;
-  s.head = s.tail = 0;
   s.acquire = g_acquire_after_flag.load(std::memory_order_relaxed);
   const int grid_limit = g_grid_limit.load(std::memory_order_relaxed);
-  const uint32_t halves = g_force_halves.load(std::memory_order_relaxed);
-  const int force_head = (halves & 0xFFFFu) == 0xFFFFu ? -1 : (int)(halves & 0xFFFFu);
-  const int force_tail = (halves >> 16) == 0xFFFFu ? -1 : (int)(halves >> 16);
   pick_tile(M, N, comm_block_m, s.BM, s.BN, cus);
   const int tn = (N + s.BN - 1) / s.BN;
   const int total = (M / s.BM) * tn;
@@ -1221,16 +1166,6 @@ static GemmSchedule make_schedule(int M, int N, int K, int rank, int world_size,
         s.grid = g;
       }
     }
-  }
-  // Half-width phases are off unless asked for (smr_set_ag_matmul_halves).  They let
-  // every workgroup of a gated launch start on local rows, but half tiles are bound
-  // by their loads, and with a producer that delivers a chunk in less than a pass it
-  // is cheaper to let the workgroups of the first remote comm block wait for it.
-  const int n_comm = M / comm_block_m;
-  if (gated && elem_bytes == 2 && s.BN == 256 && force_head >= 0 && force_tail >= 0 &&
-      force_head + force_tail <= n_comm) {
-    s.head = force_head;
-    s.tail = force_tail;
   }
   // Rows per group: the divisor of the comm block's row tiles for which an XCD's run of
   // a full pass touches the fewest slabs (rows of the patch + columns of the patch).
@@ -1262,7 +1197,6 @@ struct FusedArgs {
   const uint64_t* buffer_ptrs_dev;
   uint32_t* state_dev;           // flags, tickets, finished, exits
   int producer_wgs;              // copy-only workgroups; 0 = the plan's
-  int pull_first;                // 1: every GEMM workgroup copies at the first remote chunk before its first tile
 };
 
 static int launch_gemm(int elem_bytes, const void* a_shard_dev, const void* a_out_dev, const void* b_nk_dev,
@@ -1305,18 +1239,16 @@ static int launch_gemm(int elem_bytes, const void* a_shard_dev, const void* a_ou
     job.rank = rank;
     job.world_size = world_size;
     job.gemm_grid = s.grid;
-    job.pull_chunk = -1;
-    if (world_size > 1) {
-      // the first remote chunk of the walk: split 0 of rank + 1
-      const int first = ((rank + 1) % world_size) * splits;
-      if (fused->pull_first > 0) job.pull_chunk = first;
-    }
     int producers = fused->producer_wgs > 0 ? fused->producer_wgs
                                             : estimate_fused(s, cus, s.grid, elem_bytes).producer_wgs;
     // a workgroup of this kernel fills a compute unit: more of them than there are compute
     // units would only queue up behind the GEMM's
     if (producers > cus - s.grid) producers = cus - s.grid;
-    if (producers < 0) producers = 0;
+    // Never none: the GEMM's workgroups copy only the chunks their own tiles wait for and read
+    // the local rows from the shard itself, so the local shard reaches a_out through a
+    // copy-only workgroup.  Pieces are taken by ticket, so one that is dispatched late (a part
+    // with fewer compute units than the grid) still finds whatever is left.
+    if (producers < 1) producers = 1;
     grid += (unsigned)producers;
     progress_dev = job.flags;
   }
@@ -1361,7 +1293,7 @@ int smr_ag_matmul_fused_state_words(int world_size, int splits_per_rank) {
 int smr_ag_matmul_fused(const void* a_shard_dev, void* a_out_dev, const void* b_nk_dev, void* c_dev,
                         uint32_t* state_dev, const uint64_t* buffer_ptrs_dev, int elem_bytes, int M, int N,
                         int K, int rank, int world_size, int comm_block_m, int producer_workgroups,
-                        int pull_first, uint32_t* status, void* stream) {
+                        uint32_t* status, void* stream) {
   using namespace smr;
   const char* why;
   if (elem_bytes != 1 && elem_bytes != 2)
@@ -1375,7 +1307,7 @@ int smr_ag_matmul_fused(const void* a_shard_dev, void* a_out_dev, const void* b_
     return fail(SMR_E_INVALID, "smr_ag_matmul_fused: chunks must be 16-byte multiples");
   if (producer_workgroups < 0 || producer_workgroups > 1024)
     return fail(SMR_E_INVALID, "smr_ag_matmul_fused: producer_workgroups must be 0..1024");
-  const FusedArgs fa = {buffer_ptrs_dev, state_dev, producer_workgroups, pull_first};
+  const FusedArgs fa = {buffer_ptrs_dev, state_dev, producer_workgroups};
   return launch_gemm(elem_bytes, a_shard_dev, a_out_dev, b_nk_dev, c_dev, nullptr, M, N, K, rank, world_size,
                      comm_block_m, status, stream, &fa);
 }
@@ -1421,13 +1353,6 @@ int smr_set_ag_matmul_grid_limit(int workgroups) {
   return 0;
 }
 
-int smr_set_ag_matmul_halves(int head, int tail) {
-  if ((head < 0) != (tail < 0)) return smr::fail(SMR_E_INVALID, "smr_set_ag_matmul_halves: both or neither negative");
-  if (head > 0xFFFE || tail > 0xFFFE) return smr::fail(SMR_E_INVALID, "smr_set_ag_matmul_halves: too large");
-  smr::g_force_halves.store(head < 0 ? 0xFFFFFFFFu : ((uint32_t)head | ((uint32_t)tail << 16)), std::memory_order_relaxed);
-  return 0;
-}
-
 // Fills the plan of a fused launch: {GEMM grid, producer workgroups, estimated
 // microseconds fused, estimated microseconds copy-then-multiply, sequential}.
 static void fill_plan(int M, int N, int K, int world_size, int comm_block_m, int elem_bytes, int32_t* out5) {
@@ -1440,7 +1365,7 @@ static void fill_plan(int M, int N, int K, int world_size, int comm_block_m, int
   const GemmSchedule u = make_schedule(M, N, K, 0, world_size, comm_block_m, cus, false, elem_bytes);
   const double tile_us = model_tile_us(u.BM, u.BN, K, elem_bytes, false);
   const int tiles = (M / u.BM) * ceil_div(N, u.BN);
-  // the ungated schedule ends on a pass of half tiles when that is shorter: count passes in halves
+  // (fitted with the rest of the model: a last pass that fills at most half of the grid counts as half a pass)
   const double passes = ceil_div(2 * tiles, u.grid) * 0.5;
   // (all chunks at once, the own shard included: read + write at what a copy reaches on the part)
   const double gather_us = 2.0 * elem_bytes * M * K / 5.4e6 + 4.0;
@@ -1487,7 +1412,7 @@ int smr_ag_matmul_schedule(int M, int N, int K, int rank, int world_size, int co
         rec[2] = t.row0;
         rec[3] = t.col0;
         rec[4] = s.BM;
-        rec[5] = t.cols;
+        rec[5] = s.BN;
         rec[6] = t.comm_block;
         rec[7] = t.local;
       }

@@ -14,12 +14,8 @@
 // written through the L2 (agent scope) and a chunk is published by waiting for their
 // acknowledgement: releasing cached stores instead costs a cache-wide write-back per
 // wave and chunk, which stalled the GEMM next to it (fused M=16384 N=3584 K=8192:
-// 860 us with the write-backs, 760 us without).  The producer can be paced
-// (smr_set_gather_pacing: full width for the first chunks, fewer workgroups after);
-// with write-through stores that no longer gains anything and is off by default.
-#include <atomic>
-
-#include "smr_device.hpp"
+// 860 us with the write-backs, 760 us without).
+#include "smr_internal.hpp"
 
 namespace smr {
 
@@ -28,10 +24,6 @@ namespace smr {
 // whichever of the two kernels is dispatched first.
 constexpr int kGatherThreads = 1024;
 constexpr int kGatherDefaultWorkgroups = 8;
-// Pacing (smr_set_gather_pacing): chunks copied at full width, workgroups that stay
-// for the rest.
-// (one atomic word, fast chunks in the low half: a launch reads the pair once)
-static std::atomic<uint32_t> g_gather_pacing{1024u << 16};
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef __attribute__((address_space(1))) u32x4 GlobalVec;
@@ -47,16 +39,13 @@ __device__ __forceinline__ void store_through(GlobalVec* p, u32x4 v) {
 __global__ __launch_bounds__(kGatherThreads) void all_gather_kernel(
     const uint64_t* __restrict__ buffer_ptrs, uint8_t* __restrict__ a_out,
     uint32_t* __restrict__ progress, uint32_t* __restrict__ counters, int rank, int world_size,
-    int64_t chunk_vecs, int splits_per_rank, uint64_t* trace, int fast_chunks, int slow_wgs) {
-  int done_chunks = 0;
+    int64_t chunk_vecs, int splits_per_rank, uint64_t* trace) {
   if (trace != nullptr && blockIdx.x == 0 && threadIdx.x == 0) trace[kTraceProducerWords - 1] = wall_clock64();
   for (int step = 0; step < world_size; ++step) {
     const int src_rank = (rank + step + 1) % world_size;
     for (int split = 0; split < splits_per_rank; ++split) {
       const int idx = src_rank * splits_per_rank + split;
-      // workgroups taking part in this chunk
-      const int nwg = done_chunks++ < fast_chunks ? (int)gridDim.x : slow_wgs;
-      if ((int)blockIdx.x >= nwg) continue;
+      const int nwg = (int)gridDim.x;
       const GlobalVec* src =
           (const GlobalVec*)(uintptr_t)buffer_ptrs[src_rank] + (int64_t)split * chunk_vecs;
       GlobalVec* dst = (GlobalVec*)(uintptr_t)a_out + (int64_t)idx * chunk_vecs;
@@ -139,15 +128,6 @@ __global__ __launch_bounds__(kGatherThreads) void all_gather_at_once_kernel(
 
 }  // namespace smr
 
-extern "C" int smr_set_gather_pacing(int fast_chunks, int slow_workgroups) {
-  if (fast_chunks < 0 || slow_workgroups < 0 || slow_workgroups > 1024)
-    return smr::fail(SMR_E_INVALID, "smr_set_gather_pacing: negative or too large");
-  if (fast_chunks > 0xFFFF) return smr::fail(SMR_E_INVALID, "smr_set_gather_pacing: negative or too large");
-  smr::g_gather_pacing.store((uint32_t)fast_chunks | ((uint32_t)(slow_workgroups == 0 ? 1024 : slow_workgroups) << 16),
-                             std::memory_order_relaxed);
-  return 0;
-}
-
 static int launch_gather(const uint64_t* buffer_ptrs_dev, void* a_out_dev, uint32_t* progress_dev,
                          uint32_t* counters_dev, int rank, int world_size, int64_t shard_bytes,
                          int splits_per_rank, int num_workgroups, void* stream, bool at_once) {
@@ -172,13 +152,10 @@ static int launch_gather(const uint64_t* buffer_ptrs_dev, void* a_out_dev, uint3
                        chunk_bytes / 16, splits_per_rank);
     return check_hip(hipGetLastError(), "smr_all_gather launch");
   }
-  const uint32_t pacing = g_gather_pacing.load(std::memory_order_relaxed);
-  const int fast_chunks = (int)(pacing & 0xFFFFu), slow_wgs = (int)(pacing >> 16);
   hipLaunchKernelGGL(all_gather_kernel, dim3(nwg), dim3(kGatherThreads), 0,
                      reinterpret_cast<hipStream_t>(stream), buffer_ptrs_dev,
                      reinterpret_cast<uint8_t*>(a_out_dev), progress_dev, counters_dev, rank,
-                     world_size, chunk_bytes / 16, splits_per_rank, trace_buffer(kTraceProducerWords),
-                     fast_chunks, slow_wgs < nwg ? slow_wgs : nwg);
+                     world_size, chunk_bytes / 16, splits_per_rank, trace_buffer(kTraceProducerWords));
   return check_hip(hipGetLastError(), "smr_all_gather_with_progress launch");
 }
 

@@ -15,7 +15,7 @@
 // handshake have adjacent ids, and with ws == 8 rank r's workgroups land on
 // XCD r, so every flag and every payload chunk crosses an XCD boundary like it
 // would cross a link between GPUs.
-#include "smr_device.hpp"
+#include "smr_internal.hpp"
 
 namespace smr {
 

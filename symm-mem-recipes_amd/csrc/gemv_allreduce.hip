@@ -25,7 +25,7 @@
 #include <cstdio>
 #include <mutex>
 
-#include "smr_device.hpp"
+#include "smr_internal.hpp"
 
 namespace smr {
 
@@ -425,11 +425,11 @@ static int static_scratch(unsigned char** out) {
 }
 
 // Validation and launch shared by the entry points.  `flag_capacity` (words) and
-// `partial_capacity` (bytes) bound what the kernel may touch of the two scratch arrays;
-// negative = the caller vouches for them.
+// `partial_capacity` (bytes) bound what the kernel may touch of the two scratch arrays; a
+// problem that needs more returns `too_small`.
 static int launch_gemv(const char* who, const void* x_dev, const void* w_dev, float* partials_dev,
-                       uint32_t* flags_dev, int64_t flag_capacity, int64_t partial_capacity, void* out_dev,
-                       int batch, int K, int N, int world_size, uint32_t* status, void* stream,
+                       uint32_t* flags_dev, int64_t flag_capacity, int64_t partial_capacity, int too_small,
+                       void* out_dev, int batch, int K, int N, int world_size, uint32_t* status, void* stream,
                        bool clear_flags) {
   char msg[160];
   auto bad = [&](int code, const char* what) {
@@ -451,9 +451,9 @@ static int launch_gemv(const char* who, const void* x_dev, const void* w_dev, fl
   if (grid64 > 4096) return bad(SMR_E_UNSUPPORTED, "more than 4096 workgroups cannot be co-resident");
   const unsigned grid = (unsigned)grid64;
   const int64_t flag_words = (int64_t)cblocks * (world_size * sub + 1);
-  if (flag_capacity >= 0 && flag_words > flag_capacity) return bad(SMR_E_UNSUPPORTED, "too many flags for the flag array");
-  if (partial_capacity >= 0 && (int64_t)world_size * sub * batch * N * 4 > partial_capacity)
-    return bad(SMR_E_UNSUPPORTED, "partial sums exceed the scratch array (senders * batch * N * 4 bytes)");
+  if (flag_words > flag_capacity) return bad(too_small, "the flag array is too small (smr_gemv_flag_words)");
+  if ((int64_t)world_size * sub * batch * N * 4 > partial_capacity)
+    return bad(too_small, "the partial sums exceed their array (senders * batch * N * 4 bytes)");
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
   const uint16_t* x = reinterpret_cast<const uint16_t*>(x_dev);
   const uint8_t* w = reinterpret_cast<const uint8_t*>(w_dev);
@@ -532,11 +532,11 @@ int smr_gemv_senders(int N, int K, int world_size) {
   return world_size * smr::gemv_sub_for(smr::gemv_launch_knobs(), N, K, world_size);
 }
 
-int smr_gemv_allreduce(const void* x_dev, const void* w_dev, float* partials_dev, uint32_t* flags_dev,
-                       void* out_dev, int batch, int K, int N, int world_size, uint32_t* status,
-                       void* stream) {
-  return smr::launch_gemv("smr_gemv_allreduce", x_dev, w_dev, partials_dev, flags_dev, -1, -1, out_dev, batch,
-                          K, N, world_size, status, stream, false);
+int smr_gemv_allreduce(const void* x_dev, const void* w_dev, float* partials_dev, int64_t partials_bytes,
+                       uint32_t* flags_dev, int64_t flag_words, void* out_dev, int batch, int K, int N,
+                       int world_size, uint32_t* status, void* stream) {
+  return smr::launch_gemv("smr_gemv_allreduce", x_dev, w_dev, partials_dev, flags_dev, flag_words, partials_bytes,
+                          SMR_E_INVALID, out_dev, batch, K, N, world_size, status, stream, false);
 }
 
 int smr_gemv_allreduce_static(const void* x_dev, const void* w_dev, void* out_dev, int batch, int K, int N,
@@ -549,7 +549,7 @@ int smr_gemv_allreduce_static(const void* x_dev, const void* w_dev, void* out_de
   // The array keeps whatever the last call left: a call that timed out may have left flags
   // up, so they are cleared (by a kernel) ahead of every launch.
   return launch_gemv("smr_gemv_allreduce_static", x_dev, w_dev, partials, flags, kStaticFlagWords,
-                     kStaticPartialBytes, out_dev, batch, K, N, world_size, status, stream, true);
+                     kStaticPartialBytes, SMR_E_UNSUPPORTED, out_dev, batch, K, N, world_size, status, stream, true);
 }
 
 int64_t smr_gemv_static_scratch_bytes(void) { return smr::kStaticPartialBytes; }

@@ -20,7 +20,7 @@
 // the spins end.
 #include <atomic>
 
-#include "smr_device.hpp"
+#include "smr_internal.hpp"
 
 namespace smr {
 

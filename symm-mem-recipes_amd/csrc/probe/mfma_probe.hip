@@ -7,9 +7,23 @@
 // fragments per wave (the GEMM's register tile), one wave per SIMD, operands taken once from
 // a caller's buffer, no LDS or memory traffic inside the loop.  It reports the elapsed ticks
 // of the GPU's constant 100 MHz clock and the elapsed shader cycles per workgroup.
-#include "smr_device.hpp"
+//
+// Built into a library of its own (libsmr_probe.so) that only the benchmark and its test
+// load: it is no part of the C ABI of libsmr_gfx950.so.  No reference counterpart (the
+// reference's launch metadata publishes flops for a profiler,
+// symm_mem_recipes/triton_all_gather_matmul.py:59-69).
+//
+//   int smr_probe_mfma_only(values_dev, nvalues, workgroups, iters, ticks_dev, sink_dev, stream)
+//     values_dev bf16 [nvalues]: operands, read once
+//     ticks_dev  uint64 [2 * workgroups]: per workgroup, elapsed ticks of the 100 MHz clock and
+//                elapsed shader clock cycles
+//     sink_dev   float [256 * workgroups]: keeps the arithmetic alive
+//     returns 0, -1 for a bad argument, or the hipError_t of the launch
+//   FLOPs issued: workgroups * 4 waves * 64 * iters * 16384.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
 
-namespace smr {
+namespace smr_probe {
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
@@ -49,16 +63,14 @@ __global__ __launch_bounds__(256, 1) void mfma_only_kernel(const uint16_t* __res
   }
 }
 
-}  // namespace smr
+}  // namespace smr_probe
 
 extern "C" int smr_probe_mfma_only(const void* values_dev, int nvalues, int workgroups, int iters,
                                    uint64_t* ticks_dev, float* sink_dev, void* stream) {
-  using namespace smr;
-  if (values_dev == nullptr || ticks_dev == nullptr || sink_dev == nullptr)
-    return fail(SMR_E_INVALID, "smr_probe_mfma_only: null pointer");
-  if (nvalues < 1 || workgroups < 1 || workgroups > 1024 || iters < 1)
-    return fail(SMR_E_INVALID, "smr_probe_mfma_only: nvalues, workgroups (1..1024) and iters must be positive");
+  using namespace smr_probe;
+  if (values_dev == nullptr || ticks_dev == nullptr || sink_dev == nullptr) return -1;
+  if (nvalues < 1 || workgroups < 1 || workgroups > 1024 || iters < 1) return -1;
   hipLaunchKernelGGL(mfma_only_kernel, dim3(workgroups), dim3(256), 0, reinterpret_cast<hipStream_t>(stream),
                      reinterpret_cast<const uint16_t*>(values_dev), nvalues, iters, ticks_dev, sink_dev);
-  return check_hip(hipGetLastError(), "smr_probe_mfma_only launch");
+  return (int)hipGetLastError();
 }

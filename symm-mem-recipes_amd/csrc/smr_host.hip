@@ -3,7 +3,7 @@
 #include <cstdio>
 #include <cstring>
 
-#include "smr_device.hpp"
+#include "smr_internal.hpp"
 
 namespace smr {
 

@@ -50,19 +50,16 @@ SIGNATURES = {
     "smr_all_gather_with_progress": (_i, [_p, _p, _p, _p, _i, _i, _i64, _i, _i, _p]),
     "smr_all_gather_at_once": (_i, [_p, _p, _p, _p, _i, _i, _i64, _i, _i, _p]),
     "smr_set_ag_matmul_acquire": (_i, [_i]),
-    "smr_ag_matmul_fused": (_i, [_p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _i, _p, _p]),
+    "smr_ag_matmul_fused": (_i, [_p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _p, _p]),
     "smr_ag_matmul_fused_state_words": (_i, [_i, _i]),
-    "smr_set_gather_pacing": (_i, [_i, _i]),
     "smr_ag_matmul": (_i, [_p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _p, _p]),
     "smr_ag_matmul_schedule": (_i, [_i, _i, _i, _i, _i, _i, _i, _p, _i]),
     "smr_ag_matmul_grid": (_i, [_i, _i, _i, _i, _i, _i]),
-    "smr_set_ag_matmul_halves": (_i, [_i, _i]),
     "smr_set_ag_matmul_grid_limit": (_i, [_i]),
     "smr_ag_matmul_plan": (_i, [_i, _i, _i, _i, _i, _p]),
     "smr_ag_matmul_fp8": (_i, [_p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _p, _p]),
     "smr_ag_matmul_plan_fp8": (_i, [_i, _i, _i, _i, _i, _p]),
-    "smr_probe_mfma_only": (_i, [_p, _i, _i, _i, _p, _p, _p]),
-    "smr_gemv_allreduce": (_i, [_p, _p, _p, _p, _p, _i, _i, _i, _i, _p, _p]),
+    "smr_gemv_allreduce": (_i, [_p, _p, _p, _i64, _p, _i64, _p, _i, _i, _i, _i, _p, _p]),
     "smr_gemv_allreduce_static": (_i, [_p, _p, _p, _i, _i, _i, _i, _p, _p]),
     "smr_gemv_static_scratch_bytes": (_i64, []),
     "smr_gemv_flag_blocks": (_i, [_i]),
@@ -73,6 +70,22 @@ SIGNATURES = {
 }
 
 _lib: Optional[C.CDLL] = None
+_probe: Optional[C.CDLL] = None
+
+PROBE_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "libsmr_probe.so")
+
+
+def load_probe() -> C.CDLL:
+    """libsmr_probe.so: the MFMA-only measurement kernel (csrc/probe/mfma_probe.hip), a library
+    of its own that only the benchmark and its test load - no part of the C ABI."""
+    global _probe
+    if _probe is None:
+        if not os.path.exists(PROBE_PATH):
+            raise SmrError(f"{PROBE_PATH} is missing: build it with `make -C symm-mem-recipes_amd/csrc`")
+        _probe = C.CDLL(PROBE_PATH)
+        _probe.smr_probe_mfma_only.restype = _i
+        _probe.smr_probe_mfma_only.argtypes = [_p, _i, _i, _i, _p, _p, _p]
+    return _probe
 
 
 class SmrError(RuntimeError):

@@ -17,7 +17,7 @@ from typing import Optional
 import torch
 
 from . import _lib
-from .symm_mem import EmulatedSymmetricMemory
+from .symm_mem import EmulatedSymmetricMemory, _get_backend_stream
 
 #: Flags, tickets and counters of the fused launch, one array per (device, stream, size): the
 #: kernel leaves it zeroed, so it is filled once when it is made and never again.
@@ -81,8 +81,7 @@ def _launch_producer(symm_mem, output, inp, progress, counters, splits_per_rank,
 def all_gather_matmul_tma_persistent(a_shard: torch.Tensor, b: torch.Tensor, a_out: torch.Tensor,
                                      c_out: torch.Tensor, configs: Optional[dict] = None,
                                      mm_only: bool = False, *, splits_per_rank: int = 1,
-                                     fused: Optional[bool] = None, pull_first: Optional[bool] = None,
-                                     producer_workgroups: Optional[int] = None,
+                                     fused=None, producer_workgroups: Optional[int] = None,
                                      check: bool = False) -> torch.Tensor:
     """``c_out = cat(all ranks' a_shard) @ b.T`` with ``b`` of shape [N, K]
     (K-contiguous), bf16 or - all four tensors - float8_e4m3fn.  ``mm_only`` skips the gather and the flags and multiplies
@@ -93,9 +92,11 @@ def all_gather_matmul_tma_persistent(a_shard: torch.Tensor, b: torch.Tensor, a_o
     Keyword arguments beyond the reference's signature (triton_all_gather_matmul.py:219-221):
     ``fused``      None: the library's plan decides between the fused launch and, for a GEMM too
                    short to hide the copy behind, copy-then-multiply; True / False force one.
-    ``pull_first`` True: every GEMM workgroup copies at the first remote chunk before its first
-                   tile; None / False: only the workgroups that wait for a chunk copy at it.
-    ``producer_workgroups`` copy-only workgroups of the fused launch; None = the plan's.
+                   "streams": the reference's own choreography (:246-253, 318) - fresh zeroed
+                   flags, the stand-alone producer on the backend stream, the GEMM on the
+                   current stream gated on flags that the producer raises, stream join.
+    ``producer_workgroups`` copy-only workgroups of the fused launch (workgroups of the producer
+                   kernel with "streams"); None = the plan's.
     ``check``      synchronise and raise if a bounded wait inside the kernel expired (the result
                    is then not valid); without it the caller looks at ``check_status()`` later.
     """
@@ -118,6 +119,7 @@ def all_gather_matmul_tma_persistent(a_shard: torch.Tensor, b: torch.Tensor, a_o
     N = b.shape[0]
     K = a_shard.shape[1]
 
+    assert fused in (None, True, False, "streams"), "fused must be None, True, False or 'streams'"
     assert b.shape[1] == K
     assert a_out.shape[0] == M
     assert a_out.shape[1] == K
@@ -148,7 +150,23 @@ def all_gather_matmul_tma_persistent(a_shard: torch.Tensor, b: torch.Tensor, a_o
     sequential = bool(plan[4]) if fused is None else not fused
     chunks = world_size * splits_per_rank
     state = None
-    if sequential:
+    if fused == "streams":
+        # The reference's form: `progress` starts at zero, the producer runs on the backend
+        # stream behind everything queued so far, the GEMM on the current stream waits for each
+        # chunk's flag, and the current stream joins the backend stream at the end.  The GEMM's
+        # grid leaves compute units free for the producer (smr_ag_matmul_grid), so the two run
+        # side by side whichever is dispatched first; every wait inside the GEMM is bounded.
+        flags = torch.zeros(2 * chunks, dtype=torch.int32, device=device)     # progress, arrival counters
+        backend_stream = _get_backend_stream()
+        flags.record_stream(backend_stream)
+        backend_stream.wait_stream(current)
+        _launch_producer(symm_mem, a_out, a_shard, flags[:chunks], flags[chunks:], splits_per_rank,
+                         int(plan[1]) if producer_workgroups is None else int(producer_workgroups),
+                         backend_stream.cuda_stream)
+        rc = gemm(a_shard.data_ptr(), a_out.data_ptr(), b.data_ptr(), c_out.data_ptr(), flags.data_ptr(), M, N, K,
+                  rank, world_size, COMM_BLOCK_SIZE_M, status_ptr, current.cuda_stream)
+        current.wait_stream(backend_stream)
+    elif sequential:
         # Too small to hide the copy behind the GEMM: the whole GPU copies, then the whole
         # GPU multiplies, in stream order (the GEMM then needs no flags).
         scratch = torch.zeros(2 * chunks, dtype=torch.int32, device=device)
@@ -165,8 +183,7 @@ def all_gather_matmul_tma_persistent(a_shard: torch.Tensor, b: torch.Tensor, a_o
         rc = lib.smr_ag_matmul_fused(
             a_shard.data_ptr(), a_out.data_ptr(), b.data_ptr(), c_out.data_ptr(), state.data_ptr(),
             symm_mem.buffer_ptrs_dev, 1 if fp8 else 2, M, N, K, rank, world_size, COMM_BLOCK_SIZE_M,
-            0 if producer_workgroups is None else int(producer_workgroups),
-            -1 if pull_first is None else int(bool(pull_first)), status_ptr, current.cuda_stream)
+            0 if producer_workgroups is None else int(producer_workgroups), status_ptr, current.cuda_stream)
     _lib.check(rc, "all_gather_matmul")
     if check:
         try:
@@ -271,6 +288,15 @@ def main(argv=None) -> None:
     lat_us = benchmark_with_event(
         lambda: all_gather_matmul_tma_persistent(a_shard, b, a, c, configs), flush_l2=True)
     print(f"hip all_gather_matmul: {lat_us} us")
+    symm_mem.check_status()
+    # the reference's own choreography: producer on the backend stream, GEMM gated on its flags
+    c2 = torch.empty_like(c)
+    all_gather_matmul_tma_persistent(a_shard, b, a, c2, configs, fused="streams")
+    symm_mem.check_status()
+    assert torch.equal(c1.view(torch.int16), c2.view(torch.int16))
+    lat_us = benchmark_with_event(
+        lambda: all_gather_matmul_tma_persistent(a_shard, b, a, c, configs, fused="streams"), flush_l2=True)
+    print(f"hip all_gather_matmul, producer on a second stream: {lat_us} us")
     symm_mem.check_status()
 
 

@@ -61,9 +61,9 @@ def gemv_all_reduce(x: torch.Tensor, w: torch.Tensor, world_size: int = 8,
     assert workspace.flags.numel() >= lib.smr_gemv_flag_words(N, K, world_size), "workspace has too few flags"
     if out is None:
         out = torch.empty(batch, N, dtype=torch.bfloat16, device=x.device)
-    rc = _lib.load().smr_gemv_allreduce(
-        x.data_ptr(), w.data_ptr(), workspace.partials.data_ptr(), workspace.flags.data_ptr(),
-        out.data_ptr(), batch, K, N, world_size, workspace.status.data_ptr(),
-        torch.cuda.current_stream(x.device).cuda_stream)
+    rc = lib.smr_gemv_allreduce(
+        x.data_ptr(), w.data_ptr(), workspace.partials.data_ptr(), workspace.partials.numel() * 4,
+        workspace.flags.data_ptr(), workspace.flags.numel(), out.data_ptr(), batch, K, N, world_size,
+        workspace.status.data_ptr(), torch.cuda.current_stream(x.device).cuda_stream)
     _lib.check(rc, "gemv_all_reduce")
     return out

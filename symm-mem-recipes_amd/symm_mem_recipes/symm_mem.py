@@ -73,6 +73,9 @@ class _Group:
         self.buffer_ptrs = torch.tensor(self.buffer_addrs, dtype=torch.int64, device=device)
         self.pad_ptrs = torch.tensor(self.pad_addrs, dtype=torch.int64, device=device)
         self.status = torch.zeros(_lib.STATUS_WORDS, dtype=torch.int32, device=device)
+        #: prepared launches of the entry points, keyed by (rank, size, options); they hold
+        #: addresses of this allocation and go with it
+        self.launches: Dict[tuple, tuple] = {}
 
 
 class EmulatedSymmetricMemory:

@@ -30,8 +30,8 @@ def trace_launch(M: int, N: int, K: int, mode: str = "fused", world_size: int = 
                  warm: int = 20, device=None, dtype: torch.dtype = torch.bfloat16) -> dict:
     """Run ``warm`` launches and return the time stamps of the last one, in microseconds from
     the first workgroup's entry.  ``mode``: "ungated", "fused" (the library's default launch),
-    "fused-pull" (every GEMM workgroup copies at the first remote chunk first) or "sequential"
-    (copy-then-multiply).
+    "streams" (the reference's choreography: stand-alone producer on the backend stream, GEMM
+    gated on its flags) or "sequential" (copy-then-multiply).
 
     Returns ``{"end_us", "producer_start_us", "flags_us": {chunk: t}, "steps": [per-step dict]}``;
     a step holds the medians over the workgroups of: start, wait (flag wait, with the copying
@@ -55,8 +55,7 @@ def trace_launch(M: int, N: int, K: int, mode: str = "fused", world_size: int = 
     words = PRODUCER_WORDS + GEMM_WORDS
     trace = torch.zeros(words, dtype=torch.int64, device=device)
 
-    kwargs = {"fused": {"sequential": False, "ungated": None}.get(mode, True),
-              "pull_first": mode == "fused-pull"}
+    kwargs = {"fused": {"sequential": False, "ungated": None, "streams": "streams"}.get(mode, True)}
     try:
         _lib.check(lib.smr_set_trace_buffer(trace.data_ptr(), words), "trace")
         for _ in range(warm):
@@ -75,7 +74,7 @@ def trace_launch(M: int, N: int, K: int, mode: str = "fused", world_size: int = 
     t0 = min(starts)
     us = lambda ticks: (ticks - t0) / TICKS_PER_US
     out = {"mode": mode, "steps": [], "flags_us": {}, "producer_start_us": None}
-    if mode in ("fused", "fused-pull"):
+    if mode in ("fused", "streams"):
         out["producer_start_us"] = us(t[PRODUCER_WORDS - 1])
         chunks = world_size * 1
         out["flags_us"] = {i: us(t[i]) for i in range(chunks) if t[i] > t0}
@@ -104,7 +103,7 @@ def main(argv=None) -> None:
     ap.add_argument("--N", type=int, default=3584)
     ap.add_argument("--K", type=int, default=8192)
     ap.add_argument("--fp8", action="store_true")
-    ap.add_argument("--modes", default="ungated,fused,fused-pull")
+    ap.add_argument("--modes", default="ungated,fused,streams")
     args = ap.parse_args(argv)
     dtype = torch.float8_e4m3fn if args.fp8 else torch.bfloat16
     for mode in args.modes.split(","):

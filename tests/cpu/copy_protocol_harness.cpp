@@ -56,7 +56,7 @@ int main(int argc, char** argv) {
   job.flags = state.data(); job.tickets = state.data() + chunks; job.finished = state.data() + 2 * chunks;
   job.exits = state.data() + 3 * chunks;
   job.chunk_vecs = chunk_vecs; job.pieces = (int)((chunk_vecs + kPullPieceVecs - 1) / kPullPieceVecs);
-  job.chunks = chunks; job.splits = splits; job.rank = 0; job.world_size = ws; job.gemm_grid = helper_wgs; job.pull_chunk = -1;
+  job.chunks = chunks; job.splits = splits; job.rank = 0; job.world_size = ws; job.gemm_grid = helper_wgs;
   const int wgs = copy_wgs + helper_wgs;
   gridDim.x = wgs;
   std::vector<pthread_barrier_t> bars(wgs);

@@ -25,7 +25,7 @@ def test_header_symbols_all_exported(lib):
 
 
 def test_version_and_timeout_roundtrip(lib):
-    assert lib.smr_version() == 100
+    assert lib.smr_version() == 110
     old = lib.smr_get_spin_timeout_us()
     assert old == 2_000_000
     assert lib.smr_set_spin_timeout_us(1234) == 0
@@ -136,9 +136,41 @@ def test_fused_entry_argument_errors(lib):
     f = lib.smr_ag_matmul_fused
     assert lib.smr_ag_matmul_fused_state_words(8, 2) == 49
     assert lib.smr_ag_matmul_fused_state_words(9, 1) == 0
-    assert f(p, p, p, p, None, p, 2, 2048, 256, 256, 0, 8, 256, 0, -1, None, None) == -1     # no state
-    assert f(p, p, p, p, p, None, 2, 2048, 256, 256, 0, 8, 256, 0, -1, None, None) == -1     # no address table
-    assert f(p, p, p, p, p, p, 3, 2048, 256, 256, 0, 8, 256, 0, -1, None, None) == -1        # element size
-    assert f(p, p, p, p, p, p, 2, 2048, 256, 200, 0, 8, 256, 0, -1, None, None) == -2        # K % 64
-    assert f(p, p, p, p, p, p, 2, 2048, 256, 256, 0, 8, 256, 2000, -1, None, None) == -1     # producer count
-    assert f(p, p, p, p, p, p, 1, 2048, 256, 192, 0, 8, 256, 0, -1, None, None) == -2        # e4m3fn: K % 128
+    assert f(p, p, p, p, None, p, 2, 2048, 256, 256, 0, 8, 256, 0, None, None) == -1     # no state
+    assert f(p, p, p, p, p, None, 2, 2048, 256, 256, 0, 8, 256, 0, None, None) == -1     # no address table
+    assert f(p, p, p, p, p, p, 3, 2048, 256, 256, 0, 8, 256, 0, None, None) == -1        # element size
+    assert f(p, p, p, p, p, p, 2, 2048, 256, 200, 0, 8, 256, 0, None, None) == -2        # K % 64
+    assert f(p, p, p, p, p, p, 2, 2048, 256, 256, 0, 8, 256, 2000, None, None) == -1     # producer count
+    assert f(p, p, p, p, p, p, 1, 2048, 256, 192, 0, 8, 256, 0, None, None) == -2        # e4m3fn: K % 128
+
+
+def test_gemv_scratch_sizes_are_checked_on_the_host(lib):
+    """smr_gemv_allreduce is told what the caller allocated: scratch sized under another
+    setting of the launch knobs, or by an older formula, is refused before any launch."""
+    p = 0x1000
+    K = N = 8192
+    words = lib.smr_gemv_flag_words(N, K, 8)
+    senders = lib.smr_gemv_senders(N, K, 8)
+    assert words == lib.smr_gemv_flag_blocks(N) * (senders + 1)
+    need = senders * 4 * N * 4
+    g = lib.smr_gemv_allreduce
+    assert g(p, p, p, need, p, words - 1, p, 4, K, N, 8, None, None) == -1
+    assert b"flag array" in lib.smr_last_error_string()
+    assert g(p, p, p, need - 4, p, words, p, 4, K, N, 8, None, None) == -1
+    assert b"partial sums" in lib.smr_last_error_string()
+    assert g(p, p, p, need, p, lib.smr_gemv_flag_blocks(N) * senders, p, 4, K, N, 8, None, None) == -1   # the old layout
+
+
+def test_device_header_is_device_only():
+    """include/smr_device.h is what kernels of other libraries include: it must not need the
+    library's private headers, and it declares no host function."""
+    text = open(os.path.join(ROOT, "include", "smr_device.h")).read()
+    includes = re.findall(r'#include\s+[<"]([^>"]+)[>"]', text)
+    assert sorted(includes) == ["hip/hip_runtime.h", "smr.h", "stdint.h"], includes
+    body = re.sub(r"/\*.*?\*/|//[^\n]*", "", text, flags=re.S)
+    for name in ("blockwise_barrier", "send_signal", "wait_signal", "wait_signal_reset"):
+        assert re.search(r"__device__ __forceinline__ \w+ " + name + r"\(", body), name
+    # every function in it is a device function
+    for line in body.splitlines():
+        if re.match(r"^\w[\w:<> ]* \w+\(.*", line) and "constexpr" not in line and "struct" not in line:
+            assert "__device__" in line, line

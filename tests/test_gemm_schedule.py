@@ -94,30 +94,6 @@ def test_schedule_other_shapes(M, N, K, ws, splits):
             assert ring == sorted(ring)
 
 
-@pytest.mark.parametrize("head,tail", [(0, 0), (1, 0), (0, 1), (1, 1), (2, 0), (2, 3), (4, 4)])
-def test_schedule_forced_half_tile_phases(lib, head, tail):
-    """Whatever comm blocks are cut into half tiles, every output tile is visited once
-    and in ring order - also by workgroups that sit out the ragged last pass of a
-    phase and have work again in the next one."""
-    try:
-        assert lib.smr_set_ag_matmul_halves(head, tail) == 0
-        for (M, N, K, ws) in [(8192, 1280, 192, 8), (16384, 3584, 8192, 8), (8192, 4096, 256, 8)]:
-            for rank in (0, 5):
-                s = gemm_schedule(M, N, K, rank, ws, M // ws)
-                _covers_exactly(s, M, N)
-                cols_of = {t["comm_block"]: t["cols"] for t in s}
-                order = [(rank + i) % ws for i in range(ws)]
-                assert [cols_of[cb] for cb in order] == [128] * head + [256] * (ws - head - tail) + [128] * tail
-                for tiles in _by_wg(s).values():
-                    ring = [(t["comm_block"] - rank) % ws for t in tiles]
-                    assert ring == sorted(ring)
-                    steps = [t["step"] for t in tiles]
-                    assert steps == sorted(set(steps))
-    finally:
-        lib.smr_set_ag_matmul_halves(-1, -1)
-    assert lib.smr_set_ag_matmul_halves(-1, 2) == -1
-
-
 def test_grid_leaves_room_for_the_producer(lib):
     # gated launches never take every compute unit (256 assumed without a GPU)
     for (M, N, K) in [(16384, 3584, 8192), (16384, 6656, 16384), (4096, 1792, 4096), (32768, 8192, 1024)]:

@@ -174,23 +174,6 @@ def test_fused_parity_splits_per_rank(cuda, either_form, M, N, K, ws, rank, spli
     assert np.array_equal(_t_bits(a_out), np.concatenate(shards))
 
 
-@pytest.mark.parametrize("head,tail", [(0, 0), (1, 0), (1, 1), (2, 0), (0, 2), (3, 3)])
-def test_fused_parity_half_tile_phases(cuda, lib, force_fused, head, tail):
-    """Every split of the gated schedule into half-width and full-width phases computes
-    the same product (the library picks one by cost; this forces the others)."""
-    from symm_mem_recipes import all_gather_matmul_tma_persistent
-    M, N, K, ws, rank = 8192, 1280, 192, 8, 5        # enough 256x256 tiles that the library keeps that shape
-    a_shard, h, shards, b, b_bits, a_out, c_out = _setup(M, N, K, ws, rank, cuda)
-    try:
-        assert lib.smr_set_ag_matmul_halves(head, tail) == 0
-        c_out.zero_()
-        all_gather_matmul_tma_persistent(a_shard, b, a_out, c_out, None, **force_fused)
-        h.check_status()
-    finally:
-        lib.smr_set_ag_matmul_halves(-1, -1)
-    _check(_t_bits(c_out), O.ag_matmul_ref(shards, b_bits))
-
-
 def test_fused_back_to_back_calls_are_identical(cuda, either_form):
     """Twenty fused launches in a row without a host synchronisation in between, the
     gathered operand wiped before each: flags, arrival counters and the two streams
@@ -272,28 +255,6 @@ def test_fused_launch_replays_from_a_graph(cuda, either_form, M, N, K):
     del graph
 
 
-@pytest.mark.parametrize("M,N,K,rank,splits", [(16384, 2048, 256, 0, 1), (16384, 2048, 192, 5, 1), (16384, 3072, 128, 7, 2)])
-def test_first_chunk_pulled_by_the_gemm(cuda, lib, M, N, K, rank, splits):
-    """On request every GEMM workgroup copies at the first remote chunk before its first tile:
-    same product, bit for bit, as with the copying left to the copy-only workgroups and the
-    waiters (the default); gathered operand complete; state zero again."""
-    from symm_mem_recipes import all_gather_matmul_tma_persistent
-    ws = 8
-    a_shard, h, shards, b, b_bits, a_out, c_out = _setup(M, N, K, ws, rank, cuda)
-    outs = []
-    for pull in (False, True, None):
-        a_out.zero_()
-        c = torch.full_like(c_out, float("nan"))
-        all_gather_matmul_tma_persistent(a_shard, b, a_out, c, None, splits_per_rank=splits, fused=True,
-                                         pull_first=pull)
-        h.check_status()
-        assert np.array_equal(_t_bits(a_out), np.concatenate(shards))
-        outs.append(c)
-    _check(_t_bits(outs[0]), O.ag_matmul_ref(shards, b_bits))
-    assert torch.equal(outs[0].view(torch.int16), outs[1].view(torch.int16))
-    assert torch.equal(outs[0].view(torch.int16), outs[2].view(torch.int16))
-
-
 @pytest.mark.parametrize("producers", [1, 8, 64])
 def test_fused_entry_through_the_abi(cuda, lib, producers):
     """smr_ag_matmul_fused called directly, twice on one state array that is zeroed once:
@@ -310,7 +271,7 @@ def test_fused_entry_through_the_abi(cuda, lib, producers):
         c_out.fill_(float("nan"))
         rc = lib.smr_ag_matmul_fused(a_shard.data_ptr(), a_out.data_ptr(), b.data_ptr(), c_out.data_ptr(),
                                      state.data_ptr(), h.buffer_ptrs_dev, 2, M, N, K, rank, ws, M // ws // splits,
-                                     producers, -1, h.status.data_ptr(), torch.cuda.current_stream(cuda).cuda_stream)
+                                     producers, h.status.data_ptr(), torch.cuda.current_stream(cuda).cuda_stream)
         assert rc == 0, lib.smr_last_error_string()
         h.check_status()
         assert state.cpu().tolist() == [0] * words, call
@@ -318,10 +279,10 @@ def test_fused_entry_through_the_abi(cuda, lib, producers):
         _check(_t_bits(c_out), want)
     bad = lib.smr_ag_matmul_fused
     args = (a_shard.data_ptr(), a_out.data_ptr(), b.data_ptr(), c_out.data_ptr())
-    assert bad(*args, None, h.buffer_ptrs_dev, 2, M, N, K, rank, ws, M // ws, 0, -1, None, None) == -1
-    assert bad(*args, state.data_ptr(), None, 2, M, N, K, rank, ws, M // ws, 0, -1, None, None) == -1
-    assert bad(*args, state.data_ptr(), h.buffer_ptrs_dev, 4, M, N, K, rank, ws, M // ws, 0, -1, None, None) == -1
-    assert bad(*args, state.data_ptr(), h.buffer_ptrs_dev, 2, M, N, K, rank, ws, M // ws, -3, -1, None, None) == -1
+    assert bad(*args, None, h.buffer_ptrs_dev, 2, M, N, K, rank, ws, M // ws, 0, None, None) == -1
+    assert bad(*args, state.data_ptr(), None, 2, M, N, K, rank, ws, M // ws, 0, None, None) == -1
+    assert bad(*args, state.data_ptr(), h.buffer_ptrs_dev, 4, M, N, K, rank, ws, M // ws, 0, None, None) == -1
+    assert bad(*args, state.data_ptr(), h.buffer_ptrs_dev, 2, M, N, K, rank, ws, M // ws, -3, None, None) == -1
 
 
 def test_fused_launch_needs_no_second_stream(cuda, lib):
@@ -347,9 +308,9 @@ def test_fused_launch_needs_no_second_stream(cuda, lib):
         state = torch.zeros(words, dtype=torch.int32, device=cuda)
         a_out.zero_()
         c_out.fill_(float("nan"))
-        # 1 producer asked for, but pull_first off and one copy-only workgroup: the waiters do most of it
+        # one copy-only workgroup: the waiters do most of the copying
         rc = lib.smr_ag_matmul_fused(a_shard.data_ptr(), a_out.data_ptr(), b.data_ptr(), c_out.data_ptr(),
-                                     state.data_ptr(), h.buffer_ptrs_dev, 2, M, N, K, rank, ws, M // ws, 1, 0,
+                                     state.data_ptr(), h.buffer_ptrs_dev, 2, M, N, K, rank, ws, M // ws, 1,
                                      h.status.data_ptr(), torch.cuda.current_stream(cuda).cuda_stream)
         assert rc == 0
         h.check_status()

@@ -108,34 +108,30 @@ def test_fp8_parity_random_shapes(cuda, either_form, M, N, K, ws, rank):
     _check(_bits(c_out), O.ag_matmul_ref_fp8(shards, b_bits))
 
 
-def test_fp8_first_chunk_pulled_by_the_gemm(cuda, lib):
-    """A launch wide enough that every GEMM workgroup copies at the first remote chunk before
-    its first tile: same codes as without, gathered operand complete; and the fused entry
-    through the C ABI with e4m3fn operands leaves its state zeroed."""
+def test_fp8_fused_entry_through_the_abi(cuda, lib):
+    """The fused entry through the C ABI with e4m3fn operands: the codes of the Python call,
+    gathered operand complete, state left zeroed."""
     from symm_mem_recipes import all_gather_matmul_tma_persistent
     M, N, K, ws, rank = 16384, 2048, 256, 8, 6
     a_shard, h, shards, b, b_bits, a_out, c_out = _setup(M, N, K, ws, rank, cuda)
-    outs = []
-    for pull in (False, True):
-        a_out.view(torch.uint8).zero_()
-        c = torch.full_like(c_out.view(torch.uint8), 0x7F).view(torch.float8_e4m3fn)
-        all_gather_matmul_tma_persistent(a_shard, b, a_out, c, None, fused=True, pull_first=pull)
-        h.check_status()
-        assert np.array_equal(_bits(a_out), np.concatenate(shards))
-        outs.append(_bits(c))
-    _check(outs[0], O.ag_matmul_ref_fp8(shards, b_bits))
-    assert np.array_equal(outs[0], outs[1])
+    a_out.view(torch.uint8).zero_()
+    c = torch.full_like(c_out.view(torch.uint8), 0x7F).view(torch.float8_e4m3fn)
+    all_gather_matmul_tma_persistent(a_shard, b, a_out, c, None, fused=True)
+    h.check_status()
+    assert np.array_equal(_bits(a_out), np.concatenate(shards))
+    want = _bits(c)
+    _check(want, O.ag_matmul_ref_fp8(shards, b_bits))
     words = lib.smr_ag_matmul_fused_state_words(ws, 1)
     state = torch.zeros(words, dtype=torch.int32, device=cuda)
     a_out.view(torch.uint8).zero_()
     rc = lib.smr_ag_matmul_fused(a_shard.data_ptr(), a_out.data_ptr(), b.data_ptr(), c_out.data_ptr(),
-                                 state.data_ptr(), h.buffer_ptrs_dev, 1, M, N, K, rank, ws, M // ws, 0, 1,
+                                 state.data_ptr(), h.buffer_ptrs_dev, 1, M, N, K, rank, ws, M // ws, 0,
                                  h.status.data_ptr(), torch.cuda.current_stream(cuda).cuda_stream)
     assert rc == 0
     h.check_status()
     assert state.cpu().tolist() == [0] * words
     assert np.array_equal(_bits(a_out), np.concatenate(shards))
-    assert np.array_equal(_bits(c_out), outs[0])
+    assert np.array_equal(_bits(c_out), want)
 
 
 def test_fp8_saturation_and_exact_small_integers(cuda, either_form):

@@ -56,21 +56,23 @@ def test_trace_of_a_launch(cuda):
     """The kernels' own time stamps: every workgroup's tiles in order, the producer's flags
     behind its start, and the fused launch's first wait no longer than the whole launch."""
     from symm_mem_recipes import trace
-    for mode in ("ungated", "fused", "fused-pull", "sequential"):
+    for mode in ("ungated", "fused", "streams", "sequential"):
         r = trace.trace_launch(16384, 2048, 256, mode, warm=2)
         assert r["end_us"] > 0 and r["steps"], mode
         assert sum(s["workgroups"] for s in r["steps"]) == (16384 // 256) * (2048 // 256), mode
         for s in r["steps"]:
             assert s["k_loop_us"] > 0 and s["wait_us"] >= 0 and s["last_stored_us"] <= r["end_us"]
-        if mode.startswith("fused"):
+        if mode in ("fused", "streams"):
             assert r["producer_start_us"] is not None and len(r["flags_us"]) >= 6
             assert all(v > r["producer_start_us"] for v in r["flags_us"].values())
 
 
-def test_mfma_only_probe(cuda, lib):
+def test_mfma_only_probe(cuda):
     """The measurement aid behind the bench's "mfma_only" figure: it runs, every workgroup
     reports its two clocks, and back-to-back MFMAs issue at 16 cycles apiece (a little more
     with the loop's branch), which is what the figure's FLOP count assumes."""
+    from symm_mem_recipes import _lib
+    lib = _lib.load_probe()
     wgs, iters = 16, 2000
     vals = torch.empty(4096, dtype=torch.bfloat16, device=cuda).normal_(0, 0.02)
     ticks = torch.zeros(2 * wgs, dtype=torch.int64, device=cuda)

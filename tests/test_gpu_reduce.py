@@ -285,6 +285,50 @@ def test_full_size_properties_64mib(cuda, dtype):
         assert _same(_bits(out[s:s + win]), want)
 
 
+
+@pytest.mark.parametrize("form", ["write_all", "two_shot"])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_write_back_forms_at_64mib(cuda, dtype, form):
+    """The forms that write the sum back into all eight buffers, at the largest sweep point
+    (64 MiB per buffer): (i) small integers over the whole message - exact in every order - all
+    eight buffers compared with an int32 sum taken before the call; (ii) real-valued data,
+    bit for bit against the oracle on three 1 MiB windows (head, unaligned middle, tail) of
+    every buffer."""
+    from symm_mem_recipes import one_shot_all_reduce
+    nbytes = 64 << 20
+    item = 2 if dtype == torch.bfloat16 else 4
+    numel = nbytes // item
+    t, h = _alloc(numel, dtype, cuda)
+    kwargs = dict(write_all=True, all_ranks=True) if form == "two_shot" else dict(write_all=True)
+    g = torch.Generator(device=cuda).manual_seed(2)
+    exact = torch.zeros(numel, dtype=torch.int32, device=cuda)
+    for r in range(WS):
+        buf = h.get_buffer(r, (numel,), dtype)
+        buf.copy_(torch.randint(-8, 9, (numel,), generator=g, device=cuda).to(dtype))
+        exact += buf.to(torch.int32)
+    one_shot_all_reduce(t, **kwargs)
+    h.check_status()
+    for r in range(WS):
+        assert torch.equal(h.get_buffer(r, (numel,), dtype).to(torch.int32), exact), r
+    del exact
+    win = (1 << 20) // item
+    starts = [0, (numel // 2 + 8 * 1237) // 8 * 8, numel - win]
+    bufs = {s: [] for s in starts}
+    for r in range(WS):
+        buf = h.get_buffer(r, (numel,), dtype)
+        buf.normal_(generator=g)
+        for s in starts:
+            bufs[s].append(_bits(buf[s:s + win]))
+    one_shot_all_reduce(t, **kwargs)
+    h.check_status()
+    for s in starts:
+        want = O.reduce_ref(bufs[s], "bf16" if dtype == torch.bfloat16 else "fp32")
+        for r in range(WS):
+            assert _same(_bits(h.get_buffer(r, (numel,), dtype)[s:s + win]), want), (s, r)
+    for r in range(WS):
+        assert int(h.get_signal_pad(r).abs().sum()) == 0
+
+
 def test_golden_vectors(cuda):
     """The committed vectors (tests/golden/reduce.npz), independent of the oracle's code."""
     import os

@@ -114,3 +114,34 @@ def test_assembly_stores_keep_their_data_registers(gemm_asm, tmp_path):
                 lines = [x.strip() for x in block.strip().splitlines()]
                 assert lines[-1].startswith("s_nop 1"), lines
     assert stores >= 2
+
+
+@pytest.mark.parametrize("key", [(256, 256, True), (256, 128, True), (128, 128, True)])
+def test_fp8_saturation_mode_surrounds_the_conversions_only(kernels, key):
+    """The e4m3fn epilogue converts with v_cvt_pk_fp8_f32 while MODE.FP16_OVFL (bit 23) is set, and
+    the MFMAs must never run with it: with the bit set they read a NaN operand as a number.  The
+    conversions are intrinsics with no ordering edge to the mode write, so the compiled code is
+    what is checked: in program order every conversion lies between the write that sets the bit
+    and the write that clears it, and no MFMA lies in such a window."""
+    assert key in kernels, sorted(kernels)
+    on, conversions, windows = False, 0, 0
+    for ln in kernels[key]:
+        code = ln.split(";")[0]
+        m = re.search(r"s_setreg_imm32_b32 hwreg\(HW_REG_MODE, 23, 1\), (\d+)", code)
+        if m:
+            assert on != (m.group(1) == "1"), "mode written twice the same way"
+            on = m.group(1) == "1"
+            windows += on
+            continue
+        assert not re.search(r"s_setreg", code), code.strip()        # no other mode write in the kernel
+        if "v_cvt_pk_fp8_f32" in code:
+            assert on, "conversion outside the saturation window"
+            conversions += 1
+        if "v_mfma_" in code:
+            assert not on, "MFMA inside the saturation window"
+    assert not on and windows >= 1 and conversions >= 16
+
+
+@pytest.mark.parametrize("key", [(256, 256, False), (256, 128, False), (128, 128, False)])
+def test_bf16_kernels_never_touch_the_mode_register(kernels, key):
+    assert not any("s_setreg" in ln.split(";")[0] for ln in kernels[key])
