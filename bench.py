@@ -246,7 +246,8 @@ def bench_mfma_only(dev):
 def bench_ag_matmul(dev, gated=True):
     import torch
     counters = _counters().get("gemm", {})
-    from symm_mem_recipes import EmulatedSymmetricMemory as SM, all_gather_matmul_tma_persistent
+    from symm_mem_recipes import EmulatedSymmetricMemory as SM, _lib, all_gather_matmul_tma_persistent
+    lib = _lib.load()
     M, N, K = 16384, 3584, 8192
     a_shard = SM.empty_strided_p2p((M // WS, K), (K, 1), torch.bfloat16, dev, world_size=WS, rank=0)
     h = SM.rendezvous(a_shard)
@@ -260,18 +261,39 @@ def bench_ag_matmul(dev, gated=True):
     c = torch.empty(M, N, dtype=torch.bfloat16, device=dev)
     flush = torch.empty(1 << 28, dtype=torch.int32, device=dev)      # 1 GiB > last-level cache
     flops = 2.0 * M * N * K
+    gated_grid = lib.smr_ag_matmul_grid(M, N, K, WS, M // WS, 1)
+
+    def ungated_on_the_gated_grid():
+        # the ungated launch held to the workgroups (and so the tiles) of the gated one: what the
+        # flags themselves cost is the gated launch against THIS; the whole-GPU launch below is
+        # also ahead by the compute units that the copy occupies on one GPU
+        lib.smr_set_ag_matmul_grid_limit(gated_grid)
+        try:
+            all_gather_matmul_tma_persistent(a_shard, b, a_out, c, None, mm_only=True)
+        finally:
+            lib.smr_set_ag_matmul_grid_limit(0)
+
     fns = [lambda: all_gather_matmul_tma_persistent(a_shard, b, a_out, c, None, mm_only=True),
-           lambda: torch.matmul(a_out, b.T, out=c)]
+           lambda: torch.matmul(a_out, b.T, out=c), ungated_on_the_gated_grid]
     if gated:
         fns.append(lambda: all_gather_matmul_tma_persistent(a_shard, b, a_out, c, None))
+        fns.append(lambda: all_gather_matmul_tma_persistent(a_shard, b, a_out, c, None, fused="streams"))
     us = _time_interleaved(fns, 25, 10, pre=flush.zero_)
-    us_ungated, us_lib, us_gated = us[0], us[1], (us[2] if gated else float("nan"))
+    us_ungated, us_lib, us_same_grid = us[0], us[1], us[2]
+    us_gated, us_streams = (us[3], us[4]) if gated else (float("nan"), float("nan"))
     h.check_status()
     SM.release()
     return dict(workload="all-gather matmul M=16384 N=3584 K=8192 bf16, 8 shards of [2048, 8192], rank 0",
                 flops=flops, us_gated=us_gated, us_ungated=us_ungated,
+                us_ungated_on_the_gated_grid=us_same_grid, gated_grid=gated_grid,
+                us_two_streams=us_streams, tflops_two_streams=flops / us_streams / 1e6,
                 tflops_gated=flops / us_gated / 1e6, tflops_ungated=flops / us_ungated / 1e6,
-                gating_overhead=us_gated / us_ungated - 1.0,
+                frac_ungated=flops / us_ungated / 1e6 / MFMA_BF16_PEAK_TFLOPS,
+                gating_overhead=us_gated / us_same_grid - 1.0,
+                gating_overhead_note="fused launch against the ungated launch on the same grid and tiles (the cost "
+                                     "of the flags and of the copy's traffic); against the ungated launch that "
+                                     "also has the copy's compute units: overhead_vs_whole_gpu",
+                overhead_vs_whole_gpu=us_gated / us_ungated - 1.0,
                 roofline={"bound": "mfma", "achieved": flops / us_gated / 1e6, "peak": MFMA_BF16_PEAK_TFLOPS,
                           "unit": "TFLOP/s", "frac": flops / us_gated / 1e6 / MFMA_BF16_PEAK_TFLOPS,
                           "traffic": counters.get("fused", {}).get("traffic"),

@@ -102,12 +102,14 @@ int smr_one_shot_all_reduce(const uint64_t* buffer_ptrs_dev, const uint64_t* sig
                             void* out, int64_t numel, int dtype, int rank, int world_size,
                             int write_all, int barrier_mode, uint32_t* status, void* stream);
 
-/* The same call for a host that knows the peers' buffer addresses: `buffer_ptrs_host` is a
- * HOST array of world_size device addresses, read during the call and passed to the kernel
- * as arguments, so no thread starts with a dependent load from the device table that the
- * reference's kernel reads (triton_one_shot_all_reduce.py:86-87).  Everything else, results
- * included, as smr_one_shot_all_reduce. */
-int smr_one_shot_all_reduce_addrs(const uint64_t* buffer_ptrs_host, const uint64_t* signal_pad_ptrs_dev,
+/* The same call for a host that knows the peers' addresses: `buffer_ptrs_host` and
+ * `signal_pad_ptrs_host` (NULL allowed when barrier_mode == SMR_BARRIER_NONE) are HOST arrays
+ * of world_size device addresses, read during the call and passed to the kernel as
+ * arguments, so no thread starts with a dependent load from the device tables that the
+ * reference's kernels read (triton_one_shot_all_reduce.py:86-87, triton_barrier.py:100-110):
+ * one memory round trip less in front of the data, one in front of the handshake.
+ * Everything else, results included, as smr_one_shot_all_reduce. */
+int smr_one_shot_all_reduce_addrs(const uint64_t* buffer_ptrs_host, const uint64_t* signal_pad_ptrs_host,
                                   void* out, int64_t numel, int dtype, int rank, int world_size,
                                   int write_all, int barrier_mode, uint32_t* status, void* stream);
 
@@ -196,16 +198,39 @@ int smr_all_gather_at_once(const uint64_t* buffer_ptrs_dev, void* a_out_dev,
  *   all others from a_out after waiting for progress[comm_block] == 1; tiles are
  *   visited starting at the local shard and proceeding in ring order.
  *   progress_dev NULL = ungated (the reference's mm_only comparator, :246-247).
- *   comm_block_m  rows per progress flag = M / ws / splits_per_rank. */
+ *   comm_block_m  rows per progress flag = M / ws / splits_per_rank.
+ *   whole_gpu     only looked at for a gated launch.  0: the launch leaves compute units free
+ *                 for a producer kernel that needs them (smr_all_gather_with_progress; see
+ *                 smr_ag_matmul_grid).  1: whoever raises the flags needs no compute units of
+ *                 his own - copy engines as in the reference (:46-55), or smr_all_gather_beside,
+ *                 whose workgroups fit beside this kernel's on the same compute units - and the
+ *                 launch takes every compute unit, like an ungated one. */
 int smr_ag_matmul(const void* a_shard_dev, const void* a_out_dev, const void* b_nk_dev,
                   void* c_dev, const uint32_t* progress_dev, int M, int N, int K, int rank,
-                  int world_size, int comm_block_m, uint32_t* status, void* stream);
+                  int world_size, int comm_block_m, int whole_gpu, uint32_t* status, void* stream);
+
+/* The same producer (same arguments, same order of chunks and flags, same final state) in a
+ * form that needs no compute units of its own, like the copy engines it stands in for
+ * (triton_all_gather_matmul.py:46-55): workgroups of 256 threads with a few dozen registers and
+ * no LDS, which the hardware places beside the GEMM's workgroups on the same compute units (a
+ * bf16 GEMM workgroup leaves at least 88 of a SIMD's 512 registers per lane).  The GEMM it
+ * feeds is launched with whole_gpu = 1.  The first rank's chunks - the ones half of the GEMM's
+ * workgroups wait for at the start - are copied at full speed, the others a little at a time:
+ * the GEMM needs a chunk per pass, and a copy that runs flat out beside it slows it down.
+ * Exception: the 256x256 tile of smr_ag_matmul_fp8 takes every register of its compute unit,
+ * so nothing fits beside it - with that GEMM use smr_all_gather_with_progress and whole_gpu = 0.
+ *   num_workgroups  0 = one per compute unit of a 256-CU part */
+int smr_all_gather_beside(const uint64_t* buffer_ptrs_dev, void* a_out_dev, uint32_t* progress_dev,
+                          uint32_t* counters_dev, int rank, int world_size, int64_t shard_bytes,
+                          int splits_per_rank, int num_workgroups, void* stream);
 
 /* Host-only: the tile order smr_ag_matmul uses on a 256-CU part.  Writes up to
  * max_tiles records of 8 int32 (workgroup, step, row0, col0, tile rows, tile
  * columns, comm_block, local; grouped by workgroup, in visiting order) and
  * returns the number of tiles, or a negative SMR_E_* code.
- * Counterpart of the index arithmetic at triton_all_gather_matmul.py:125-174. */
+ * Counterpart of the index arithmetic at triton_all_gather_matmul.py:125-174.
+ *   gated  0: ungated launch, 1: gated with compute units left to a producer kernel,
+ *          2: gated with whole_gpu = 1 */
 int smr_ag_matmul_schedule(int M, int N, int K, int rank, int world_size, int comm_block_m,
                            int gated, int32_t* out_records, int max_tiles);
 
@@ -241,7 +266,7 @@ int smr_ag_matmul_fused_state_words(int world_size, int splits_per_rank);
  * K % 128 == 0, N % 16 == 0; otherwise as smr_ag_matmul (same tile shapes, same schedule). */
 int smr_ag_matmul_fp8(const void* a_shard_dev, const void* a_out_dev, const void* b_nk_dev, void* c_dev,
                       const uint32_t* progress_dev, int M, int N, int K, int rank, int world_size,
-                      int comm_block_m, uint32_t* status, void* stream);
+                      int comm_block_m, int whole_gpu, uint32_t* status, void* stream);
 /* smr_ag_matmul_plan for the e4m3fn GEMM. */
 int smr_ag_matmul_plan_fp8(int M, int N, int K, int world_size, int comm_block_m, int32_t* out5);
 
@@ -275,9 +300,9 @@ int smr_set_ag_matmul_acquire(int on);
  * Process-wide.  No reference counterpart (its grid is NUM_SMS, triton_all_gather_matmul.py:287-294). */
 int smr_set_ag_matmul_grid_limit(int workgroups);
 
-/* Workgroups smr_ag_matmul launches on the current device for this shape; a
- * gated launch (progress_dev != NULL) keeps at least 8 compute units free for the
- * producer, whose workgroup count should not exceed the number left free.
+/* Workgroups smr_ag_matmul launches on the current device for this shape (gated: 0, 1 or 2
+ * as for smr_ag_matmul_schedule); a gated launch without whole_gpu keeps at least 8 compute
+ * units free for the producer, whose workgroup count should not exceed the number left free.
  * Host-only, no reference counterpart (the reference's producer is a copy
  * engine and needs no compute units, triton_all_gather_matmul.py:46-49). */
 int smr_ag_matmul_grid(int M, int N, int K, int world_size, int comm_block_m, int gated);

@@ -184,21 +184,47 @@ __device__ __forceinline__ void wait_signal(const uint32_t* addr, uint64_t limit
 
 // Blockwise barrier across the (emulated) ranks for one block index.
 //   lane r < ws:         send: CAS 0 -> 1 on pad[r][block*ws + rank]
-//   lane ws + r < 2*ws:  wait: CAS 1 -> 0 on pad[rank][block*ws + r]
+//   lane ws + r < 2*ws:  wait: until pad[rank][block*ws + r] == 1, then back to 0
 // The two halves are independent memory operations, so they run on different
 // lanes of the same wave and a round costs one atomic round trip, not two.  Pads
 // are all-zero again afterwards.
 //
+// A wait lane polls with loads and consumes the flag with a read-modify-write whose result
+// nobody waits for: only this lane ever takes the slot from 1 to 0, so once it has seen the
+// 1 the transition cannot fail, and the workgroup goes on one memory round trip after the
+// flag went up - as a CAS 1 -> 0 that finds the flag up does, but a CAS that comes too early
+// costs three (CAS, poll, CAS) where this costs two.  The write is acknowledged before this
+// lane polls the slot again: the next call starts by waiting for the wave's outstanding
+// memory operations, which by then have long returned.  (A second poll in flight half a
+// round trip behind the first was measured: the wave waits for both, 0.1 to 0.4 us slower.)
+//
 // Only the first wave touches memory-ordering machinery: the workgroup barrier in
 // front collects every wave's earlier stores, then that one wave releases (when
 // `publish` is set: the workgroup wrote data inside this kernel that the peers
-// will read), flips the flags and acquires; the closing workgroup barrier hands
-// the acquired view to the other waves, which share its L1 and L2.  A cache
+// will read), flips the flags and acquires (when `acquire` is set: the workgroup, or
+// anybody else on its compute unit or XCD, may have read the peers' data earlier inside
+// this kernel, so that stale lines could sit in a cache); the closing workgroup barrier
+// hands the acquired view to the other waves, which share its L1 and L2.  A cache
 // write-back and an invalidate per wave would otherwise dominate the round.
 // After the call every thread sees what the peers wrote before their call.
 // Needs at least 2*ws threads.  Returns false (to every thread of the workgroup
 // alike) when a spin timed out.
-__device__ __forceinline__ bool blockwise_barrier(const uint64_t* signal_pad_ptrs,
+//
+// `pads` is anything that yields rank r's pad address as pads[r]: the device table the
+// reference passes (const uint64_t*), or SignalPads, the same addresses by value - kernel
+// arguments, which saves the first wave a dependent load from memory in front of its atomics.
+struct SignalPads {
+  uint64_t p[SMR_MAX_WORLD_SIZE];
+  __device__ __forceinline__ uint64_t operator[](int r) const {
+    uint64_t v = p[0];
+#pragma unroll
+    for (int i = 1; i < SMR_MAX_WORLD_SIZE; ++i) v = (r == i) ? p[i] : v;
+    return v;
+  }
+};
+
+template <typename Pads>
+__device__ __forceinline__ bool blockwise_barrier(const Pads& signal_pad_ptrs,
                                                   uint32_t block_id, int rank, int world_size,
                                                   uint64_t limit_ticks, uint32_t* status,
                                                   bool publish = true, bool acquire = true) {
@@ -207,6 +233,8 @@ __device__ __forceinline__ bool blockwise_barrier(const uint64_t* signal_pad_ptr
   int bad = 0;
   if (lane < 64) {
     if (publish) __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+    // the consuming write of an earlier call on this slot has been performed
+    else wait_stores_acknowledged();
     if (lane < 2 * world_size) {
       const bool is_send = lane < world_size;
       const int peer = is_send ? lane : lane - world_size;
@@ -214,20 +242,17 @@ __device__ __forceinline__ bool blockwise_barrier(const uint64_t* signal_pad_ptr
       uint32_t* slot = pad + (size_t)block_id * world_size + (is_send ? rank : peer);
       // One loop for both kinds of lane: the wait lane of the rank's own slot
       // depends on the send lane next to it, so neither may spin in a loop of its
-      // own while the other is masked off.  Wait lanes poll with a plain load and
-      // attempt the CAS only when the flag is up.
-      const uint32_t from = is_send ? 0u : 1u, to = is_send ? 1u : 0u;
+      // own while the other is masked off.
       SpinClock clk(limit_ticks);
       uint32_t level = 0;
       bool ok = false;
       for (;;) {
-        // attempt first (the flag is usually already there); after a failed
-        // attempt a wait lane polls with plain loads until the flag shows up
-        if (is_send || level == 0 ||
-            __hip_atomic_load(slot, __ATOMIC_RELAXED, kScope) == from) {
-          uint32_t expected = from;
-          ok = __hip_atomic_compare_exchange_strong(slot, &expected, to, __ATOMIC_RELAXED,
+        if (is_send) {
+          uint32_t expected = 0u;
+          ok = __hip_atomic_compare_exchange_strong(slot, &expected, 1u, __ATOMIC_RELAXED,
                                                     __ATOMIC_RELAXED, kScope);
+        } else {
+          ok = __hip_atomic_load(slot, __ATOMIC_RELAXED, kScope) == 1u;
         }
         if (ok) break;
         backoff_sleep(level);
@@ -236,6 +261,8 @@ __device__ __forceinline__ bool blockwise_barrier(const uint64_t* signal_pad_ptr
       if (!ok) {
         report(status, is_send ? SMR_ST_SEND_TIMEOUT : SMR_ST_WAIT_TIMEOUT, rank, block_id, peer);
         bad = 1;
+      } else if (!is_send) {
+        __hip_atomic_fetch_and(slot, 0u, __ATOMIC_RELAXED, kScope);       // consume: 1 -> 0
       }
     }
     if (acquire) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");

@@ -473,8 +473,13 @@ __device__ __forceinline__ void run_tile(const TileContext& cx, const TileRef& t
   // order, so no barrier is needed.
   constexpr int kChunks = WN / 8;                 // 16-byte chunks per wave-tile row
   constexpr int kRowsPerStore = 64 / kChunks;
+  // (a row of 14 chunks - the 224-wide tile - is 224 bytes: consecutive rows start 32 bytes
+  // apart in the 256-byte bank row by themselves, and no position swizzle is needed)
+  constexpr bool kPow2 = (kChunks & (kChunks - 1)) == 0;
+  static_assert(32 % kRowsPerStore == 0, "whole store instructions per band");
   const uint32_t turn = lds0 + (kRingSlots - 1) * kSlot + wave * (32 * WN * 2);
   const int rd_row = ln / kChunks, rd_chunk = ln % kChunks;
+  const bool rd_lane = rd_row < kRowsPerStore;    // 64 lanes = 4 rows of 14 chunks and 8 lanes over
 #pragma unroll
   for (int band = 0; band < FM / 2; ++band) {
 #pragma unroll
@@ -487,16 +492,18 @@ __device__ __forceinline__ void run_tile(const TileContext& cx, const TileRef& t
         v.x = pack_bf16x2(d[0], d[1]);
         v.y = pack_bf16x2(d[2], d[3]);
         const int chunk = ni * 2 + (ln >> 5);
-        lds_write_b64(turn + wr_row * (WN * 2) + (((chunk ^ wr_row) & (kChunks - 1)) << 4) + ((ln >> 4) & 1) * 8, v);
+        const int pos = kPow2 ? ((chunk ^ wr_row) & (kChunks - 1)) : chunk;
+        lds_write_b64(turn + wr_row * (WN * 2) + (pos << 4) + ((ln >> 4) & 1) * 8, v);
       }
     }
 #pragma unroll
     for (int i = 0; i < 32 / kRowsPerStore; ++i) {
-      const int r = i * kRowsPerStore + rd_row;
-      const u32x4 v = lds_read_b128(turn + r * (WN * 2) + (((rd_chunk ^ r) & (kChunks - 1)) << 4));
+      const int r = i * kRowsPerStore + (rd_lane ? rd_row : 0);
+      const int pos = kPow2 ? ((rd_chunk ^ r) & (kChunks - 1)) : rd_chunk;
+      const u32x4 v = lds_read_b128(turn + r * (WN * 2) + (pos << 4));
       const int m = tile.row0 + wm * WM + band * 32 + r;
       const int n = tile.col0 + wn * WN + rd_chunk * 8;
-      if (n < s.N) *reinterpret_cast<u32x4*>(c + ((int64_t)m * s.N + n) * 2) = v;
+      if (rd_lane && n < s.N) *reinterpret_cast<u32x4*>(c + ((int64_t)m * s.N + n) * 2) = v;
     }
     // one 32-row band at a time: keeps the accumulator read-out from flooding
     // the vector registers
@@ -1015,10 +1022,21 @@ __global__ __launch_bounds__(kGemmThreads, 1) void ag_matmul_kernel(
 
 // Tile shape: the largest the flags' granularity allows, stepped down while the
 // problem has too few tiles to occupy more than half of the compute units.
-static int pick_tile(int M, int N, int comm_block_m, int& BM, int& BN, int cus = 256) {
+static int pick_tile(int M, int N, int comm_block_m, int& BM, int& BN, int cus = 256, bool wide_ok = false) {
   if (comm_block_m % 256 == 0) {
     BM = 256;
     BN = N >= 256 ? 256 : 128;
+    // 256x224 tiles when they fill every compute unit in whole passes and 256x256 tiles do not
+    // (M=16384 N=3584: 1024 tiles = 4 passes of 256 against 896 tiles = 4 passes of 224):
+    // the same number of passes, each an eighth shorter.  Only for a launch that has the
+    // whole GPU (bf16, no copy beside it).
+    if (wide_ok && N % 224 == 0 && cus % 8 == 0) {
+      const int t224 = (M / 256) * (N / 224), t256 = (M / 256) * ceil_div(N, 256);
+      if (t224 % cus == 0 && (int64_t)ceil_div(t224, cus) * 224 < (int64_t)ceil_div(t256, cus) * 256) {
+        BN = 224;
+        return 0;
+      }
+    }
     if (BN == 256 && (M / 256) * ceil_div(N, 256) * 2 <= cus) BN = 128;
     if (BN == 128 && (M / 256) * ceil_div(N, 128) * 2 <= cus) BM = 128;
   } else if (comm_block_m % 128 == 0) {
@@ -1135,23 +1153,28 @@ static FusedEstimate estimate_fused(const GemmSchedule& s, int cus, int grid, in
 static std::atomic<int> g_acquire_after_flag{0};
 static std::atomic<int> g_grid_limit{0};                     // smr_set_ag_matmul_grid_limit: 0 = none
 
+// How a launch shares the GPU: not gated at all; gated with compute units left free for a
+// producer kernel; gated by somebody who needs no compute units of his own (copy engines, or
+// the producer whose workgroups fit beside this kernel's: smr_all_gather_beside).
+enum GateKind : int { kUngated = 0, kGatedShare = 1, kGatedWhole = 2 };
+
 static GemmSchedule make_schedule(int M, int N, int K, int rank, int world_size, int comm_block_m,
-                                  int cus, bool gated, int elem_bytes = 2) {
+                                  int cus, int gated, int elem_bytes = 2) {
   GemmSchedule s;
   s.M = M; s.N = N; s.K = K;
   s.rank = rank; s.world_size = world_size; s.comm_block_m = comm_block_m;
   s.acquire = g_acquire_after_flag.load(std::memory_order_relaxed);
   const int grid_limit = g_grid_limit.load(std::memory_order_relaxed);
-  pick_tile(M, N, comm_block_m, s.BM, s.BN, cus);
-  const int tn = (N + s.BN - 1) / s.BN;
-  const int total = (M / s.BM) * tn;
-  int max_grid = ((gated ? cus - kReservedCus : cus) / 8) * 8;
+  int max_grid = ((gated == kGatedShare ? cus - kReservedCus : cus) / 8) * 8;
   if (grid_limit > 0 && grid_limit < max_grid) max_grid = grid_limit / 8 * 8;
   if (max_grid < 8) max_grid = 8;
+  pick_tile(M, N, comm_block_m, s.BM, s.BN, max_grid, gated != kGatedShare && elem_bytes == 2);
+  const int tn = (N + s.BN - 1) / s.BN;
+  const int total = (M / s.BM) * tn;
   const int passes = (total + max_grid - 1) / max_grid;
   const int need = ((total + passes - 1) / passes + 7) / 8 * 8;
   s.grid = need < max_grid ? need : max_grid;
-  if (gated) {
+  if (gated == kGatedShare) {
     // The producer runs on the compute units this grid leaves free, and a small or
     // skinny problem is over before a narrow producer has copied the shards.  Take
     // the grid (a multiple of 8) for which the later of the two - the GEMM's passes,
@@ -1201,7 +1224,7 @@ struct FusedArgs {
 
 static int launch_gemm(int elem_bytes, const void* a_shard_dev, const void* a_out_dev, const void* b_nk_dev,
                        void* c_dev, const uint32_t* progress_dev, int M, int N, int K, int rank,
-                       int world_size, int comm_block_m, uint32_t* status, void* stream,
+                       int world_size, int comm_block_m, int whole_gpu, uint32_t* status, void* stream,
                        const FusedArgs* fused) {
   using namespace smr;
   if (a_shard_dev == nullptr || a_out_dev == nullptr || b_nk_dev == nullptr || c_dev == nullptr)
@@ -1211,8 +1234,8 @@ static int launch_gemm(int elem_bytes, const void* a_shard_dev, const void* a_ou
     return fail(SMR_E_INVALID, elem_bytes == 1 ? "smr_ag_matmul_fp8: operands must be 16-byte aligned"
                                                : "smr_ag_matmul: operands must be 16-byte aligned");
   const int cus = cu_count();
-  const GemmSchedule s = make_schedule(M, N, K, rank, world_size, comm_block_m, cus,
-                                       progress_dev != nullptr || fused != nullptr, elem_bytes);
+  const int gate = fused != nullptr ? kGatedShare : (progress_dev == nullptr ? kUngated : (whole_gpu ? kGatedWhole : kGatedShare));
+  const GemmSchedule s = make_schedule(M, N, K, rank, world_size, comm_block_m, cus, gate, elem_bytes);
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
   const uint8_t* a0 = reinterpret_cast<const uint8_t*>(a_shard_dev);
   const uint8_t* a1 = reinterpret_cast<const uint8_t*>(a_out_dev);
@@ -1264,6 +1287,9 @@ static int launch_gemm(int elem_bytes, const void* a_shard_dev, const void* a_ou
   else if (s.BM == 256 && s.BN == 256)
     hipLaunchKernelGGL((ag_matmul_kernel<256, 256>), dim3(grid), dim3(kGemmThreads), 0, st, a0, a1, b,
                        c, progress_dev, s, lim, status, tb, job);
+  else if (s.BM == 256 && s.BN == 224)
+    hipLaunchKernelGGL((ag_matmul_kernel<256, 224>), dim3(grid), dim3(kGemmThreads), 0, st, a0, a1, b,
+                       c, progress_dev, s, lim, status, tb, job);
   else if (s.BM == 256)
     hipLaunchKernelGGL((ag_matmul_kernel<256, 128>), dim3(grid), dim3(kGemmThreads), 0, st, a0, a1, b,
                        c, progress_dev, s, lim, status, tb, job);
@@ -1277,12 +1303,12 @@ static int validate_fp8(int M, int N, int K, int rank, int world_size, int comm_
 
 int smr_ag_matmul(const void* a_shard_dev, const void* a_out_dev, const void* b_nk_dev, void* c_dev,
                   const uint32_t* progress_dev, int M, int N, int K, int rank, int world_size,
-                  int comm_block_m, uint32_t* status, void* stream) {
+                  int comm_block_m, int whole_gpu, uint32_t* status, void* stream) {
   using namespace smr;
   const char* why;
   if (int rc = validate(M, N, K, rank, world_size, comm_block_m, &why)) return fail(rc, why);
   return launch_gemm(2, a_shard_dev, a_out_dev, b_nk_dev, c_dev, progress_dev, M, N, K, rank, world_size,
-                     comm_block_m, status, stream, nullptr);
+                     comm_block_m, whole_gpu, status, stream, nullptr);
 }
 
 int smr_ag_matmul_fused_state_words(int world_size, int splits_per_rank) {
@@ -1309,7 +1335,7 @@ int smr_ag_matmul_fused(const void* a_shard_dev, void* a_out_dev, const void* b_
     return fail(SMR_E_INVALID, "smr_ag_matmul_fused: producer_workgroups must be 0..1024");
   const FusedArgs fa = {buffer_ptrs_dev, state_dev, producer_workgroups};
   return launch_gemm(elem_bytes, a_shard_dev, a_out_dev, b_nk_dev, c_dev, nullptr, M, N, K, rank, world_size,
-                     comm_block_m, status, stream, &fa);
+                     comm_block_m, 0, status, stream, &fa);
 }
 
 static void fill_plan(int M, int N, int K, int world_size, int comm_block_m, int elem_bytes, int32_t* out5);
@@ -1325,12 +1351,12 @@ static int validate_fp8(int M, int N, int K, int rank, int world_size, int comm_
 
 int smr_ag_matmul_fp8(const void* a_shard_dev, const void* a_out_dev, const void* b_nk_dev, void* c_dev,
                       const uint32_t* progress_dev, int M, int N, int K, int rank, int world_size,
-                      int comm_block_m, uint32_t* status, void* stream) {
+                      int comm_block_m, int whole_gpu, uint32_t* status, void* stream) {
   using namespace smr;
   const char* why;
   if (int rc = validate_fp8(M, N, K, rank, world_size, comm_block_m, &why)) return fail(rc, why);
   return launch_gemm(1, a_shard_dev, a_out_dev, b_nk_dev, c_dev, progress_dev, M, N, K, rank, world_size,
-                     comm_block_m, status, stream, nullptr);
+                     comm_block_m, whole_gpu, status, stream, nullptr);
 }
 
 int smr_set_ag_matmul_acquire(int on) {
@@ -1358,11 +1384,11 @@ int smr_set_ag_matmul_grid_limit(int workgroups) {
 static void fill_plan(int M, int N, int K, int world_size, int comm_block_m, int elem_bytes, int32_t* out5) {
   using namespace smr;
   const int cus = cu_count();
-  const GemmSchedule s = make_schedule(M, N, K, 0, world_size, comm_block_m, cus, true, elem_bytes);
+  const GemmSchedule s = make_schedule(M, N, K, 0, world_size, comm_block_m, cus, kGatedShare, elem_bytes);
   const FusedEstimate e = estimate_fused(s, cus, s.grid, elem_bytes);
   // The alternative for a problem too small to hide the copy behind: copy with the
   // whole GPU, then multiply with the whole GPU.
-  const GemmSchedule u = make_schedule(M, N, K, 0, world_size, comm_block_m, cus, false, elem_bytes);
+  const GemmSchedule u = make_schedule(M, N, K, 0, world_size, comm_block_m, cus, kUngated, elem_bytes);
   const double tile_us = model_tile_us(u.BM, u.BN, K, elem_bytes, false);
   const int tiles = (M / u.BM) * ceil_div(N, u.BN);
   // (fitted with the rest of the model: a last pass that fills at most half of the grid counts as half a pass)
@@ -1390,7 +1416,8 @@ int smr_ag_matmul_grid(int M, int N, int K, int world_size, int comm_block_m, in
   using namespace smr;
   const char* why;
   if (int rc = validate(M, N, K, 0, world_size, comm_block_m, &why)) return fail(rc, why);
-  return make_schedule(M, N, K, 0, world_size, comm_block_m, cu_count(), gated != 0).grid;
+  if (gated < 0 || gated > 2) return fail(SMR_E_INVALID, "smr_ag_matmul_grid: gated must be 0, 1 or 2");
+  return make_schedule(M, N, K, 0, world_size, comm_block_m, cu_count(), gated).grid;
 }
 
 int smr_ag_matmul_schedule(int M, int N, int K, int rank, int world_size, int comm_block_m,
@@ -1399,7 +1426,8 @@ int smr_ag_matmul_schedule(int M, int N, int K, int rank, int world_size, int co
   const char* why;
   if (int rc = validate(M, N, K, rank, world_size, comm_block_m, &why)) return fail(rc, why);
   // host-only: the schedule of a 256-CU part, the one the kernels are tuned for
-  const GemmSchedule s = make_schedule(M, N, K, rank, world_size, comm_block_m, 256, gated != 0);
+  if (gated < 0 || gated > 2) return fail(SMR_E_INVALID, "smr_ag_matmul_schedule: gated must be 0, 1 or 2");
+  const GemmSchedule s = make_schedule(M, N, K, rank, world_size, comm_block_m, 256, gated);
   int count = 0;
   for (int wg = 0; wg < s.grid; ++wg) {
     TileRef t;

@@ -24,6 +24,7 @@ namespace smr {
 // whichever of the two kernels is dispatched first.
 constexpr int kGatherThreads = 1024;
 constexpr int kGatherDefaultWorkgroups = 8;
+constexpr int kBesideDefaultWorkgroups = 256;
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef __attribute__((address_space(1))) u32x4 GlobalVec;
@@ -36,16 +37,30 @@ __device__ __forceinline__ void store_through(GlobalVec* p, u32x4 v) {
   asm volatile("global_store_dwordx4 %0, %1, off sc1\n\ts_nop 1" : : "v"(p), "v"(v) : "memory");
 }
 
-__global__ __launch_bounds__(kGatherThreads) void all_gather_kernel(
+// THREADS = 1024: a workgroup fills a compute unit (the producer beside a GEMM that leaves
+// compute units free).  THREADS = 256: one wave per SIMD with a few dozen registers and no LDS -
+// a workgroup that fits BESIDE a workgroup of the GEMM on the same compute unit (the GEMM's
+// waves hold 424 of a SIMD's 512 registers per lane), so the copy needs no compute units of its
+// own, like the copy engines it stands in for.  That form copies the first rank's chunks - the
+// ones half of the GEMM's workgroups wait for - as fast as it can and the others two loads per
+// thread at a time: the GEMM needs a chunk per pass, not as fast as memory can deliver it.
+template <int THREADS>
+__global__ __launch_bounds__(THREADS) void all_gather_kernel(
     const uint64_t* __restrict__ buffer_ptrs, uint8_t* __restrict__ a_out,
     uint32_t* __restrict__ progress, uint32_t* __restrict__ counters, int rank, int world_size,
     int64_t chunk_vecs, int splits_per_rank, uint64_t* trace) {
+  constexpr int kGatherThreads = THREADS;
   if (trace != nullptr && blockIdx.x == 0 && threadIdx.x == 0) trace[kTraceProducerWords - 1] = wall_clock64();
+  int done_chunks = 0;
   for (int step = 0; step < world_size; ++step) {
     const int src_rank = (rank + step + 1) % world_size;
     for (int split = 0; split < splits_per_rank; ++split) {
       const int idx = src_rank * splits_per_rank + split;
       const int nwg = (int)gridDim.x;
+      // (beside a GEMM: the first rank's chunks at full speed, the others two loads at a time -
+      // a burst of loads and stores fills the compute unit's memory pipeline, which the GEMM
+      // workgroup on the same compute unit feeds its tiles through)
+      const bool trickle = THREADS == 256 && done_chunks++ >= splits_per_rank;
       const GlobalVec* src =
           (const GlobalVec*)(uintptr_t)buffer_ptrs[src_rank] + (int64_t)split * chunk_vecs;
       GlobalVec* dst = (GlobalVec*)(uintptr_t)a_out + (int64_t)idx * chunk_vecs;
@@ -53,6 +68,18 @@ __global__ __launch_bounds__(kGatherThreads) void all_gather_kernel(
       // workgroup, which is what one compute unit needs to stream at its share
       const int64_t stride = (int64_t)nwg * kGatherThreads;
       int64_t i = (int64_t)blockIdx.x * kGatherThreads + threadIdx.x;
+      if (trickle) {
+        // (pairs with 6000 clocks of sleep in between finish the gather of 7 x 32 MiB in about
+        // 500 us, within the GEMM it feeds; without the sleep the GEMM beside it ran 2 % slower,
+        // single loads or twice the sleep fall behind the GEMM's need)
+        for (; i + stride < chunk_vecs; i += 2 * stride) {
+          const u32x4 v0 = __builtin_nontemporal_load(src + i), v1 = __builtin_nontemporal_load(src + i + stride);
+          store_through(dst + i, v0);
+          store_through(dst + i + stride, v1);
+#pragma unroll
+          for (int z = 0; z < 6; ++z) __builtin_amdgcn_s_sleep(16);
+        }
+      }
       for (; i + 7 * stride < chunk_vecs; i += 8 * stride) {
         u32x4 v[8];
 #pragma unroll
@@ -130,7 +157,8 @@ __global__ __launch_bounds__(kGatherThreads) void all_gather_at_once_kernel(
 
 static int launch_gather(const uint64_t* buffer_ptrs_dev, void* a_out_dev, uint32_t* progress_dev,
                          uint32_t* counters_dev, int rank, int world_size, int64_t shard_bytes,
-                         int splits_per_rank, int num_workgroups, void* stream, bool at_once) {
+                         int splits_per_rank, int num_workgroups, void* stream, bool at_once,
+                         bool beside = false) {
   using namespace smr;
   if (buffer_ptrs_dev == nullptr || a_out_dev == nullptr || progress_dev == nullptr ||
       counters_dev == nullptr)
@@ -144,7 +172,7 @@ static int launch_gather(const uint64_t* buffer_ptrs_dev, void* a_out_dev, uint3
     return fail(SMR_E_INVALID, "smr_all_gather_with_progress: chunks must be 16-byte multiples");
   if (num_workgroups < 0 || num_workgroups > 1024)
     return fail(SMR_E_INVALID, "smr_all_gather_with_progress: num_workgroups must be 0..1024");
-  const int nwg = num_workgroups == 0 ? kGatherDefaultWorkgroups : num_workgroups;
+  const int nwg = num_workgroups == 0 ? (beside ? kBesideDefaultWorkgroups : kGatherDefaultWorkgroups) : num_workgroups;
   if (at_once) {
     hipLaunchKernelGGL(all_gather_at_once_kernel, dim3(nwg), dim3(kGatherThreads), 0,
                        reinterpret_cast<hipStream_t>(stream), buffer_ptrs_dev,
@@ -152,10 +180,16 @@ static int launch_gather(const uint64_t* buffer_ptrs_dev, void* a_out_dev, uint3
                        chunk_bytes / 16, splits_per_rank);
     return check_hip(hipGetLastError(), "smr_all_gather launch");
   }
-  hipLaunchKernelGGL(all_gather_kernel, dim3(nwg), dim3(kGatherThreads), 0,
-                     reinterpret_cast<hipStream_t>(stream), buffer_ptrs_dev,
-                     reinterpret_cast<uint8_t*>(a_out_dev), progress_dev, counters_dev, rank,
-                     world_size, chunk_bytes / 16, splits_per_rank, trace_buffer(kTraceProducerWords));
+  if (beside)
+    hipLaunchKernelGGL(all_gather_kernel<256>, dim3(nwg), dim3(256), 0,
+                       reinterpret_cast<hipStream_t>(stream), buffer_ptrs_dev,
+                       reinterpret_cast<uint8_t*>(a_out_dev), progress_dev, counters_dev, rank,
+                       world_size, chunk_bytes / 16, splits_per_rank, trace_buffer(kTraceProducerWords));
+  else
+    hipLaunchKernelGGL(all_gather_kernel<kGatherThreads>, dim3(nwg), dim3(kGatherThreads), 0,
+                       reinterpret_cast<hipStream_t>(stream), buffer_ptrs_dev,
+                       reinterpret_cast<uint8_t*>(a_out_dev), progress_dev, counters_dev, rank,
+                       world_size, chunk_bytes / 16, splits_per_rank, trace_buffer(kTraceProducerWords));
   return check_hip(hipGetLastError(), "smr_all_gather_with_progress launch");
 }
 
@@ -173,4 +207,11 @@ extern "C" int smr_all_gather_at_once(const uint64_t* buffer_ptrs_dev, void* a_o
                                       int num_workgroups, void* stream) {
   return launch_gather(buffer_ptrs_dev, a_out_dev, progress_dev, counters_dev, rank, world_size,
                        shard_bytes, splits_per_rank, num_workgroups, stream, true);
+}
+
+extern "C" int smr_all_gather_beside(const uint64_t* buffer_ptrs_dev, void* a_out_dev, uint32_t* progress_dev,
+                                     uint32_t* counters_dev, int rank, int world_size, int64_t shard_bytes,
+                                     int splits_per_rank, int num_workgroups, void* stream) {
+  return launch_gather(buffer_ptrs_dev, a_out_dev, progress_dev, counters_dev, rank, world_size,
+                       shard_bytes, splits_per_rank, num_workgroups, stream, false, true);
 }

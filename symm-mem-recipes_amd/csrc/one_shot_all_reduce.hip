@@ -150,7 +150,7 @@ __device__ __forceinline__ Vec16 sum_in_rank_order(const Vec16 (&v)[WS]) {
 template <int KIND, int WS, bool WRITE_ALL>
 __global__ __launch_bounds__(kReduceMaxThreads) void one_shot_all_reduce_kernel(
     const uint64_t* __restrict__ buffer_ptrs, PeerPtrs by_value, const uint64_t* __restrict__ signal_pad_ptrs,
-    Vec16* __restrict__ out, int64_t nvec, int rank, int layout, int nblocks, int do_barrier,
+    SignalPads pads_by_value, Vec16* __restrict__ out, int64_t nvec, int rank, int layout, int nblocks, int do_barrier,
     uint64_t limit_ticks, uint32_t* status) {
   int block = blockIdx.x;
   const int nthreads = blockDim.x;
@@ -163,11 +163,13 @@ __global__ __launch_bounds__(kReduceMaxThreads) void one_shot_all_reduce_kernel(
       const int b = blockIdx.x * per_proxy + (threadIdx.x >> 3);
       const int j = threadIdx.x & 7;
       if (b < nblocks && j < WS && j != rank) {
-        uint32_t* to_rank = reinterpret_cast<uint32_t*>(signal_pad_ptrs[rank]) + (size_t)b * WS + j;
-        uint32_t* from_rank = reinterpret_cast<uint32_t*>(signal_pad_ptrs[j]) + (size_t)b * WS + rank;
+        const bool by_val = pads_by_value.p[0] != 0;
+        uint32_t* to_rank = reinterpret_cast<uint32_t*>(by_val ? pads_by_value[rank] : signal_pad_ptrs[rank]) + (size_t)b * WS + j;
+        uint32_t* from_rank = reinterpret_cast<uint32_t*>(by_val ? pads_by_value[j] : signal_pad_ptrs[j]) + (size_t)b * WS + rank;
         // one round per handshake of the rank's block (leading, and trailing if asked for)
         for (int round = 0; round < do_barrier; ++round) {
-          if (!send_signal(to_rank, limit_ticks)) {
+          // (a proxy publishes nothing: the peers' data are the work of earlier kernels)
+          if (!send_signal_relaxed(to_rank, limit_ticks)) {
             report(status, SMR_ST_SEND_TIMEOUT, j, b, rank);
             break;
           }
@@ -193,7 +195,16 @@ __global__ __launch_bounds__(kReduceMaxThreads) void one_shot_all_reduce_kernel(
   }
 
   // the peers' buffers were written by earlier kernels: nothing of this kernel to publish
-  if (do_barrier) blockwise_barrier(signal_pad_ptrs, block, rank, WS, limit_ticks, status, false);
+  // The peers' buffers were written by earlier kernels: nothing of this kernel to publish.
+  // And nothing to invalidate: a launch starts from invalidated caches, and no workgroup reads
+  // a peer's line before its own handshake (a line is never shared by two blocks: a block's
+  // slots are nthreads * 16 bytes in a row), so no cache can hold a line of the peers' data
+  // that is older than the handshake.  The invalidate an acquire stands for cost 1.3 us of a
+  // 14 us launch.
+  if (do_barrier) {
+    if (pads_by_value.p[0] != 0) blockwise_barrier(pads_by_value, block, rank, WS, limit_ticks, status, false, false);
+    else blockwise_barrier(signal_pad_ptrs, block, rank, WS, limit_ticks, status, false, false);
+  }
 
   GlobalVec* src[WS];
   if (buffer_ptrs != nullptr) {
@@ -220,31 +231,34 @@ __global__ __launch_bounds__(kReduceMaxThreads) void one_shot_all_reduce_kernel(
   }
   // Trailing handshake: nobody's buffer is overwritten (or, with write-back, read)
   // before every rank is through; it publishes this workgroup's stores.
-  if (do_barrier == 2) blockwise_barrier(signal_pad_ptrs, block, rank, WS, limit_ticks, status, true, true);
+  if (do_barrier == 2) {
+    if (pads_by_value.p[0] != 0) blockwise_barrier(pads_by_value, block, rank, WS, limit_ticks, status, true, true);
+    else blockwise_barrier(signal_pad_ptrs, block, rank, WS, limit_ticks, status, true, true);
+  }
 }
 
 template <int KIND, int WS>
 static int launch_ws(bool write_all, dim3 grid, int threads, hipStream_t s, const uint64_t* bp,
-                     const PeerPtrs& pv, const uint64_t* sp,
+                     const PeerPtrs& pv, const uint64_t* sp, const SignalPads& spv,
                      Vec16* out, int64_t nvec, int rank, int layout, int nblocks, int do_barrier,
                      uint32_t* status) {
   const uint64_t lim = spin_limit_ticks();
   if (write_all)
     hipLaunchKernelGGL((one_shot_all_reduce_kernel<KIND, WS, true>), grid, dim3(threads), 0, s,
-                       bp, pv, sp, out, nvec, rank, layout, nblocks, do_barrier, lim, status);
+                       bp, pv, sp, spv, out, nvec, rank, layout, nblocks, do_barrier, lim, status);
   else
     hipLaunchKernelGGL((one_shot_all_reduce_kernel<KIND, WS, false>), grid, dim3(threads), 0, s,
-                       bp, pv, sp, out, nvec, rank, layout, nblocks, do_barrier, lim, status);
+                       bp, pv, sp, spv, out, nvec, rank, layout, nblocks, do_barrier, lim, status);
   return check_hip(hipGetLastError(), "smr_one_shot_all_reduce launch");
 }
 
 template <int KIND>
 static int launch_dtype(int ws, bool write_all, dim3 grid, int threads, hipStream_t s, const uint64_t* bp,
-                        const PeerPtrs& pv, const uint64_t* sp, Vec16* out, int64_t nvec, int rank, int layout,
+                        const PeerPtrs& pv, const uint64_t* sp, const SignalPads& spv, Vec16* out, int64_t nvec, int rank, int layout,
                         int nblocks, int do_barrier, uint32_t* status) {
 #define SMR_WS_CASE(W)                                                                          \
   case W:                                                                                       \
-    return launch_ws<KIND, W>(write_all, grid, threads, s, bp, pv, sp, out, nvec, rank, layout, nblocks, \
+    return launch_ws<KIND, W>(write_all, grid, threads, s, bp, pv, sp, spv, out, nvec, rank, layout, nblocks, \
                               do_barrier, status);
   switch (ws) {
     SMR_WS_CASE(1) SMR_WS_CASE(2) SMR_WS_CASE(3) SMR_WS_CASE(4)
@@ -259,7 +273,7 @@ static int launch_dtype(int ws, bool write_all, dim3 grid, int threads, hipStrea
 // Validation and launch behind both entry points: the peers' addresses come either from the
 // device table (`buffer_ptrs_dev`) or, by value, from the host array `buffer_ptrs_host`.
 static int reduce_entry(const uint64_t* buffer_ptrs_dev, const uint64_t* buffer_ptrs_host,
-                        const uint64_t* signal_pad_ptrs_dev, void* out, int64_t numel, int dtype, int rank,
+                        const uint64_t* signal_pad_ptrs_dev, const uint64_t* signal_pad_ptrs_host, void* out, int64_t numel, int dtype, int rank,
                         int world_size, int write_all, int barrier_mode, uint32_t* status, void* stream) {
   using namespace smr;
   if (dtype != SMR_DTYPE_BF16 && dtype != SMR_DTYPE_FP32 && dtype != SMR_DTYPE_BF16_STEPWISE)
@@ -283,8 +297,16 @@ static int reduce_entry(const uint64_t* buffer_ptrs_dev, const uint64_t* buffer_
   }
   if (barrier_mode != SMR_BARRIER_NONE && barrier_mode != SMR_BARRIER_PROXY && barrier_mode != SMR_BARRIER_BOTH)
     return fail(SMR_E_INVALID, "smr_one_shot_all_reduce: unknown barrier_mode");
-  if (barrier_mode != SMR_BARRIER_NONE && signal_pad_ptrs_dev == nullptr)
+  if (barrier_mode != SMR_BARRIER_NONE && signal_pad_ptrs_dev == nullptr && signal_pad_ptrs_host == nullptr)
     return fail(SMR_E_INVALID, "smr_one_shot_all_reduce: signal pads required for the barrier");
+  SignalPads spv = {};
+  if (signal_pad_ptrs_host != nullptr && barrier_mode != SMR_BARRIER_NONE) {
+    for (int r = 0; r < world_size; ++r) {
+      if (signal_pad_ptrs_host[r] == 0 || (signal_pad_ptrs_host[r] & 3u))
+        return fail(SMR_E_INVALID, "smr_one_shot_all_reduce_addrs: signal pad addresses must be non-zero and 4-byte aligned");
+      spv.p[r] = signal_pad_ptrs_host[r];
+    }
+  }
   if (write_all && rank < 0 && barrier_mode != SMR_BARRIER_BOTH)
     return fail(SMR_E_INVALID, "smr_one_shot_all_reduce: the two-shot form (all ranks, write-back) needs SMR_BARRIER_BOTH");
   if (!write_all && out == nullptr)
@@ -313,13 +335,13 @@ static int reduce_entry(const uint64_t* buffer_ptrs_dev, const uint64_t* buffer_
   const uint64_t* table = buffer_ptrs_host != nullptr ? nullptr : buffer_ptrs_dev;
   if (dtype == SMR_DTYPE_BF16)
     return launch_dtype<SMR_DTYPE_BF16>(world_size, write_all != 0, dim3(grid), threads, s, table, pv,
-                                        signal_pad_ptrs_dev, o, nvec, rank, layout, nblocks, do_barrier, status);
+                                        signal_pad_ptrs_dev, spv, o, nvec, rank, layout, nblocks, do_barrier, status);
   if (dtype == SMR_DTYPE_BF16_STEPWISE)
     return launch_dtype<SMR_DTYPE_BF16_STEPWISE>(world_size, write_all != 0, dim3(grid), threads, s, table, pv,
-                                                 signal_pad_ptrs_dev, o, nvec, rank, layout, nblocks, do_barrier,
+                                                 signal_pad_ptrs_dev, spv, o, nvec, rank, layout, nblocks, do_barrier,
                                                  status);
   return launch_dtype<SMR_DTYPE_FP32>(world_size, write_all != 0, dim3(grid), threads, s, table, pv,
-                                      signal_pad_ptrs_dev, o, nvec, rank, layout, nblocks, do_barrier, status);
+                                      signal_pad_ptrs_dev, spv, o, nvec, rank, layout, nblocks, do_barrier, status);
 }
 
 extern "C" {
@@ -343,16 +365,16 @@ int smr_reduce_num_blocks(int64_t numel, int dtype) {
 int smr_one_shot_all_reduce(const uint64_t* buffer_ptrs_dev, const uint64_t* signal_pad_ptrs_dev,
                             void* out, int64_t numel, int dtype, int rank, int world_size,
                             int write_all, int barrier_mode, uint32_t* status, void* stream) {
-  return reduce_entry(buffer_ptrs_dev, nullptr, signal_pad_ptrs_dev, out, numel, dtype, rank, world_size,
+  return reduce_entry(buffer_ptrs_dev, nullptr, signal_pad_ptrs_dev, nullptr, out, numel, dtype, rank, world_size,
                       write_all, barrier_mode, status, stream);
 }
 
-int smr_one_shot_all_reduce_addrs(const uint64_t* buffer_ptrs_host, const uint64_t* signal_pad_ptrs_dev,
+int smr_one_shot_all_reduce_addrs(const uint64_t* buffer_ptrs_host, const uint64_t* signal_pad_ptrs_host,
                                   void* out, int64_t numel, int dtype, int rank, int world_size,
                                   int write_all, int barrier_mode, uint32_t* status, void* stream) {
   if (buffer_ptrs_host == nullptr)
     return smr::fail(SMR_E_INVALID, "smr_one_shot_all_reduce_addrs: buffer_ptrs_host is NULL");
-  return reduce_entry(nullptr, buffer_ptrs_host, signal_pad_ptrs_dev, out, numel, dtype, rank, world_size,
+  return reduce_entry(nullptr, buffer_ptrs_host, nullptr, signal_pad_ptrs_host, out, numel, dtype, rank, world_size,
                       write_all, barrier_mode, status, stream);
 }
 

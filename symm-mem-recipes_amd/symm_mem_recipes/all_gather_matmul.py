@@ -139,7 +139,7 @@ def all_gather_matmul_tma_persistent(a_shard: torch.Tensor, b: torch.Tensor, a_o
 
     if mm_only:
         rc = gemm(a_shard.data_ptr(), a_out.data_ptr(), b.data_ptr(), c_out.data_ptr(), 0, M, N, K, rank,
-                  world_size, COMM_BLOCK_SIZE_M, status_ptr, current.cuda_stream)
+                  world_size, COMM_BLOCK_SIZE_M, 0, status_ptr, current.cuda_stream)
         _lib.check(rc, "all_gather_matmul")
         return c_out
 
@@ -153,18 +153,25 @@ def all_gather_matmul_tma_persistent(a_shard: torch.Tensor, b: torch.Tensor, a_o
     if fused == "streams":
         # The reference's form: `progress` starts at zero, the producer runs on the backend
         # stream behind everything queued so far, the GEMM on the current stream waits for each
-        # chunk's flag, and the current stream joins the backend stream at the end.  The GEMM's
-        # grid leaves compute units free for the producer (smr_ag_matmul_grid), so the two run
-        # side by side whichever is dispatched first; every wait inside the GEMM is bounded.
+        # chunk's flag, and the current stream joins the backend stream at the end.  For bf16 the
+        # producer is the one whose workgroups fit beside the GEMM's on the same compute units
+        # (smr_all_gather_beside: it costs no compute units, like the reference's copy engines),
+        # and the GEMM takes the whole GPU.  The widest e4m3fn tile leaves no registers for a
+        # neighbour: there the producer gets compute units of its own and the GEMM's grid leaves
+        # them free.  Every wait inside the GEMM is bounded.
         flags = torch.zeros(2 * chunks, dtype=torch.int32, device=device)     # progress, arrival counters
         backend_stream = _get_backend_stream()
         flags.record_stream(backend_stream)
         backend_stream.wait_stream(current)
-        _launch_producer(symm_mem, a_out, a_shard, flags[:chunks], flags[chunks:], splits_per_rank,
-                         int(plan[1]) if producer_workgroups is None else int(producer_workgroups),
-                         backend_stream.cuda_stream)
+        beside = not fp8
+        producer = lib.smr_all_gather_beside if beside else lib.smr_all_gather_with_progress
+        wgs = (0 if beside else int(plan[1])) if producer_workgroups is None else int(producer_workgroups)
+        rc = producer(symm_mem.buffer_ptrs_dev, a_out.data_ptr(), flags.data_ptr(), flags[chunks:].data_ptr(),
+                      rank, world_size, a_shard.numel() * a_shard.element_size(), int(splits_per_rank), wgs,
+                      backend_stream.cuda_stream)
+        _lib.check(rc, "all_gather_with_progress")
         rc = gemm(a_shard.data_ptr(), a_out.data_ptr(), b.data_ptr(), c_out.data_ptr(), flags.data_ptr(), M, N, K,
-                  rank, world_size, COMM_BLOCK_SIZE_M, status_ptr, current.cuda_stream)
+                  rank, world_size, COMM_BLOCK_SIZE_M, int(beside), status_ptr, current.cuda_stream)
         current.wait_stream(backend_stream)
     elif sequential:
         # Too small to hide the copy behind the GEMM: the whole GPU copies, then the whole
@@ -174,7 +181,7 @@ def all_gather_matmul_tma_persistent(a_shard: torch.Tensor, b: torch.Tensor, a_o
         _launch_producer(symm_mem, a_out, a_shard, scratch[:chunks], scratch[chunks:], splits_per_rank, wide,
                          current.cuda_stream, at_once=True)
         rc = gemm(a_shard.data_ptr(), a_out.data_ptr(), b.data_ptr(), c_out.data_ptr(), 0, M, N, K, rank,
-                  world_size, COMM_BLOCK_SIZE_M, status_ptr, current.cuda_stream)
+                  world_size, COMM_BLOCK_SIZE_M, 0, status_ptr, current.cuda_stream)
     else:
         # One launch on the current stream: GEMM workgroups and copy-only workgroups in one
         # grid, flags in an array the kernel itself leaves zeroed (no fill, no second stream;
@@ -210,10 +217,12 @@ def all_gather_matmul(a_shard: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
 
 
 def gemm_schedule(M: int, N: int, K: int, rank: int, world_size: int, comm_block_m: int,
-                  gated: bool = True):
+                  gated=True):
     """The tile order the GEMM uses on a 256-CU part, as a list of dicts in each
     workgroup's visiting order (host-only; the counterpart of the index
-    arithmetic at triton_all_gather_matmul.py:125-174)."""
+    arithmetic at triton_all_gather_matmul.py:125-174).  ``gated``: False / 0 an ungated
+    launch, True / 1 a gated one that leaves compute units to a producer kernel, 2 a gated one
+    that takes the whole GPU (``whole_gpu`` of smr_ag_matmul)."""
     import ctypes
     lib = _lib.load()
     n = lib.smr_ag_matmul_schedule(M, N, K, rank, world_size, comm_block_m, int(gated), None, 0)

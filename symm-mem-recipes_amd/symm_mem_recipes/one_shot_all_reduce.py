@@ -42,10 +42,11 @@ def one_shot_all_reduce(tensor: torch.Tensor, *, barrier: bool = True, write_all
     ``trailing_barrier`` a second handshake after the last store (the reference
                    has none behind triton_one_shot_all_reduce.py:93): no peer
                    can overwrite its buffer while another still reads it.
-    ``device_table`` let the kernel read the peers' addresses from the table in device
-                   memory, as the reference's does (triton_one_shot_all_reduce.py:86-87);
-                   by default they are passed as kernel arguments, which saves every
-                   thread a dependent load in front of its first data load.
+    ``device_table`` let the kernel read the peers' buffer and signal pad addresses from the
+                   tables in device memory, as the reference's does
+                   (triton_one_shot_all_reduce.py:86-87, triton_barrier.py:100-110); by default
+                   they are passed as kernel arguments, which saves a dependent load in front
+                   of the handshake and another in front of the first data load.
     ``accumulate`` "fp32" (default) keeps an fp32 accumulator and rounds once;
                    "bf16" rounds the accumulator to bf16 after every add, which is
                    bit for bit the reference's add.bf16x2 chain
@@ -110,12 +111,13 @@ def _prepare(tensor: torch.Tensor, entry, key):
         kind = _OUT_ALL_RANKS
     else:
         kind = _OUT_NEW
-    fn, table = ((lib.smr_one_shot_all_reduce, symm_mem.buffer_ptrs_dev) if device_table
-                 else (lib.smr_one_shot_all_reduce_addrs, symm_mem.buffer_ptrs_host))
+    fn, table, pads = ((lib.smr_one_shot_all_reduce, symm_mem.buffer_ptrs_dev, symm_mem.signal_pad_ptrs_dev)
+                       if device_table else
+                       (lib.smr_one_shot_all_reduce_addrs, symm_mem.buffer_ptrs_host, symm_mem.signal_pad_ptrs_host))
     barrier_mode = ((_lib.BARRIER_BOTH if (trailing_barrier or two_shot) else _lib.BARRIER_PROXY) if barrier
                     else _lib.BARRIER_NONE)
     device_index = tensor.device.index if tensor.device.index is not None else torch.cuda.current_device()
-    launch = (fn, table, symm_mem.signal_pad_ptrs_dev, tensor.numel(),
+    launch = (fn, table, pads, tensor.numel(),
               _lib.DTYPE_BF16_STEPWISE if accumulate == "bf16" else _DTYPE_CODE[tensor.dtype],
               -1 if all_ranks else symm_mem.rank, symm_mem.world_size, 1 if write_all else 0, barrier_mode,
               symm_mem.status.data_ptr(), kind, device_index)

@@ -70,6 +70,7 @@ class _Group:
         self.pad_addrs = [pbase + r * SIGNAL_PAD_SIZE for r in range(world_size)]
         # the same addresses as a host array, for entry points that take them by value
         self.buffer_addrs_host = (ctypes.c_uint64 * _lib.MAX_WORLD_SIZE)(*self.buffer_addrs)
+        self.pad_addrs_host = (ctypes.c_uint64 * _lib.MAX_WORLD_SIZE)(*self.pad_addrs)
         self.buffer_ptrs = torch.tensor(self.buffer_addrs, dtype=torch.int64, device=device)
         self.pad_ptrs = torch.tensor(self.pad_addrs, dtype=torch.int64, device=device)
         self.status = torch.zeros(_lib.STATUS_WORDS, dtype=torch.int32, device=device)
@@ -105,6 +106,11 @@ class EmulatedSymmetricMemory:
     def buffer_ptrs_host(self):
         """ctypes array of the ranks' buffer addresses in host memory."""
         return self._group.buffer_addrs_host
+
+    @property
+    def signal_pad_ptrs_host(self):
+        """ctypes array of the ranks' signal pad addresses in host memory."""
+        return self._group.pad_addrs_host
 
     @property
     def buffer_ptrs(self) -> List[int]:

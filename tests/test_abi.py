@@ -74,6 +74,15 @@ def test_reduce_argument_errors_before_launch(lib):
     assert b"16-byte aligned" in lib.smr_last_error_string()
     addrs[5] = 0
     assert by_value(addrs, p, p, 16, 0, 0, 8, 0, 0, None, None) == -1
+    # the signal pads come from a host array too, and are only looked at when there is a handshake
+    addrs[5] = 0x60000
+    pads = (ctypes.c_uint64 * 8)(*[0x100000 * (r + 1) for r in range(8)])
+    assert by_value(addrs, None, p, 16, 0, 0, 8, 0, 1, None, None) == -1
+    assert b"signal pads" in lib.smr_last_error_string()
+    pads[3] = 0
+    assert by_value(addrs, pads, p, 16, 0, 0, 8, 0, 1, None, None) == -1
+    assert b"signal pad addresses" in lib.smr_last_error_string()
+    assert by_value(addrs, pads, p, 0, 0, 0, 8, 0, 1, None, None) == -1        # checked before the empty-message shortcut
 
 
 def test_barrier_argument_errors(lib):

@@ -20,39 +20,55 @@ def _covers_exactly(s, M, N):
     """The tiles are disjoint rectangles whose union is the whole output."""
     cells = set()
     for t in s:
-        assert t["row0"] % 128 == 0 and t["col0"] % 64 == 0
+        assert t["row0"] % 128 == 0 and t["col0"] % 32 == 0
         for r in range(t["row0"], t["row0"] + t["rows"], 128):
-            for c in range(t["col0"], min(t["col0"] + t["cols"], (N + 63) // 64 * 64), 64):
+            for c in range(t["col0"], min(t["col0"] + t["cols"], (N + 31) // 32 * 32), 32):
                 assert (r, c) not in cells, "tile overlap"
                 cells.add((r, c))
-    assert len(cells) == (M // 128) * ((N + 63) // 64)
+    assert len(cells) == (M // 128) * ((N + 31) // 32)
 
 
 @pytest.mark.parametrize("rank", [0, 3, 7])
-def test_schedule_config5_ungated(rank):
+@pytest.mark.parametrize("gated", [0, 2], ids=["ungated", "gated-whole-gpu"])
+def test_schedule_config5_whole_gpu(lib, rank, gated):
+    """A launch that has every compute unit (ungated, or gated by somebody who needs none):
+    256x224 tiles, 64 x 16 = 1024 of them = 4 whole passes of 256 workgroups, where 256x256
+    tiles are 896 = 4 passes of 224."""
     M, N, K, ws = 16384, 3584, 8192, 8
-    s = gemm_schedule(M, N, K, rank, ws, M // ws, gated=False)
-    assert len(s) == 64 * 14
-    assert {(t["rows"], t["cols"]) for t in s} == {(256, 256)}
+    assert lib.smr_ag_matmul_grid(M, N, K, ws, M // ws, gated) == 256
+    s = gemm_schedule(M, N, K, rank, ws, M // ws, gated=gated)
+    assert len(s) == 64 * 16
+    assert {(t["rows"], t["cols"]) for t in s} == {(256, 224)}
     _covers_exactly(s, M, N)
     for t in s:
         assert t["comm_block"] == t["row0"] // 2048
         assert t["local"] == int(t["comm_block"] == rank)                  # only local tiles skip the wait
     by = _by_wg(s)
-    # 896 tiles finish in 4 passes on 224 workgroups as on 256
-    assert len(by) == 224 and all(len(v) == 4 for v in by.values())
+    assert len(by) == 256 and all(len(v) == 4 for v in by.values())
     for wg, tiles in by.items():
         assert [t["step"] for t in tiles] == list(range(len(tiles)))
         ring = [(t["comm_block"] - rank) % ws for t in tiles]
         assert ring == sorted(ring)                                        # ready order of the gather
     first = [t for t in s if t["step"] == 0]
-    assert sum(t["local"] for t in first) == 8 * 14
-    # XCD locality: the 28 tiles an XCD holds in the first pass share few A/B slabs
+    assert sum(t["local"] for t in first) == 8 * 16
+    # XCD locality: the 32 tiles an XCD holds in the first pass share few A/B slabs
     for x in range(8):
         mine = [t for t in first if t["wg"] % 8 == x]
-        assert len(mine) == 28
+        assert len(mine) == 32
         slabs = len({t["row0"] for t in mine}) + len({t["col0"] for t in mine})
-        assert slabs <= 20                                                 # 56 when unrelated
+        assert slabs <= 20                                                 # 64 when unrelated
+
+
+def test_schedule_config5_on_the_gated_grid(lib):
+    """The same problem held to the gated launch's 224 workgroups (the grid limit): 256x256 tiles."""
+    M, N, K, ws = 16384, 3584, 8192, 8
+    try:
+        assert lib.smr_set_ag_matmul_grid_limit(224) == 0
+        s = gemm_schedule(M, N, K, 0, ws, M // ws, gated=0)
+    finally:
+        lib.smr_set_ag_matmul_grid_limit(0)
+    assert len(s) == 64 * 14 and {(t["rows"], t["cols"]) for t in s} == {(256, 256)}
+    assert len(_by_wg(s)) == 224
 
 
 @pytest.mark.parametrize("rank", [0, 3, 7])

@@ -409,7 +409,7 @@ def test_gemm_waits_for_flags(cuda, lib):
     lib.smr_set_spin_timeout_us(500)
     try:
         rc = lib.smr_ag_matmul(a_shard.data_ptr(), a_out.data_ptr(), b.data_ptr(), c_out.data_ptr(),
-                               progress.data_ptr(), M, N, K, 0, ws, M // ws, h.status.data_ptr(),
+                               progress.data_ptr(), M, N, K, 0, ws, M // ws, 0, h.status.data_ptr(),
                                torch.cuda.current_stream().cuda_stream)
         assert rc == 0
         with pytest.raises(_lib.SmrError, match="wait_signal timed out"):

@@ -121,7 +121,7 @@ def _ungated_bits(lib, kind, a_shard, h, shards, b, M, N, K, ws, rank, splits, c
     a_ref = kind.to_t(np.concatenate(shards)).to(cuda)
     c_ref = torch.zeros(M * N * kind.elem, dtype=torch.uint8, device=cuda).view(kind.dtype).view(M, N)
     rc = _gemm_entry(lib, kind)(a_shard.data_ptr(), a_ref.data_ptr(), b.data_ptr(), c_ref.data_ptr(), None, M, N, K,
-                                rank, ws, M // ws // splits, h.status.data_ptr(),
+                                rank, ws, M // ws // splits, 0, h.status.data_ptr(),
                                 torch.cuda.current_stream(cuda).cuda_stream)
     assert rc == 0, lib.smr_last_error_string()
     h.check_status()
@@ -151,7 +151,7 @@ def test_gated_gemm_behind_the_stand_alone_producer(cuda, lib, acquire_mode, kin
                                           rank, ws, (M // ws) * K * kind.elem, splits, 16, st)
     assert rc == 0, lib.smr_last_error_string()
     rc = _gemm_entry(lib, kind)(a_shard.data_ptr(), a_out.data_ptr(), b.data_ptr(), c_out.data_ptr(),
-                                progress.data_ptr(), M, N, K, rank, ws, M // ws // splits, h.status.data_ptr(), st)
+                                progress.data_ptr(), M, N, K, rank, ws, M // ws // splits, 0, h.status.data_ptr(), st)
     assert rc == 0, lib.smr_last_error_string()
     h.check_status()
     assert progress.cpu().tolist() == [1] * chunks
@@ -161,15 +161,19 @@ def test_gated_gemm_behind_the_stand_alone_producer(cuda, lib, acquire_mode, kin
     kind.check(got, kind.ref(shards, b_bits))
 
 
+@pytest.mark.parametrize("beside", [False, True], ids=["producer-on-its-own-CUs", "producer-beside-the-GEMM"])
 @pytest.mark.parametrize("kind_name,M,N,K,rank,splits", [
     ("bf16", 8192, 1024, 1024, 0, 1), ("bf16", 8192, 1024, 1024, 5, 2),
     ("e4m3fn", 8192, 1024, 1024, 5, 1), ("e4m3fn", 8192, 1280, 512, 0, 2),
     ("bf16", 16384, 3584, 8192, 0, 1),            # the full-size problem
 ])
-def test_gated_gemm_beside_the_producer_on_another_stream(cuda, lib, acquire_mode, kind_name, M, N, K, rank, splits):
+def test_gated_gemm_beside_the_producer_on_another_stream(cuda, lib, acquire_mode, beside, kind_name, M, N, K, rank, splits):
     """The reference's choreography through the C ABI: progress zeroed, the producer on a side
-    stream, smr_ag_matmul(progress) on the current stream, join.  The GEMM's grid leaves compute
-    units free for the producer, so the two run side by side whichever is dispatched first."""
+    stream, smr_ag_matmul(progress) on the current stream, join.  Either the GEMM's grid leaves
+    compute units free for the producer (smr_all_gather_with_progress, whole_gpu = 0), or the
+    producer's workgroups fit beside the GEMM's on the same compute units and the GEMM takes
+    them all (smr_all_gather_beside, whole_gpu = 1); the two kernels run side by side whichever
+    is dispatched first."""
     import ctypes
     kind, ws = KINDS[kind_name], 8
     a_shard, h, shards, b, b_bits, a_out, c_out = _setup(kind, M, N, K, ws, rank, cuda)
@@ -184,13 +188,14 @@ def test_gated_gemm_beside_the_producer_on_another_stream(cuda, lib, acquire_mod
     side = torch.cuda.Stream(cuda)
     side.wait_stream(current)
     print(f"producer beside gated GEMM: {kind_name} M {M} N {N} K {K} rank {rank} splits {splits} "
-          f"acquire {acquire_mode} grid {plan[0]} + {plan[1]}", flush=True)
-    rc = lib.smr_all_gather_with_progress(h.buffer_ptrs_dev, a_out.data_ptr(), progress.data_ptr(), counters.data_ptr(),
-                                          rank, ws, (M // ws) * K * kind.elem, splits, plan[1], side.cuda_stream)
+          f"acquire {acquire_mode} beside {beside} grid {plan[0]} + {plan[1]}", flush=True)
+    producer = lib.smr_all_gather_beside if beside else lib.smr_all_gather_with_progress
+    rc = producer(h.buffer_ptrs_dev, a_out.data_ptr(), progress.data_ptr(), counters.data_ptr(),
+                  rank, ws, (M // ws) * K * kind.elem, splits, 0 if beside else plan[1], side.cuda_stream)
     assert rc == 0, lib.smr_last_error_string()
     rc = _gemm_entry(lib, kind)(a_shard.data_ptr(), a_out.data_ptr(), b.data_ptr(), c_out.data_ptr(),
-                                progress.data_ptr(), M, N, K, rank, ws, M // ws // splits, h.status.data_ptr(),
-                                current.cuda_stream)
+                                progress.data_ptr(), M, N, K, rank, ws, M // ws // splits, int(beside),
+                                h.status.data_ptr(), current.cuda_stream)
     assert rc == 0, lib.smr_last_error_string()
     current.wait_stream(side)
     h.check_status()
@@ -234,7 +239,7 @@ def test_flags_raised_one_by_one_with_stream_write_value32(cuda, lib, acquire_mo
                 out_chunks[idx].copy_(src[split * rows:(split + 1) * rows])
                 h.stream_write_value32(progress.data_ptr() + idx * progress.element_size(), 1)
     rc = lib.smr_ag_matmul(a_shard.data_ptr(), a_out.data_ptr(), b.data_ptr(), c_out.data_ptr(), progress.data_ptr(),
-                           M, N, K, rank, ws, rows, h.status.data_ptr(), current.cuda_stream)
+                           M, N, K, rank, ws, rows, 0, h.status.data_ptr(), current.cuda_stream)
     assert rc == 0, lib.smr_last_error_string()
     current.wait_stream(backend)
     h.check_status()

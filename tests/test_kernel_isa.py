@@ -59,7 +59,7 @@ def _k_loops(lines):
 
 
 @pytest.mark.parametrize("key", [(256, 256, False), (256, 256, True), (256, 128, False), (128, 128, False),
-                                 (256, 128, True), (128, 128, True)])
+                                 (256, 128, True), (128, 128, True), (256, 224, False)])
 def test_k_loop_keeps_its_registers(kernels, key):
     assert key in kernels, sorted(kernels)
     loops = _k_loops(kernels[key])
@@ -69,7 +69,7 @@ def test_k_loop_keeps_its_registers(kernels, key):
     for body in loops:
         text = "\n".join(body)
         mfma = len(re.findall(r"v_mfma_", text))
-        assert mfma in (4, 8, 16, 32, 64, 128), mfma             # whole slab pairs (full or half-width tile)
+        assert mfma in (4, 8, 16, 32, 64, 112, 128), mfma        # whole slab pairs (112: the 256x224 tile)
         assert "scratch_" not in text, "spill inside the K loop"
         assert "v_accvgpr" not in text, "accumulators moved between register files inside the K loop"
         assert "lane_b32" not in text, "scalar registers spilled inside the K loop"
@@ -142,6 +142,35 @@ def test_fp8_saturation_mode_surrounds_the_conversions_only(kernels, key):
     assert not on and windows >= 1 and conversions >= 16
 
 
-@pytest.mark.parametrize("key", [(256, 256, False), (256, 128, False), (128, 128, False)])
+@pytest.mark.parametrize("key", [(256, 256, False), (256, 224, False), (256, 128, False), (128, 128, False)])
 def test_bf16_kernels_never_touch_the_mode_register(kernels, key):
     assert not any("s_setreg" in ln.split(";")[0] for ln in kernels[key])
+
+
+def _register_counts(asm):
+    """kernel name -> registers per lane a wave of it occupies (.vgpr_count of the metadata: vector
+    plus accumulation registers, as allocated)."""
+    out = {}
+    for m in re.finditer(r"\.name:\s+(\S+)\n(?:.*\n)*?\s+\.vgpr_count:\s+(\d+)", asm):
+        out[m.group(1)] = int(m.group(2))
+    return out
+
+
+def test_producer_fits_beside_the_gemm(gemm_asm, tmp_path):
+    """smr_all_gather_beside promises workgroups that the hardware can place on a compute unit a
+    GEMM workgroup already fills: one wave per SIMD, no LDS, and few enough registers that a
+    GEMM wave and a producer wave fit a SIMD's 512 registers per lane together (allocation is
+    in steps of 8).  True for every bf16 tile and the narrower e4m3fn ones; the 256x256 e4m3fn
+    tile takes every register, which the header says."""
+    gather_asm = _compile(os.path.join(os.path.dirname(SRC), "all_gather.hip"), tmp_path / "all_gather.s")
+    producer = [v for k, v in _register_counts(gather_asm).items() if "all_gather_kernelILi256E" in k]
+    assert len(producer) == 1
+    slim = (producer[0] + 7) // 8 * 8
+    gemm = {k: v for k, v in _register_counts(gemm_asm).items() if "ag_matmul_kernel" in k}
+    assert len(gemm) == 7
+    for name, regs in gemm.items():
+        fits = (regs + 7) // 8 * 8 + slim <= 512
+        if "ILi256ELi256ELb1E" in name:
+            assert not fits, "the header's exception no longer holds: update include/smr.h"
+        else:
+            assert fits, (name, regs, slim)
