@@ -406,9 +406,21 @@ def bench_barrier(dev):
     h.check_status()
     assert int(mism.item()) == 0, "signal-round checksum mismatch"
     SM.release()
+    # One rank's real share: on eight GPUs each runs its own 304 workgroups; the emulation runs
+    # all 8 x 304 on one, and the cache write-back and invalidate of an ordered round are served
+    # one after the other per XCD, so their cost grows with the workgroups that ask for them.
+    # 304 workgroups of a single rank (each handshakes with itself) pay what one GPU would.
+    t1 = SM.empty_strided_p2p((1024,), (1,), torch.int32, dev, world_size=1)
+    h1 = SM.rendezvous(t1)
+    us_one_rank = _time_events(lambda: blockwise_barrier(h1, blocks, 2000), 3, 1) / 2000
+    us_one_rank_flags = _time_events(lambda: blockwise_barrier(h1, blocks, 2000, order_memory=False), 3, 1) / 2000
+    h1.check_status()
+    SM.release()
     written = WS * blocks * chunk
     return dict(workgroups=WS * blocks, rounds_flags=rounds, us_per_round_flags=us_flags,
                 us_per_round_flags_no_cache_maintenance=us_flags_only,
+                one_rank_share={"workgroups": blocks, "us_per_round_flags": us_one_rank,
+                                "us_per_round_flags_no_cache_maintenance": us_one_rank_flags},
                 rounds_payload=prounds, us_per_round_payload=us_payload,
                 payload_written_mib=written / 2 ** 20, payload_read_mib=WS * written / 2 ** 20,
                 payload_gbs=(written + WS * written) / us_payload / 1e3)
