@@ -194,7 +194,6 @@ __global__ __launch_bounds__(kReduceMaxThreads) void one_shot_all_reduce_kernel(
     }
   }
 
-  // the peers' buffers were written by earlier kernels: nothing of this kernel to publish
   // The peers' buffers were written by earlier kernels: nothing of this kernel to publish.
   // And nothing to invalidate: a launch starts from invalidated caches, and no workgroup reads
   // a peer's line before its own handshake (a line is never shared by two blocks: a block's
