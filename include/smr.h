@@ -77,7 +77,8 @@ int smr_set_spin_timeout_us(int64_t us);
  * GPU's 100 MHz constant clock.  Words 0..62: time progress flag i was raised,
  * word 63: producer start.  Words 64 + (workgroup*16 + step)*4 + k: GEMM
  * workgroup's step-th tile, k = 0 tile picked (step 0: kernel entry), 1 flag wait
- * over (step 0: the pull of the first chunk included), 2 K loop done, 3 tile stored.  Needs 64 + 256*16*4 words for the GEMM part.  The reference's
+ * over (in a fused launch: the workgroup's copying at the chunk included), 2 K loop
+ * done, 3 tile stored.  Needs 64 + 256*16*4 words for the GEMM part.  The reference's
  * counterpart is its profiler hook (symm_mem_recipes/utils.py:41-52). */
 int smr_set_trace_buffer(uint64_t* trace_dev, int64_t words);
 int64_t smr_get_spin_timeout_us(void);
@@ -240,8 +241,9 @@ int smr_ag_matmul_schedule(int M, int N, int K, int rank, int world_size, int co
  * producer is a copy engine and costs no SMs; on one GPU the copy runs on compute units, and
  * here it runs inside the GEMM's own grid:
  *   - `producer_workgroups` extra workgroups (0 = the plan's, see smr_ag_matmul_plan; never
- *     fewer than one: the local shard reaches a_out through them) only copy: the peers' shards from buffer_ptrs_dev into a_out in the reference's order
- *     (sources rank+1, ..., rank+ws-1, rank; :43-44), in 64 KiB pieces taken by ticket;
+ *     fewer than one: the local shard reaches a_out through them) only copy: the peers'
+ *     shards from buffer_ptrs_dev into a_out in the reference's order (sources rank+1, ...,
+ *     rank+ws-1, rank; :43-44), in 64 KiB pieces taken by ticket;
  *   - a GEMM workgroup whose next tile's chunk is not in place takes pieces of that chunk
  *     too instead of spinning, so the launch finishes whichever of its workgroups are
  *     resident, and needs no second stream and no kernel running beside it;
