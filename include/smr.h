@@ -36,7 +36,7 @@
 extern "C" {
 #endif
 
-#define SMR_VERSION 110
+#define SMR_VERSION 111
 
 #define SMR_DTYPE_BF16 0
 #define SMR_DTYPE_FP32 1
@@ -216,14 +216,32 @@ int smr_ag_matmul(const void* a_shard_dev, const void* a_out_dev, const void* b_
  * no LDS, which the hardware places beside the GEMM's workgroups on the same compute units (a
  * bf16 GEMM workgroup leaves at least 88 of a SIMD's 512 registers per lane).  The GEMM it
  * feeds is launched with whole_gpu = 1.  The first rank's chunks - the ones half of the GEMM's
- * workgroups wait for at the start - are copied at full speed, the others a little at a time:
- * the GEMM needs a chunk per pass, and a copy that runs flat out beside it slows it down.
+ * workgroups wait for at the start - are copied at full speed, the others on a timetable when
+ * the caller gives one (step_us, lead_ranks): the GEMM needs a rank's chunks per world_size-th
+ * of its run, and a copy that runs flat out beside it slows it down.
  * Exception: the 256x256 tile of smr_ag_matmul_fp8 takes every register of its compute unit,
  * so nothing fits beside it - with that GEMM use smr_all_gather_with_progress and whole_gpu = 0.
- *   num_workgroups  0 = one per compute unit of a 256-CU part */
+ *   num_workgroups  0 = one per compute unit of a 256-CU part
+ *   step_us, lead_ranks  the timetable (smr_ag_matmul_pace gives both for a GEMM).  The ranks at
+ *                   ring positions 1 .. lead_ranks-1 (1 = the next rank) are copied flat out: the
+ *                   GEMM's first pass waits for them.  The rank at position r >= lead_ranks is
+ *                   spread over [r - lead_ranks, r - lead_ranks + 1) * step_us from the kernel's
+ *                   start, less a margin of an eighth; a producer that is behind its timetable
+ *                   copies flat out.  step_us = 0: no timetable, everything flat out - right for a
+ *                   GEMM that is shorter than the copy, 2 % slower for the M=16384 N=3584 K=8192 one. */
 int smr_all_gather_beside(const uint64_t* buffer_ptrs_dev, void* a_out_dev, uint32_t* progress_dev,
                           uint32_t* counters_dev, int rank, int world_size, int64_t shard_bytes,
-                          int splits_per_rank, int num_workgroups, void* stream);
+                          int splits_per_rank, int num_workgroups, int64_t step_us, int lead_ranks,
+                          void* stream);
+
+/* Host-only: the timetable on which a gated smr_ag_matmul (elem_bytes 2) or smr_ag_matmul_fp8 (1)
+ * with whole_gpu = 1 needs its chunks on the current device.  out2 = {step_us, lead_ranks} for
+ * smr_all_gather_beside: a world_size-th of the planner's estimate of the GEMM's time, and the
+ * number of ranks whose tiles the first pass of the persistent grid touches (the local one
+ * included).  {0, world_size} for a GEMM of a single pass, which needs everything at once.
+ * Negative SMR_E_* for shapes the GEMM refuses.  No reference counterpart (its copy engines
+ * run flat out and disturb nobody, triton_all_gather_matmul.py:46-55). */
+int smr_ag_matmul_pace(int M, int N, int K, int world_size, int comm_block_m, int elem_bytes, int32_t* out2);
 
 /* Host-only: the tile order smr_ag_matmul uses on a 256-CU part.  Writes up to
  * max_tiles records of 8 int32 (workgroup, step, row0, col0, tile rows, tile

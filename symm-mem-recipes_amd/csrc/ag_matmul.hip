@@ -1108,7 +1108,7 @@ struct FusedEstimate {
 constexpr int kMaxProducerWgs = 128;
 constexpr double kCopyOnlyBytesPerUs = 25.0e3, kWaiterBytesPerUs = 12.0e3, kWaitShows = 0.6, kFusedFixedUs = 18.0;
 static double model_tile_us(int BM, int BN, int K, int elem_bytes, bool beside_copy) {
-  double rate = BM == 256 && BN == 256 ? (beside_copy ? 6.5e6 : 6.6e6) : 4.6e6;      // FLOP per us
+  double rate = BM == 256 && BN >= 224 ? (beside_copy ? 6.5e6 : 6.6e6) : 4.6e6;      // FLOP per us
   if (elem_bytes == 1) rate = BM == 256 && BN == 256 ? (beside_copy ? 14.2e6 : 14.0e6) : 9.2e6;
   return 2.0 * BM * BN * K / rate + 6.0;
 }
@@ -1379,6 +1379,19 @@ int smr_set_ag_matmul_grid_limit(int workgroups) {
   return 0;
 }
 
+// The model's time for the ungated GEMM with the whole GPU: passes of the grid times a tile.
+static double model_ungated_us(int M, int N, int K, int world_size, int comm_block_m, int elem_bytes) {
+  using namespace smr;
+  const GemmSchedule u = make_schedule(M, N, K, 0, world_size, comm_block_m, cu_count(), kUngated, elem_bytes);
+  const int tiles = (M / u.BM) * ceil_div(N, u.BN);
+  // (fitted with the rest of the model: a last pass that fills at most half of the grid counts as half a pass)
+  const double passes = ceil_div(2 * tiles, u.grid) * 0.5;
+  // (the tile model is that of a launch which leaves compute units idle; with all of them busy
+  // the part settles at a lower clock: a workgroup's rate drops by 6 %)
+  const double clock = u.grid > cu_count() - kReservedCus ? 0.94 : 1.0;
+  return passes * ((model_tile_us(u.BM, u.BN, K, elem_bytes, false) - 6.0) / clock + 6.0);
+}
+
 // Fills the plan of a fused launch: {GEMM grid, producer workgroups, estimated
 // microseconds fused, estimated microseconds copy-then-multiply, sequential}.
 static void fill_plan(int M, int N, int K, int world_size, int comm_block_m, int elem_bytes, int32_t* out5) {
@@ -1388,14 +1401,9 @@ static void fill_plan(int M, int N, int K, int world_size, int comm_block_m, int
   const FusedEstimate e = estimate_fused(s, cus, s.grid, elem_bytes);
   // The alternative for a problem too small to hide the copy behind: copy with the
   // whole GPU, then multiply with the whole GPU.
-  const GemmSchedule u = make_schedule(M, N, K, 0, world_size, comm_block_m, cus, kUngated, elem_bytes);
-  const double tile_us = model_tile_us(u.BM, u.BN, K, elem_bytes, false);
-  const int tiles = (M / u.BM) * ceil_div(N, u.BN);
-  // (fitted with the rest of the model: a last pass that fills at most half of the grid counts as half a pass)
-  const double passes = ceil_div(2 * tiles, u.grid) * 0.5;
   // (all chunks at once, the own shard included: read + write at what a copy reaches on the part)
-  const double gather_us = 2.0 * elem_bytes * M * K / 5.4e6 + 4.0;
-  const double seq_us = gather_us + passes * tile_us + 10.0;
+  const double gather_us = 2.0 * elem_bytes * M * K / 4.8e6 + 4.0;
+  const double seq_us = gather_us + model_ungated_us(M, N, K, world_size, comm_block_m, elem_bytes) + 10.0;
   out5[0] = s.grid;
   out5[1] = e.producer_wgs;
   out5[2] = (int32_t)(e.total_us + 0.5);
@@ -1409,6 +1417,28 @@ int smr_ag_matmul_plan(int M, int N, int K, int world_size, int comm_block_m, in
   if (int rc = validate(M, N, K, 0, world_size, comm_block_m, &why)) return fail(rc, why);
   if (out5 == nullptr) return fail(SMR_E_INVALID, "smr_ag_matmul_plan: out5 is NULL");
   fill_plan(M, N, K, world_size, comm_block_m, 2, out5);
+  return 0;
+}
+
+int smr_ag_matmul_pace(int M, int N, int K, int world_size, int comm_block_m, int elem_bytes, int32_t* out2) {
+  using namespace smr;
+  const char* why;
+  if (elem_bytes != 1 && elem_bytes != 2) return fail(SMR_E_INVALID, "smr_ag_matmul_pace: elem_bytes must be 1 or 2");
+  if (int rc = elem_bytes == 1 ? validate_fp8(M, N, K, 0, world_size, comm_block_m, &why)
+                               : validate(M, N, K, 0, world_size, comm_block_m, &why))
+    return fail(rc, why);
+  if (out2 == nullptr) return fail(SMR_E_INVALID, "smr_ag_matmul_pace: out2 is NULL");
+  // the launch a producer without compute units of its own feeds: gated, the whole GPU
+  const GemmSchedule g = make_schedule(M, N, K, 0, world_size, comm_block_m, cu_count(), kGatedWhole, elem_bytes);
+  const int per_rank = (M / world_size / g.BM) * ceil_div(N, g.BN);       // tiles of one rank's rows
+  const int passes = ceil_div(per_rank * world_size, g.grid);
+  if (passes <= 1) {                                  // every tile starts at once: nothing to spread
+    out2[0] = 0;
+    out2[1] = world_size;
+    return 0;
+  }
+  out2[0] = (int32_t)(model_ungated_us(M, N, K, world_size, comm_block_m, elem_bytes) / world_size + 0.5);
+  out2[1] = ceil_div(g.grid, per_rank);               // ranks whose tiles the first pass touches
   return 0;
 }
 

@@ -36,60 +36,95 @@ typedef __attribute__((address_space(1))) u32x4 GlobalVec;
 __device__ __forceinline__ void store_through(GlobalVec* p, u32x4 v) {
   asm volatile("global_store_dwordx4 %0, %1, off sc1\n\ts_nop 1" : : "v"(p), "v"(v) : "memory");
 }
+// The same with the address as a uniform base and a 32-bit byte offset per lane.
+__device__ __forceinline__ void store_through(uint8_t* base, uint32_t offset, u32x4 v) {
+  asm volatile("global_store_dwordx4 %0, %1, %2 sc1\n\ts_nop 1" : : "v"(offset), "v"(v), "s"(base) : "memory");
+}
+
+// The timetable of a producer that copies beside the GEMM it feeds, in ticks of the 100 MHz
+// clock (worked out on the host: a 64-bit division costs the kernel thirty registers, and its
+// workgroups have to fit beside the GEMM's).  step = 0: none.
+struct Timetable {
+  uint64_t step;       // from one rank's chunks to the next rank's (margin taken off)
+  uint64_t window;     // one chunk's share of a step
+  uint64_t per_trip;   // one trip's (two loads per thread) share of a window
+  int lead_ranks;      // ring positions below this one are copied flat out
+};
 
 // THREADS = 1024: a workgroup fills a compute unit (the producer beside a GEMM that leaves
 // compute units free).  THREADS = 256: one wave per SIMD with a few dozen registers and no LDS -
 // a workgroup that fits BESIDE a workgroup of the GEMM on the same compute unit (the GEMM's
 // waves hold 424 of a SIMD's 512 registers per lane), so the copy needs no compute units of its
-// own, like the copy engines it stands in for.  That form copies the first rank's chunks - the
-// ones half of the GEMM's workgroups wait for - as fast as it can and the others two loads per
-// thread at a time: the GEMM needs a chunk per pass, not as fast as memory can deliver it.
+// own, like the copy engines it stands in for.  That form can copy on a timetable: a persistent
+// GEMM takes its tiles in ring order, one pass of its grid after the other, so the chunks of the
+// ranks whose tiles the first pass holds are due at once and are copied as fast as memory
+// delivers them, and every later rank's are due one rank's share of the GEMM's time after
+// the rank before it - they are copied two loads per thread at a time, each trip at its time.
+// Not as fast as possible, because a copy that runs flat out on the compute unit of a GEMM
+// workgroup slows that workgroup down (M=16384 N=3584 K=8192: the GEMM ends 2 % later).
 template <int THREADS>
 __global__ __launch_bounds__(THREADS) void all_gather_kernel(
     const uint64_t* __restrict__ buffer_ptrs, uint8_t* __restrict__ a_out,
     uint32_t* __restrict__ progress, uint32_t* __restrict__ counters, int rank, int world_size,
-    int64_t chunk_vecs, int splits_per_rank, uint64_t* trace) {
+    int64_t chunk_vecs, int splits_per_rank, Timetable tt, uint64_t* trace) {
   constexpr int kGatherThreads = THREADS;
   if (trace != nullptr && blockIdx.x == 0 && threadIdx.x == 0) trace[kTraceProducerWords - 1] = wall_clock64();
-  int done_chunks = 0;
+  const uint64_t t_entry = tt.step != 0 ? wall_clock64() : 0;
   for (int step = 0; step < world_size; ++step) {
     const int src_rank = (rank + step + 1) % world_size;
     for (int split = 0; split < splits_per_rank; ++split) {
       const int idx = src_rank * splits_per_rank + split;
       const int nwg = (int)gridDim.x;
-      // (beside a GEMM: the first rank's chunks at full speed, the others two loads at a time -
-      // a burst of loads and stores fills the compute unit's memory pipeline, which the GEMM
-      // workgroup on the same compute unit feeds its tiles through)
-      const bool trickle = THREADS == 256 && done_chunks++ >= splits_per_rank;
-      const GlobalVec* src =
-          (const GlobalVec*)(uintptr_t)buffer_ptrs[src_rank] + (int64_t)split * chunk_vecs;
-      GlobalVec* dst = (GlobalVec*)(uintptr_t)a_out + (int64_t)idx * chunk_vecs;
+      // (ring position of the source: 1 for the next rank, ..., world_size for the own shard)
+      const bool trickle = THREADS == 256 && tt.step != 0 && step + 1 >= tt.lead_ranks;
+      // Addresses as a uniform base and a 32-bit byte offset per lane (the host keeps a chunk
+      // below 2 GiB): one register per slot in flight instead of four, which is what lets
+      // the slim form's workgroups fit beside the GEMM's.
+      const uint8_t* src = (const uint8_t*)(uintptr_t)buffer_ptrs[src_rank] + (int64_t)split * chunk_vecs * 16;
+      uint8_t* dst = a_out + (int64_t)idx * chunk_vecs * 16;
+      const uint32_t chunk_bytes = (uint32_t)chunk_vecs * 16u;
       // 8 independent 16-byte slots per thread per trip: 128 KiB in flight per
       // workgroup, which is what one compute unit needs to stream at its share
-      const int64_t stride = (int64_t)nwg * kGatherThreads;
-      int64_t i = (int64_t)blockIdx.x * kGatherThreads + threadIdx.x;
+      const uint32_t stride = (uint32_t)nwg * kGatherThreads * 16u;
+      uint32_t i = ((uint32_t)blockIdx.x * kGatherThreads + threadIdx.x) * 16u;
+      auto load = [&](uint32_t off) { return __builtin_nontemporal_load((const GlobalVec*)(uintptr_t)(src + off)); };
+      auto store = [&](uint32_t off, u32x4 v) { store_through(dst, off, v); };
       if (trickle) {
-        // (pairs with 6000 clocks of sleep in between finish the gather of 7 x 32 MiB in about
-        // 500 us, within the GEMM it feeds; without the sleep the GEMM beside it ran 2 % slower,
-        // single loads or twice the sleep fall behind the GEMM's need)
-        for (; i + stride < chunk_vecs; i += 2 * stride) {
-          const u32x4 v0 = __builtin_nontemporal_load(src + i), v1 = __builtin_nontemporal_load(src + i + stride);
-          store_through(dst + i, v0);
-          store_through(dst + i + stride, v1);
-#pragma unroll
-          for (int z = 0; z < 6; ++z) __builtin_amdgcn_s_sleep(16);
+        // The timetable: the ranks at ring positions below lead_ranks are in the GEMM's first
+        // pass (copied flat out, above); the rank at position r is due a step after the rank
+        // before it, so its chunks are spread over [r - lead_ranks, r - lead_ranks + 1) steps
+        // from the kernel's start (a step is shortened by an eighth as a margin).  A trip whose
+        // time has come already (the first ranks took longer than planned, or the estimate was
+        // short) does not wait, so a producer that is behind copies flat out until it is not.
+        // Two loads per thread and trip: single loads fall behind the GEMM's need at any pace,
+        // and a burst of eight fills the memory pipeline that the GEMM workgroup on the same
+        // compute unit feeds its tiles through.
+        uint64_t due = t_entry + tt.step * (uint64_t)(step + 1 - tt.lead_ranks) + tt.window * (uint64_t)split;
+        for (; i + stride < chunk_bytes; i += 2 * stride) {
+          while (wall_clock64() < due) __builtin_amdgcn_s_sleep(8);     // (ends: the clock runs, `due` does not)
+          due += tt.per_trip;
+          const u32x4 v0 = load(i), v1 = load(i + stride);
+          store(i, v0);
+          store(i + stride, v1);
         }
       }
-      for (; i + 7 * stride < chunk_vecs; i += 8 * stride) {
+      for (; i + 7 * stride < chunk_bytes; i += 8 * stride) {
         u32x4 v[8];
 #pragma unroll
-        for (int u = 0; u < 8; ++u) v[u] = __builtin_nontemporal_load(src + i + u * stride);
+        for (int u = 0; u < 8; ++u) v[u] = load(i + u * stride);
 #pragma unroll
-        for (int u = 0; u < 8; ++u) store_through(dst + i + u * stride, v[u]);
+        for (int u = 0; u < 8; ++u) store(i + u * stride, v[u]);
       }
-      for (; i < chunk_vecs; i += stride) {
-        u32x4 v = __builtin_nontemporal_load(src + i);
-        store_through(dst + i, v);
+      // what is left of the chunk (all of a small one): up to four slots in flight together too -
+      // one after the other they were as many trips to memory and back per chunk
+      for (; i < chunk_bytes; i += 4 * stride) {
+        u32x4 v[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+          if (i + u * stride < chunk_bytes) v[u] = load(i + u * stride);
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+          if (i + u * stride < chunk_bytes) store(i + u * stride, v[u]);
       }
       // publish: the stores went through to where every XCD sees them, so a thread
       // only has to wait for their acknowledgement - no cache-wide write-back, which
@@ -158,7 +193,7 @@ __global__ __launch_bounds__(kGatherThreads) void all_gather_at_once_kernel(
 static int launch_gather(const uint64_t* buffer_ptrs_dev, void* a_out_dev, uint32_t* progress_dev,
                          uint32_t* counters_dev, int rank, int world_size, int64_t shard_bytes,
                          int splits_per_rank, int num_workgroups, void* stream, bool at_once,
-                         bool beside = false) {
+                         bool beside = false, int64_t step_us = 0, int lead_ranks = 0) {
   using namespace smr;
   if (buffer_ptrs_dev == nullptr || a_out_dev == nullptr || progress_dev == nullptr ||
       counters_dev == nullptr)
@@ -170,9 +205,20 @@ static int launch_gather(const uint64_t* buffer_ptrs_dev, void* a_out_dev, uint3
   const int64_t chunk_bytes = shard_bytes / splits_per_rank;
   if (chunk_bytes % 16 != 0 || (reinterpret_cast<uintptr_t>(a_out_dev) & 15u))
     return fail(SMR_E_INVALID, "smr_all_gather_with_progress: chunks must be 16-byte multiples");
+  if (chunk_bytes > ((int64_t)1 << 31) - ((int64_t)1 << 28))       // (32-bit byte offsets, eight strides of slack)
+    return fail(SMR_E_UNSUPPORTED, "smr_all_gather_with_progress: a chunk (shard / splits) beyond 1.75 GiB");
   if (num_workgroups < 0 || num_workgroups > 1024)
     return fail(SMR_E_INVALID, "smr_all_gather_with_progress: num_workgroups must be 0..1024");
+  if (step_us < 0 || step_us > 1000000 || lead_ranks < 0)
+    return fail(SMR_E_INVALID, "smr_all_gather_beside: step_us must be 0..1,000,000 and lead_ranks >= 0");
   const int nwg = num_workgroups == 0 ? (beside ? kBesideDefaultWorkgroups : kGatherDefaultWorkgroups) : num_workgroups;
+  Timetable tt = {0, 0, 0, lead_ranks < 1 ? 1 : lead_ranks};
+  if (beside && step_us > 0) {
+    const int64_t trips = (chunk_bytes / 16 + 2 * (int64_t)nwg * 256 - 1) / (2 * (int64_t)nwg * 256);
+    tt.step = (uint64_t)step_us * 100u * 7 / 8;                 // 100 MHz clock, an eighth of margin
+    tt.window = tt.step / (uint64_t)splits_per_rank;
+    tt.per_trip = tt.window / (uint64_t)(trips > 0 ? trips : 1);
+  }
   if (at_once) {
     hipLaunchKernelGGL(all_gather_at_once_kernel, dim3(nwg), dim3(kGatherThreads), 0,
                        reinterpret_cast<hipStream_t>(stream), buffer_ptrs_dev,
@@ -184,12 +230,12 @@ static int launch_gather(const uint64_t* buffer_ptrs_dev, void* a_out_dev, uint3
     hipLaunchKernelGGL(all_gather_kernel<256>, dim3(nwg), dim3(256), 0,
                        reinterpret_cast<hipStream_t>(stream), buffer_ptrs_dev,
                        reinterpret_cast<uint8_t*>(a_out_dev), progress_dev, counters_dev, rank,
-                       world_size, chunk_bytes / 16, splits_per_rank, trace_buffer(kTraceProducerWords));
+                       world_size, chunk_bytes / 16, splits_per_rank, tt, trace_buffer(kTraceProducerWords));
   else
     hipLaunchKernelGGL(all_gather_kernel<kGatherThreads>, dim3(nwg), dim3(kGatherThreads), 0,
                        reinterpret_cast<hipStream_t>(stream), buffer_ptrs_dev,
                        reinterpret_cast<uint8_t*>(a_out_dev), progress_dev, counters_dev, rank,
-                       world_size, chunk_bytes / 16, splits_per_rank, trace_buffer(kTraceProducerWords));
+                       world_size, chunk_bytes / 16, splits_per_rank, tt, trace_buffer(kTraceProducerWords));
   return check_hip(hipGetLastError(), "smr_all_gather_with_progress launch");
 }
 
@@ -211,7 +257,8 @@ extern "C" int smr_all_gather_at_once(const uint64_t* buffer_ptrs_dev, void* a_o
 
 extern "C" int smr_all_gather_beside(const uint64_t* buffer_ptrs_dev, void* a_out_dev, uint32_t* progress_dev,
                                      uint32_t* counters_dev, int rank, int world_size, int64_t shard_bytes,
-                                     int splits_per_rank, int num_workgroups, void* stream) {
+                                     int splits_per_rank, int num_workgroups, int64_t step_us, int lead_ranks,
+                                     void* stream) {
   return launch_gather(buffer_ptrs_dev, a_out_dev, progress_dev, counters_dev, rank, world_size,
-                       shard_bytes, splits_per_rank, num_workgroups, stream, false, true);
+                       shard_bytes, splits_per_rank, num_workgroups, stream, false, true, step_us, lead_ranks);
 }

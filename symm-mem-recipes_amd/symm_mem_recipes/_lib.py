@@ -49,7 +49,8 @@ SIGNATURES = {
     "smr_signal_round": (_i, [_p, _p, _p, _p, _p, _p, _i, _i, _i64, _i, _p, _p]),
     "smr_all_gather_with_progress": (_i, [_p, _p, _p, _p, _i, _i, _i64, _i, _i, _p]),
     "smr_all_gather_at_once": (_i, [_p, _p, _p, _p, _i, _i, _i64, _i, _i, _p]),
-    "smr_all_gather_beside": (_i, [_p, _p, _p, _p, _i, _i, _i64, _i, _i, _p]),
+    "smr_all_gather_beside": (_i, [_p, _p, _p, _p, _i, _i, _i64, _i, _i, _i64, _i, _p]),
+    "smr_ag_matmul_pace": (_i, [_i, _i, _i, _i, _i, _i, _p]),
     "smr_set_ag_matmul_acquire": (_i, [_i]),
     "smr_ag_matmul_fused": (_i, [_p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _p, _p]),
     "smr_ag_matmul_fused_state_words": (_i, [_i, _i]),

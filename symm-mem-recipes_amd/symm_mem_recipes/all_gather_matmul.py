@@ -166,9 +166,15 @@ def all_gather_matmul_tma_persistent(a_shard: torch.Tensor, b: torch.Tensor, a_o
         beside = not fp8
         producer = lib.smr_all_gather_beside if beside else lib.smr_all_gather_with_progress
         wgs = (0 if beside else int(plan[1])) if producer_workgroups is None else int(producer_workgroups)
-        rc = producer(symm_mem.buffer_ptrs_dev, a_out.data_ptr(), flags.data_ptr(), flags[chunks:].data_ptr(),
-                      rank, world_size, a_shard.numel() * a_shard.element_size(), int(splits_per_rank), wgs,
-                      backend_stream.cuda_stream)
+        args = [symm_mem.buffer_ptrs_dev, a_out.data_ptr(), flags.data_ptr(), flags[chunks:].data_ptr(),
+                rank, world_size, a_shard.numel() * a_shard.element_size(), int(splits_per_rank), wgs]
+        if beside:
+            # its timetable: the first pass's ranks flat out, the others as the GEMM gets to them
+            # (a GEMM shorter than the copy gets everything flat out whatever the estimate says)
+            pace = (ctypes.c_int32 * 2)()
+            _lib.check(lib.smr_ag_matmul_pace(M, N, K, world_size, COMM_BLOCK_SIZE_M, 2, pace), "all_gather_matmul")
+            args += [int(pace[0]), int(pace[1])]
+        rc = producer(*args, backend_stream.cuda_stream)
         _lib.check(rc, "all_gather_with_progress")
         rc = gemm(a_shard.data_ptr(), a_out.data_ptr(), b.data_ptr(), c_out.data_ptr(), flags.data_ptr(), M, N, K,
                   rank, world_size, COMM_BLOCK_SIZE_M, int(beside), status_ptr, current.cuda_stream)

@@ -25,7 +25,7 @@ def test_header_symbols_all_exported(lib):
 
 
 def test_version_and_timeout_roundtrip(lib):
-    assert lib.smr_version() == 110
+    assert lib.smr_version() == 111
     old = lib.smr_get_spin_timeout_us()
     assert old == 2_000_000
     assert lib.smr_set_spin_timeout_us(1234) == 0

@@ -126,7 +126,8 @@ def test_fused_plan_splits_the_gpu(lib):
     import ctypes
     plans = {}
     for (M, N, K) in [(16384, 3584, 8192), (16384, 6656, 16384), (8192, 3584, 8192), (16384, 1792, 4096),
-                      (4096, 8192, 8192), (2048, 4096, 2048), (1024, 256, 256)]:
+                      (4096, 8192, 8192), (2048, 4096, 2048), (1024, 256, 256), (8192, 1792, 4096),
+                      (4096, 3584, 8192)]:
         out = (ctypes.c_int32 * 5)()
         assert lib.smr_ag_matmul_plan(M, N, K, 8, M // 8, out) == 0
         grid, wgs, fused_us, sequential_us, sequential = list(out)
@@ -138,8 +139,10 @@ def test_fused_plan_splits_the_gpu(lib):
         plans[(M, N, K)] = (grid, wgs, sequential)
     # (the choices below are the ones launches timed on MI355X bear out)
     assert plans[(16384, 3584, 8192)] == (224, 32, 0)
-    assert plans[(8192, 3584, 8192)][2] == 0
+    assert plans[(16384, 6656, 16384)][2] == 0
     assert plans[(4096, 8192, 8192)][2] == 1 and plans[(2048, 4096, 2048)][2] == 1
+    assert plans[(8192, 1792, 4096)][2] == 1 and plans[(4096, 3584, 8192)][2] == 1
+    # ((8192, 3584, 8192) and (16384, 1792, 4096) time within 2 % and 5 % either way: not asserted)
     # a problem with few passes leaves the copy more of the GPU
     assert plans[(2048, 4096, 2048)][1] > plans[(16384, 3584, 8192)][1]
     out = (ctypes.c_int32 * 5)()
@@ -148,6 +151,27 @@ def test_fused_plan_splits_the_gpu(lib):
     assert lib.smr_ag_matmul_plan_fp8(16384, 3584, 8192 + 64, 8, 2048, out) == -2      # K % 128
     assert lib.smr_ag_matmul_plan(1000, 256, 256, 8, 125, out) == -2                   # unsupported shape
     assert lib.smr_ag_matmul_plan(1024, 256, 256, 8, 128, None) == -1
+
+
+def test_timetable_of_a_gated_launch(lib):
+    """smr_ag_matmul_pace, the timetable smr_all_gather_beside is given: a world_size-th of an estimate that is
+    within a fifth of what the ungated launches take on MI355X (256 compute units assumed without a GPU), the
+    ranks of the first pass, nothing to spread for a single pass, and the GEMM's own refusals."""
+    import ctypes
+    out = (ctypes.c_int32 * 2)()
+    measured = {(16384, 3584, 8192): (630, 2), (16384, 1792, 4096): (178, 4), (16384, 7168, 8192): (1250, 2),
+                (8192, 3584, 8192): (323, 4), (16384, 8192, 2048): (406, 1)}
+    for (M, N, K), (us, lead) in measured.items():
+        assert lib.smr_ag_matmul_pace(M, N, K, 8, M // 8, 2, out) == 0
+        assert 0.8 * us <= 8 * out[0] <= 1.2 * us, (M, N, K, list(out), us)
+        assert out[1] == lead, (M, N, K, list(out))
+    assert lib.smr_ag_matmul_pace(4096, 3584, 8192, 8, 512, 2, out) == 0 and list(out) == [0, 8]     # one pass
+    assert lib.smr_ag_matmul_pace(16384, 3584, 8192, 8, 2048, 1, out) == 0
+    assert 0.4 * 630 <= 8 * out[0] <= 0.65 * 630
+    assert lib.smr_ag_matmul_pace(1000, 256, 256, 8, 125, 2, out) == -2
+    assert lib.smr_ag_matmul_pace(16384, 3584, 8192 + 64, 8, 2048, 1, out) == -2
+    assert lib.smr_ag_matmul_pace(1024, 256, 256, 8, 128, 4, out) == -1
+    assert lib.smr_ag_matmul_pace(1024, 256, 256, 8, 128, 2, None) == -1
 
 
 def test_schedule_rejects_bad_shapes():

@@ -190,8 +190,15 @@ def test_gated_gemm_beside_the_producer_on_another_stream(cuda, lib, acquire_mod
     print(f"producer beside gated GEMM: {kind_name} M {M} N {N} K {K} rank {rank} splits {splits} "
           f"acquire {acquire_mode} beside {beside} grid {plan[0]} + {plan[1]}", flush=True)
     producer = lib.smr_all_gather_beside if beside else lib.smr_all_gather_with_progress
+    # (the producer beside the GEMM on the timetable of the planner's estimate, and in the second
+    # parameter set on one four times as long: then it is the GEMM that waits, which must not matter)
+    timetable = []
+    if beside:
+        pace = (ctypes.c_int32 * 2)()
+        assert lib.smr_ag_matmul_pace(M, N, K, ws, M // ws // splits, kind.elem, pace) == 0
+        timetable = [max(pace[0], 10) * 4, 1] if splits == 2 else [pace[0], pace[1]]
     rc = producer(h.buffer_ptrs_dev, a_out.data_ptr(), progress.data_ptr(), counters.data_ptr(),
-                  rank, ws, (M // ws) * K * kind.elem, splits, 0 if beside else plan[1], side.cuda_stream)
+                  rank, ws, (M // ws) * K * kind.elem, splits, 0 if beside else plan[1], *timetable, side.cuda_stream)
     assert rc == 0, lib.smr_last_error_string()
     rc = _gemm_entry(lib, kind)(a_shard.data_ptr(), a_out.data_ptr(), b.data_ptr(), c_out.data_ptr(),
                                 progress.data_ptr(), M, N, K, rank, ws, M // ws // splits, int(beside),
