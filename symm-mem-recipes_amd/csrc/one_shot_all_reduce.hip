@@ -7,12 +7,18 @@
 // bit-identical to a sequential fp32 sum - and stores one 128-bit result.
 // The kernel is bound by HBM bandwidth: (ws + 1) * 16 bytes per slot.
 //
+// The stores are held back: a thread keeps the results of several slots in registers and
+// writes them in one go (8 slots; 64 in the kernel for large messages, which then holds a
+// whole 64 MiB launch's results and stores them at the end).  Memory serves eight read
+// streams at 6.8 TB/s and a write stream at 6.4 TB/s, but reads with a ninth of writes mixed
+// in at 6.0 to 6.3 TB/s: a launch that reads first and writes afterwards pays for the two
+// separately.
+//
 // Role of the workgroups (`layout`):
 //   kPlain     grid = nblocks: one rank's share, no handshake
-//   kProxy     grid = nproxy + nblocks: the first nproxy workgroups play the other
-//              ranks' halves of the handshake (8 lanes per block, no arithmetic)
-//              and are dispatched first, so they are resident and spinning by
-//              the time the rank's own workgroups arrive behind the barrier
+//   kProxy     grid = nblocks: one rank's share behind the handshake; the other ranks'
+//              halves of the handshake, which nobody runs in the one-rank emulation, are
+//              played by spare lanes of the wave that does the rank's own half
 //   kAllRanks  grid = ws*nblocks: workgroup id -> (block = id / ws, rank = id % ws);
 //              every emulated rank reduces into its own row of `out`
 // In kAllRanks adjacent ids hold the partners of one handshake, so in-order
@@ -147,42 +153,72 @@ __device__ __forceinline__ Vec16 sum_in_rank_order(const Vec16 (&v)[WS]) {
   return o;
 }
 
-template <int KIND, int WS, bool WRITE_ALL>
-__global__ __launch_bounds__(kReduceMaxThreads) void one_shot_all_reduce_kernel(
+// blockwise_barrier for the one-rank emulation: the rank's half of block `block_id`'s handshake
+// and, in the same wave and the same loop, the halves of the ws - 1 ranks that nobody runs.
+// Lane = role * ws + peer.  Role 0: the rank sends to `peer` (CAS 0 -> 1 on the peer's pad);
+// 1: the rank waits for `peer` (own pad); 2: `peer` sends to the rank (the rank's pad, the slot
+// role 1 polls); 3: `peer` waits for the rank (the peer's pad, the slot role 0 raised).  One
+// loop for all of them, as in blockwise_barrier: every wait depends on a send of a lane
+// beside it.  `publish` / `acquire` as there.
+template <int WS, typename Pads>
+__device__ __forceinline__ bool barrier_with_stand_ins(const Pads& pads, uint32_t block_id, int rank,
+                                                       uint64_t limit_ticks, uint32_t* status, bool publish,
+                                                       bool acquire) {
+  static_assert(4 * WS <= 64, "one wave plays all four roles");
+  __syncthreads();
+  const int lane = threadIdx.x;
+  int bad = 0;
+  if (lane < 64) {
+    if (publish) __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+    // the consuming write of an earlier call on this slot has been performed
+    else wait_stores_acknowledged();
+    const int role = lane / WS, peer = lane % WS;
+    if (role < 4 && !(role >= 2 && peer == rank)) {
+      const bool is_send = (role & 1) == 0;
+      const bool peers_pad = role == 0 || role == 3;          // else the rank's own pad
+      uint32_t* pad = reinterpret_cast<uint32_t*>(pads[peers_pad ? peer : rank]);
+      uint32_t* slot = pad + (size_t)block_id * WS + (peers_pad ? rank : peer);
+      SpinClock clk(limit_ticks);
+      uint32_t level = 0;
+      bool ok = false;
+      for (;;) {
+        if (is_send) {
+          uint32_t expected = 0u;
+          ok = __hip_atomic_compare_exchange_strong(slot, &expected, 1u, __ATOMIC_RELAXED, __ATOMIC_RELAXED, kScope);
+        } else {
+          ok = __hip_atomic_load(slot, __ATOMIC_RELAXED, kScope) == 1u;
+        }
+        if (ok) break;
+        backoff_sleep(level);
+        if (clk.expired()) break;
+      }
+      if (!ok) {
+        if (role < 2) report(status, is_send ? SMR_ST_SEND_TIMEOUT : SMR_ST_WAIT_TIMEOUT, rank, block_id, peer);
+        else report(status, is_send ? SMR_ST_SEND_TIMEOUT : SMR_ST_WAIT_TIMEOUT, peer, block_id, rank);
+        bad = 1;
+      } else if (!is_send) {
+        __hip_atomic_fetch_and(slot, 0u, __ATOMIC_RELAXED, kScope);       // consume: 1 -> 0
+      }
+    }
+    if (acquire) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+  }
+  bad = __syncthreads_or(bad);
+  return bad == 0;
+}
+
+// DEFER: results a thread holds back before it stores them (1 = each as it comes: the
+// write-back forms, and the all-ranks emulation, whose ws * nblocks workgroups must all be
+// resident for their handshake and cannot afford the registers).  The kernel with 64 takes a
+// compute unit's registers for 256 threads.
+template <int KIND, int WS, bool WRITE_ALL, int DEFER>
+__global__ __launch_bounds__(DEFER > 16 ? 256 : kReduceMaxThreads) void one_shot_all_reduce_kernel(
     const uint64_t* __restrict__ buffer_ptrs, PeerPtrs by_value, const uint64_t* __restrict__ signal_pad_ptrs,
     SignalPads pads_by_value, Vec16* __restrict__ out, int64_t nvec, int rank, int layout, int nblocks, int do_barrier,
     uint64_t limit_ticks, uint32_t* status) {
   int block = blockIdx.x;
   const int nthreads = blockDim.x;
   int64_t lo = 0, hi = nvec;             // slots this rank reduces
-  if (layout == kProxy) {
-    const int per_proxy = nthreads >> 3;
-    const int nproxy = (nblocks + per_proxy - 1) / per_proxy;
-    if ((int)blockIdx.x < nproxy) {
-      // Peer proxies: 8 lanes per block, lane j stands in for rank j's block b.
-      const int b = blockIdx.x * per_proxy + (threadIdx.x >> 3);
-      const int j = threadIdx.x & 7;
-      if (b < nblocks && j < WS && j != rank) {
-        const bool by_val = pads_by_value.p[0] != 0;
-        uint32_t* to_rank = reinterpret_cast<uint32_t*>(by_val ? pads_by_value[rank] : signal_pad_ptrs[rank]) + (size_t)b * WS + j;
-        uint32_t* from_rank = reinterpret_cast<uint32_t*>(by_val ? pads_by_value[j] : signal_pad_ptrs[j]) + (size_t)b * WS + rank;
-        // one round per handshake of the rank's block (leading, and trailing if asked for)
-        for (int round = 0; round < do_barrier; ++round) {
-          // (a proxy publishes nothing: the peers' data are the work of earlier kernels)
-          if (!send_signal_relaxed(to_rank, limit_ticks)) {
-            report(status, SMR_ST_SEND_TIMEOUT, j, b, rank);
-            break;
-          }
-          if (!wait_signal_reset(from_rank, limit_ticks)) {
-            report(status, SMR_ST_WAIT_TIMEOUT, j, b, rank);
-            break;
-          }
-        }
-      }
-      return;
-    }
-    block = blockIdx.x - nproxy;
-  } else if (layout == kAllRanks) {
+  if (layout == kAllRanks) {
     block = blockIdx.x / WS;
     rank = blockIdx.x % WS;
     if constexpr (WRITE_ALL) {
@@ -194,16 +230,26 @@ __global__ __launch_bounds__(kReduceMaxThreads) void one_shot_all_reduce_kernel(
     }
   }
 
+  // Handshake number `round` of this block: between real workgroups (all ranks in one launch),
+  // or with stand-ins for the ranks that are not there.
+  auto handshake = [&](bool publish, bool acquire) {
+    const bool by_val = pads_by_value.p[0] != 0;
+    if (layout == kProxy) {
+      if (by_val) barrier_with_stand_ins<WS>(pads_by_value, block, rank, limit_ticks, status, publish, acquire);
+      else barrier_with_stand_ins<WS>(signal_pad_ptrs, block, rank, limit_ticks, status, publish, acquire);
+    } else {
+      if (by_val) blockwise_barrier(pads_by_value, block, rank, WS, limit_ticks, status, publish, acquire);
+      else blockwise_barrier(signal_pad_ptrs, block, rank, WS, limit_ticks, status, publish, acquire);
+    }
+  };
+
   // The peers' buffers were written by earlier kernels: nothing of this kernel to publish.
   // And nothing to invalidate: a launch starts from invalidated caches, and no workgroup reads
   // a peer's line before its own handshake (a line is never shared by two blocks: a block's
   // slots are nthreads * 16 bytes in a row), so no cache can hold a line of the peers' data
   // that is older than the handshake.  The invalidate an acquire stands for cost 1.3 us of a
   // 14 us launch.
-  if (do_barrier) {
-    if (pads_by_value.p[0] != 0) blockwise_barrier(pads_by_value, block, rank, WS, limit_ticks, status, false, false);
-    else blockwise_barrier(signal_pad_ptrs, block, rank, WS, limit_ticks, status, false, false);
-  }
+  if (do_barrier) handshake(false, false);
 
   GlobalVec* src[WS];
   if (buffer_ptrs != nullptr) {
@@ -216,24 +262,51 @@ __global__ __launch_bounds__(kReduceMaxThreads) void one_shot_all_reduce_kernel(
   GlobalVec* dst = (GlobalVec*)(uintptr_t)out;
 
   const int64_t stride = (int64_t)nblocks * nthreads;
-  for (int64_t i = lo + (int64_t)block * nthreads + threadIdx.x; i < hi; i += stride) {
-    Vec16 v[WS];
+  if constexpr (DEFER > 1) {
+    int64_t i = lo + (int64_t)block * nthreads + threadIdx.x;
+    while (i < hi) {
+      Vec16 held[DEFER];
+      const int64_t first = i;
 #pragma unroll
-    for (int r = 0; r < WS; ++r) v[r] = load_stream(src[r] + i);
-    Vec16 o = sum_in_rank_order<KIND, WS>(v);
-    if constexpr (WRITE_ALL) {
+      for (int d = 0; d < DEFER; ++d) {
+        if (i < hi) {
+          Vec16 v[WS];
 #pragma unroll
-      for (int r = 0; r < WS; ++r) store_stream(src[r] + i, o);
-    } else {
-      store_stream(dst + i, o);
+          for (int r = 0; r < WS; ++r) v[r] = load_stream(src[r] + i);
+          held[d] = sum_in_rank_order<KIND, WS>(v);
+          i += stride;
+        }
+      }
+#pragma unroll
+      for (int d = 0; d < DEFER; ++d) {
+        if (first + d * stride < hi) {
+          if constexpr (WRITE_ALL) {
+            // (in place: a slot is read and written by the one thread that owns it)
+#pragma unroll
+            for (int r = 0; r < WS; ++r) store_stream(src[r] + first + d * stride, held[d]);
+          } else {
+            store_stream(dst + first + d * stride, held[d]);
+          }
+        }
+      }
+    }
+  } else {
+    for (int64_t i = lo + (int64_t)block * nthreads + threadIdx.x; i < hi; i += stride) {
+      Vec16 v[WS];
+#pragma unroll
+      for (int r = 0; r < WS; ++r) v[r] = load_stream(src[r] + i);
+      Vec16 o = sum_in_rank_order<KIND, WS>(v);
+      if constexpr (WRITE_ALL) {
+#pragma unroll
+        for (int r = 0; r < WS; ++r) store_stream(src[r] + i, o);
+      } else {
+        store_stream(dst + i, o);
+      }
     }
   }
   // Trailing handshake: nobody's buffer is overwritten (or, with write-back, read)
   // before every rank is through; it publishes this workgroup's stores.
-  if (do_barrier == 2) {
-    if (pads_by_value.p[0] != 0) blockwise_barrier(pads_by_value, block, rank, WS, limit_ticks, status, true, true);
-    else blockwise_barrier(signal_pad_ptrs, block, rank, WS, limit_ticks, status, true, true);
-  }
+  if (do_barrier == 2) handshake(true, true);
 }
 
 template <int KIND, int WS>
@@ -242,12 +315,28 @@ static int launch_ws(bool write_all, dim3 grid, int threads, hipStream_t s, cons
                      Vec16* out, int64_t nvec, int rank, int layout, int nblocks, int do_barrier,
                      uint32_t* status) {
   const uint64_t lim = spin_limit_ticks();
-  if (write_all)
-    hipLaunchKernelGGL((one_shot_all_reduce_kernel<KIND, WS, true>), grid, dim3(threads), 0, s,
-                       bp, pv, sp, spv, out, nvec, rank, layout, nblocks, do_barrier, lim, status);
-  else
-    hipLaunchKernelGGL((one_shot_all_reduce_kernel<KIND, WS, false>), grid, dim3(threads), 0, s,
-                       bp, pv, sp, spv, out, nvec, rank, layout, nblocks, do_barrier, lim, status);
+#define SMR_REDUCE_LAUNCH(WA, D)                                                                          \
+  hipLaunchKernelGGL((one_shot_all_reduce_kernel<KIND, WS, WA, D>), grid, dim3(threads), 0, s, bp, pv, sp, spv, \
+                     out, nvec, rank, layout, nblocks, do_barrier, lim, status)
+  // slots per thread: beyond 16 of them, in workgroups of at most 256 threads, the kernel that
+  // holds back 64 results (it is compiled for 256 threads)
+  const int64_t per_thread = (nvec + (int64_t)nblocks * threads - 1) / ((int64_t)nblocks * threads);
+  // (write-back to all peers, as many bytes written as read: holding results back gains 5 to 7 %
+  // up to 16 MiB per buffer and nothing beyond)
+  if (write_all && layout != kAllRanks && per_thread > 2 && per_thread <= 16) SMR_REDUCE_LAUNCH(true, 8);
+  else if (write_all) SMR_REDUCE_LAUNCH(true, 1);
+  // (a thread with one or two slots has nothing to hold back, and the loop that could costs a
+  // launch of 5 us a quarter of a microsecond)
+  else if (layout == kAllRanks || per_thread <= 2) SMR_REDUCE_LAUNCH(false, 1);
+  else if constexpr (KIND != SMR_DTYPE_BF16_STEPWISE) {
+    if (threads <= 256 && per_thread > 16) SMR_REDUCE_LAUNCH(false, 64);
+    else SMR_REDUCE_LAUNCH(false, 8);
+  } else {
+    // (the stepwise sum is an order of magnitude more arithmetic per slot; 64 of them unrolled
+    // is more code than the compiler keeps in registers)
+    SMR_REDUCE_LAUNCH(false, 8);
+  }
+#undef SMR_REDUCE_LAUNCH
   return check_hip(hipGetLastError(), "smr_one_shot_all_reduce launch");
 }
 
@@ -326,8 +415,6 @@ static int reduce_entry(const uint64_t* buffer_ptrs_dev, const uint64_t* buffer_
     grid = (unsigned)nblocks * (unsigned)world_size;
   } else if (do_barrier) {
     layout = kProxy;
-    const int per_proxy = threads / 8;
-    grid = (unsigned)nblocks + (unsigned)((nblocks + per_proxy - 1) / per_proxy);
   }
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
   Vec16* o = reinterpret_cast<Vec16*>(out);
