@@ -121,6 +121,52 @@ def test_other_world_sizes(cuda, ws):
     assert _same(_bits(out), O.reduce_ref(bufs, "bf16"))
 
 
+@pytest.mark.parametrize("launch,full,held", [((64, 16), 10, 8), ((64, 4), 20, 64), ((256, 2), 70, 64), ((512, 2), 20, 8)],
+                         ids=["8-held", "64-held", "64-held-twice", "512-threads"])
+@pytest.mark.parametrize("mode", ["bf16", "fp32", "stepwise", "write_all", "barrier", "ws5"])
+def test_results_held_back(cuda, lib, launch, full, held, mode):
+    """The kernels that keep a thread's results in registers and store them in one go (8 results
+    each; 64 in the kernel for workgroups of up to 256 threads with more than 16 slots per thread)
+    normally run at 4 MiB per buffer and beyond.  A small grid gives a small message as many slots
+    per thread: bit-exact against the oracle with a ragged last trip, every dtype and mode, behind
+    the barrier (whose stand-ins share the handshake wave), and at a world size other than 8."""
+    from symm_mem_recipes import one_shot_all_reduce
+    threads, blocks = launch
+    ws = 5 if mode == "ws5" else WS
+    dtype = torch.float32 if mode == "fp32" else torch.bfloat16
+    per_vec = 4 if dtype == torch.float32 else 8
+    # `full` whole trips of the grid, then a ragged one: a workgroup and five threads more
+    numel = (threads * blocks * full + threads + 5) * per_vec
+    assert lib.smr_set_reduce_launch(threads, blocks) == 0
+    try:
+        slots = -(-(numel // per_vec) // (threads * blocks))
+        # (the library's rule: beyond 16 slots per thread in workgroups of up to 256 threads)
+        assert slots == full + 1 and (held == 64) == (threads <= 256 and slots > 16), (slots, held)
+        t, h = _alloc(numel, dtype, cuda, ws=ws, rank=ws - 2)
+        bufs = _fill(h, numel, dtype, seed0=70)
+        print(f"held-back stores: {mode} launch {launch} numel {numel}", flush=True)
+        if mode == "stepwise":
+            want = O.reduce_ref_bf16_acc(bufs)
+            out = one_shot_all_reduce(t, barrier=False, accumulate="bf16")
+        elif mode == "write_all":
+            want = O.reduce_ref(bufs, "bf16")
+            one_shot_all_reduce(t, barrier=False, write_all=True)
+            out = h.get_buffer(0, (numel,), dtype)
+        else:
+            want = O.reduce_ref(bufs, "bf16" if dtype == torch.bfloat16 else "fp32")
+            out = one_shot_all_reduce(t, barrier=(mode == "barrier"))
+        h.check_status()
+        assert _same(_bits(out), want)
+        if mode == "write_all":
+            for r in range(ws):
+                assert _same(_bits(h.get_buffer(r, (numel,), dtype)), want)
+        if mode == "barrier":
+            for r in range(ws):
+                assert int(h.get_signal_pad(r).abs().sum().item()) == 0
+    finally:
+        lib.smr_set_reduce_launch(0, 0)
+
+
 def test_special_values(cuda):
     """Signed zeros, denormals, infinities, NaN, cancellation, bf16 ties."""
     from symm_mem_recipes import one_shot_all_reduce
