@@ -58,8 +58,8 @@ extern "C" {
 
 /* barrier_mode of smr_one_shot_all_reduce */
 #define SMR_BARRIER_NONE   0  /* no handshake: peers' data are already stream-ordered */
-#define SMR_BARRIER_PROXY  1  /* the rank's blocks run the real handshake; one proxy
-                                 workgroup per block plays the other ranks' halves */
+#define SMR_BARRIER_PROXY  1  /* the rank's blocks run the real handshake; spare lanes of the
+                                 wave that does it play the absent ranks' halves */
 #define SMR_BARRIER_BOTH   2  /* as PROXY, and a second handshake after the last store: the
                                  reference has none behind triton_one_shot_all_reduce.py:93, so
                                  a peer may overwrite its buffer while others still read it */

@@ -30,7 +30,7 @@ def one_shot_all_reduce(tensor: torch.Tensor, *, barrier: bool = True, write_all
 
     ``barrier``    run the blockwise handshake before reading the peers
                    (triton_one_shot_all_reduce.py:70); the other ranks' halves
-                   are played by proxy workgroups of the same launch.
+                   are played by spare lanes of the wave that does the rank's own.
     ``write_all``  write the result back into all peer buffers in place and
                    return the calling rank's buffer (``tensor`` itself).
     ``all_ranks``  run every emulated rank in one launch, each behind the real
