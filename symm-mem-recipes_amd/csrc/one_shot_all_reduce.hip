@@ -277,17 +277,19 @@ __global__ __launch_bounds__(DEFER > 16 ? 256 : kReduceMaxThreads) void one_shot
           i += stride;
         }
       }
+      if constexpr (WRITE_ALL) {
+        // In place (a slot is read and written by the one thread that owns it), one peer's
+        // buffer after the other: eight write streams side by side are slower than one at a
+        // time (8 MiB per buffer: 26.7 -> 24.5 us).
 #pragma unroll
-      for (int d = 0; d < DEFER; ++d) {
-        if (first + d * stride < hi) {
-          if constexpr (WRITE_ALL) {
-            // (in place: a slot is read and written by the one thread that owns it)
+        for (int r = 0; r < WS; ++r)
 #pragma unroll
-            for (int r = 0; r < WS; ++r) store_stream(src[r] + first + d * stride, held[d]);
-          } else {
-            store_stream(dst + first + d * stride, held[d]);
-          }
-        }
+          for (int d = 0; d < DEFER; ++d)
+            if (first + d * stride < hi) store_stream(src[r] + first + d * stride, held[d]);
+      } else {
+#pragma unroll
+        for (int d = 0; d < DEFER; ++d)
+          if (first + d * stride < hi) store_stream(dst + first + d * stride, held[d]);
       }
     }
   } else {
@@ -318,23 +320,25 @@ static int launch_ws(bool write_all, dim3 grid, int threads, hipStream_t s, cons
 #define SMR_REDUCE_LAUNCH(WA, D)                                                                          \
   hipLaunchKernelGGL((one_shot_all_reduce_kernel<KIND, WS, WA, D>), grid, dim3(threads), 0, s, bp, pv, sp, spv, \
                      out, nvec, rank, layout, nblocks, do_barrier, lim, status)
-  // slots per thread: beyond 16 of them, in workgroups of at most 256 threads, the kernel that
-  // holds back 64 results (it is compiled for 256 threads)
+  // Results a thread holds back.  None for one or two slots per thread (nothing to hold back,
+  // and the loop that could costs a launch of 5 us a quarter of a microsecond) and for the
+  // all-ranks emulation; 64 beyond 16 slots per thread in workgroups of at most 256 threads
+  // (the kernel is compiled for 256), but not for the stepwise sum (an order of magnitude more
+  // arithmetic per slot: 64 unrolled copies are more code than the compiler keeps in
+  // registers); otherwise 8.  Write-back to all peers, as many bytes written as read, has less
+  // to gain: 9 % at 8 MiB per buffer, 4 % at 16 and 64 MiB.
   const int64_t per_thread = (nvec + (int64_t)nblocks * threads - 1) / ((int64_t)nblocks * threads);
-  // (write-back to all peers, as many bytes written as read: holding results back gains 5 to 7 %
-  // up to 16 MiB per buffer and nothing beyond)
-  if (write_all && layout != kAllRanks && per_thread > 2 && per_thread <= 16) SMR_REDUCE_LAUNCH(true, 8);
-  else if (write_all) SMR_REDUCE_LAUNCH(true, 1);
-  // (a thread with one or two slots has nothing to hold back, and the loop that could costs a
-  // launch of 5 us a quarter of a microsecond)
-  else if (layout == kAllRanks || per_thread <= 2) SMR_REDUCE_LAUNCH(false, 1);
-  else if constexpr (KIND != SMR_DTYPE_BF16_STEPWISE) {
-    if (threads <= 256 && per_thread > 16) SMR_REDUCE_LAUNCH(false, 64);
+  const bool deep = KIND != SMR_DTYPE_BF16_STEPWISE && threads <= 256 && per_thread > 16;
+  const int held = (layout == kAllRanks || per_thread <= 2) ? 1 : (deep ? 64 : 8);
+  if (held == 1) {
+    if (write_all) SMR_REDUCE_LAUNCH(true, 1);
+    else SMR_REDUCE_LAUNCH(false, 1);
+  } else if (held == 8) {
+    if (write_all) SMR_REDUCE_LAUNCH(true, 8);
     else SMR_REDUCE_LAUNCH(false, 8);
-  } else {
-    // (the stepwise sum is an order of magnitude more arithmetic per slot; 64 of them unrolled
-    // is more code than the compiler keeps in registers)
-    SMR_REDUCE_LAUNCH(false, 8);
+  } else if constexpr (KIND != SMR_DTYPE_BF16_STEPWISE) {
+    if (write_all) SMR_REDUCE_LAUNCH(true, 64);
+    else SMR_REDUCE_LAUNCH(false, 64);
   }
 #undef SMR_REDUCE_LAUNCH
   return check_hip(hipGetLastError(), "smr_one_shot_all_reduce launch");
