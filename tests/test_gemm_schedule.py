@@ -135,19 +135,22 @@ def test_fused_plan_splits_the_gpu(lib):
         assert grid == lib.smr_ag_matmul_grid(M, N, K, 8, M // 8, 1)
         assert 1 <= wgs <= 128 and grid + wgs <= 256
         assert fused_us > 0 and sequential_us > 0
-        assert sequential == (1 if sequential_us < fused_us else 0)
+        assert sequential == (1 if sequential_us < 0.98 * fused_us else 0)
         plans[(M, N, K)] = (grid, wgs, sequential)
     # (the choices below are the ones launches timed on MI355X bear out)
     assert plans[(16384, 3584, 8192)] == (224, 32, 0)
     assert plans[(16384, 6656, 16384)][2] == 0
     assert plans[(4096, 8192, 8192)][2] == 1 and plans[(2048, 4096, 2048)][2] == 1
     assert plans[(8192, 1792, 4096)][2] == 1 and plans[(4096, 3584, 8192)][2] == 1
-    # ((8192, 3584, 8192) and (16384, 1792, 4096) time within 2 % and 5 % either way: not asserted)
+    assert plans[(8192, 3584, 8192)][2] == 0 and plans[(16384, 1792, 4096)][2] == 1
     # a problem with few passes leaves the copy more of the GPU
     assert plans[(2048, 4096, 2048)][1] > plans[(16384, 3584, 8192)][1]
     out = (ctypes.c_int32 * 5)()
     assert lib.smr_ag_matmul_plan_fp8(16384, 3584, 8192, 8, 2048, out) == 0
     assert list(out)[:2] == [224, 32] and out[4] == 0
+    # (e4m3fn: the narrow problem is the faster one copied first, 124 against 139 us)
+    assert lib.smr_ag_matmul_plan_fp8(16384, 1792, 4096, 8, 2048, out) == 0 and out[4] == 1
+    assert lib.smr_ag_matmul_plan_fp8(8192, 3584, 8192, 8, 1024, out) == 0 and out[4] == 0
     assert lib.smr_ag_matmul_plan_fp8(16384, 3584, 8192 + 64, 8, 2048, out) == -2      # K % 128
     assert lib.smr_ag_matmul_plan(1000, 256, 256, 8, 125, out) == -2                   # unsupported shape
     assert lib.smr_ag_matmul_plan(1024, 256, 256, 8, 128, None) == -1
