@@ -206,10 +206,10 @@ __device__ __forceinline__ bool barrier_with_stand_ins(const Pads& pads, uint32_
   return bad == 0;
 }
 
-// DEFER: results a thread holds back before it stores them (1 = each as it comes: the
-// write-back forms, and the all-ranks emulation, whose ws * nblocks workgroups must all be
-// resident for their handshake and cannot afford the registers).  The kernel with 64 takes a
-// compute unit's registers for 256 threads.
+// DEFER: results a thread holds back before it stores them (1 = each as it comes: messages of
+// one or two slots per thread, and the all-ranks emulation, where holding back gained nothing -
+// its time is the handshakes' fences).  The kernel with 64 takes a compute unit's registers
+// for 256 threads.
 template <int KIND, int WS, bool WRITE_ALL, int DEFER>
 __global__ __launch_bounds__(DEFER > 16 ? 256 : kReduceMaxThreads) void one_shot_all_reduce_kernel(
     const uint64_t* __restrict__ buffer_ptrs, PeerPtrs by_value, const uint64_t* __restrict__ signal_pad_ptrs,
@@ -230,8 +230,8 @@ __global__ __launch_bounds__(DEFER > 16 ? 256 : kReduceMaxThreads) void one_shot
     }
   }
 
-  // Handshake number `round` of this block: between real workgroups (all ranks in one launch),
-  // or with stand-ins for the ranks that are not there.
+  // A handshake of this block: between real workgroups (all ranks in one launch), or with
+  // stand-ins for the ranks that are not there.
   auto handshake = [&](bool publish, bool acquire) {
     const bool by_val = pads_by_value.p[0] != 0;
     if (layout == kProxy) {
