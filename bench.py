@@ -596,19 +596,26 @@ def main():
     }
     extra["calibration_copy"] = calibration_copy(dev)
     if not args.no_extra:
-        # per-buffer sizes of the size sweep; 2 and 8 MiB are the points the targets name.  The
-        # three that stream from HBM go largest first: their buffer sets (1 GiB per size) are then
-        # carved from the segments the largest one left with torch's caching allocator, as a
-        # process that starts with them would have them, instead of from whatever the driver
-        # finds next to a gigabyte of smaller blocks (8 MiB: 13.2 to 13.3 us against 13.7 to 13.8)
-        sweep = (16, 64, 256, 1024, 2048, 4096, 32768, 16384, 8192)
-        extra["reduce_rotating"] = (
-            [bench_reduce_rotating(k, dev, "bf16") for k in sweep] +
-            [bench_reduce_rotating(k, dev, "fp32") for k in (1024, 16384, 8192)] +
-            [bench_reduce_rotating(k, dev, "bf16", write_all=True) for k in (1024, 16384, 8192)] +
-            [bench_reduce_rotating(k, dev, "bf16", accumulate="bf16") for k in (8192,)] +
-            [bench_reduce_rotating(k, dev, "bf16", barrier=True) for k in (16, 1024, 32768, 16384, 8192)] +
-            [bench_reduce_rotating(k, dev, "fp32", barrier=True) for k in (16384, 8192)])
+        # The size sweep on rotating buffer sets; 2 and 8 MiB are the points the targets name.
+        # The cases that stream from HBM (8 MiB per buffer and up) run first, each group largest
+        # first: their buffer sets (1 GiB per case) are then carved from the segments the first
+        # cases left with torch's caching allocator, as a process that allocates its symmetric
+        # buffers at start-up would have them, instead of from whatever the driver finds next to
+        # gigabytes of smaller cached blocks (8 MiB: 13.2 to 13.3 us against 13.7 to 13.8).  The
+        # small cases, whose figure is the host's call rate, follow on an emptied cache.
+        import torch
+        big = ([bench_reduce_rotating(k, dev, "bf16") for k in (32768, 16384, 8192)] +
+               [bench_reduce_rotating(k, dev, "fp32") for k in (16384, 8192)] +
+               [bench_reduce_rotating(k, dev, "bf16", write_all=True) for k in (16384, 8192)] +
+               [bench_reduce_rotating(k, dev, "bf16", accumulate="bf16") for k in (8192,)] +
+               [bench_reduce_rotating(k, dev, "bf16", barrier=True) for k in (32768, 16384, 8192)] +
+               [bench_reduce_rotating(k, dev, "fp32", barrier=True) for k in (16384, 8192)])
+        torch.cuda.empty_cache()
+        small = ([bench_reduce_rotating(k, dev, "bf16") for k in (16, 64, 256, 1024, 2048, 4096)] +
+                 [bench_reduce_rotating(k, dev, "fp32") for k in (1024,)] +
+                 [bench_reduce_rotating(k, dev, "bf16", write_all=True) for k in (1024,)] +
+                 [bench_reduce_rotating(k, dev, "bf16", barrier=True) for k in (16, 1024)])
+        extra["reduce_rotating"] = sorted(small + big, key=lambda r: (r["mode"], r["accumulate"], r["dtype"], r["size_kib"]))
         extra["all_gather_matmul"] = bench_ag_matmul(dev)
         extra["all_gather_matmul"]["mfma_only"] = bench_mfma_only(dev)
         extra["all_gather_matmul_fp8"] = bench_ag_matmul_fp8(dev)
